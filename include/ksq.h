@@ -1,0 +1,143 @@
+/*
+ * ksq.h -- C ABI of the MI355X (gfx950) quantized linear-layer path.
+ *
+ * One shared library, libksq.so, exports everything below with C linkage.  All pointers are device pointers
+ * unless the parameter name ends in `_host`; `stream` is a hipStream_t passed as void* (NULL = the default
+ * stream).  Every function returns KSQ_OK (0) or a negative ksq_status; no exception crosses this boundary and
+ * ksq_last_error_string() gives the reason for the last failure on the calling thread.  Nothing here allocates
+ * device memory, synchronises the stream, or branches on device data, so the GEMM entry points are safe to call
+ * from a serving loop and under HIP graph capture.
+ *
+ * Citations name the interface of KsanaLLM that each entry point replaces
+ * (KS = src/ksana_llm, LK = 3rdparty/LLM_kernels/csrc/kernels/nvidia, LU = 3rdparty/LLM_kernels/csrc/utils/nvidia).
+ */
+#ifndef KSQ_H_
+#define KSQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum ksq_status {
+  KSQ_OK = 0,
+  KSQ_ERR_INVALID_ARGUMENT = -1, /* null pointer, zero size, bad enum */
+  KSQ_ERR_UNSUPPORTED = -2,      /* shape / group size / layout the kernels do not cover */
+  KSQ_ERR_WORKSPACE = -3,        /* workspace missing or too small where it is mandatory */
+  KSQ_ERR_HIP = -4               /* a HIP runtime call or kernel launch failed */
+} ksq_status;
+
+/* Activation / output element type (the reference instantiates its layers for half and __nv_bfloat16:
+ * KS/layers/nvidia/group_matmul_layer.cpp:171-175, fp8_matmul_layer.cpp:69-73). */
+typedef enum ksq_dtype { KSQ_F16 = 0, KSQ_BF16 = 1 } ksq_dtype;
+
+/* Source layouts the repack step reads. */
+typedef enum ksq_w4_layout {
+  /* GPTQ checkpoint: qweight int32 [K/8, N], element k = 8r + j in bits 4j..4j+3 of row r; symmetric, the
+   * zero point is 8 and qzeros are ignored (KS/models/quant/quant_weight.cpp:291-300, :73-75). */
+  KSQ_W4_GPTQ_INT32_KPACK = 0,
+  /* AWQ checkpoint: qweight int32 [K, N/8], slot j of a word holds column 8c + [0,2,4,6,1,3,5,7][j];
+   * qzeros int32 [K/g, N/8] packed the same way (KS/models/quant/quant_weight.cpp:262-287). */
+  KSQ_W4_AWQ_INT32_NPACK = 1,
+  /* ksana's canonical form after CutlassAutoUnpack: int8 [K, N/2], low nibble = even column, signed q = u - 8
+   * (KS/models/quant/quant_weight.cpp:249-251, :304-328) -- the input of the CUTLASS preprocessor that this
+   * repack replaces (LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508). */
+  KSQ_W4_ROWMAJOR_INT4_SIGNED = 2
+} ksq_w4_layout;
+
+/* How zero points are handed to the repack step. */
+typedef enum ksq_zero_kind {
+  KSQ_ZERO_NONE = 0,          /* symmetric: z = 8 for every group (GPTQ) */
+  KSQ_ZERO_AWQ_INT32 = 1,     /* AWQ qzeros int32 [K/g, N/8], as in the checkpoint */
+  KSQ_ZERO_UINT8 = 2,         /* unpacked z in [0,15], uint8 [K/g, N] */
+  KSQ_ZERO_ADDITIVE = 3       /* ksana's layer-boundary form: T [K/g, N] holding scales * (8 - z)
+                                 (KS/models/quant/quant_weight.cpp:530-536); z is recovered exactly */
+} ksq_zero_kind;
+
+typedef enum ksq_fp8_quant_mode {
+  KSQ_FP8_PER_TENSOR_DYNAMIC = 0, /* one scale from the abs-max of the whole [m,k] tensor (is_static = false) */
+  KSQ_FP8_PER_TENSOR_STATIC = 1,  /* caller-supplied scalar scale (checkpoint input_scale, is_static = true) */
+  KSQ_FP8_PER_TOKEN_DYNAMIC = 2   /* one scale per row (num_channels = m) */
+} ksq_fp8_quant_mode;
+
+/* Library / error plumbing. */
+int ksq_version(void);
+const char* ksq_last_error_string(void);
+/* Number of the compute units of the current device that the launch heuristics use (0 on failure). */
+int ksq_device_compute_units(void);
+
+/* ------------------------------------------------------------------ W4A16: load-time repack
+ *
+ * Replaces CutlassPreprocessWeightsForMixedGemmWarpper / preprocess_weights_for_mixed_gemm
+ * (KS/models/quant/quant_weight.cpp:331-346, 577-579; LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508)
+ * and the scale / zero binding of ConvertGroupTensor (quant_weight.cpp:530-536, 632-636).
+ *
+ * Output "fragment order" (K % 128 == 0, N % 16 == 0, g in {64,128}):
+ *   weight : K*N/2 bytes = tiles [N/16][K/128] of 1024 B.  Tile (nt,kt) is 64 lanes x 16 B; lane l = 16*j + c
+ *            owns column n = 16*nt + c; 32-bit word d (0..3) of the lane covers k = 128*kt + 32*d + 8*j + e,
+ *            e = 0..7, with element e in nibble e/2 when e is even and nibble 4 + e/2 when e is odd; nibbles are
+ *            the unsigned u in [0,15].  One 128-bit load per lane is the B operand of four 16x16x32 MFMAs.
+ *   sz     : (K/g)*N 32-bit words = [N/16][K/g][16]; word = scale bits (T) | z << 16 with z in [0,15]. */
+int ksq_w4a16_repack_sizes(size_t k, size_t n, size_t group_size, size_t* weight_bytes, size_t* sz_bytes);
+
+int ksq_w4a16_repack(int src_layout, const void* qweight, int zero_kind, const void* zeros, const void* scales,
+                     int scale_dtype, size_t k, size_t n, size_t group_size, void* dst_weight, void* dst_sz,
+                     void* stream);
+
+/* Same transform on host memory (no GPU needed); used when weights are prepared before upload. */
+int ksq_w4a16_repack_host(int src_layout, const void* qweight_host, int zero_kind, const void* zeros_host,
+                          const void* scales_host, int scale_dtype, size_t k, size_t n, size_t group_size,
+                          void* dst_weight_host, void* dst_sz_host);
+
+/* ------------------------------------------------------------------ W4A16: GEMM
+ *
+ * Replaces InvokeFpAIntBGroupCudaGemm / InvokeFpAIntBGroupCutlassGemm and
+ * GetFpAIntBGroupCutlassGemmWorkspaceSize (KS/kernels/nvidia/kernel_wrapper.cpp:209-302), i.e.
+ * FpAIntBGroupCudaGemmWrapper::Gemm (LK/weight_only_batched_gemv/weight_only_gemv_wrapper.cu:27-46) and
+ * FpAIntBGroupCutlassGemmWrapper::Gemm (LK/asymmetric_gemm/asymmetric_gemm_wrapper.cu:53-77):
+ *   out[m,n] = T( sum_k act[m,k] * s[k/g,n] * (u[k,n] - z[k/g,n]) ),  fp32 accumulation.
+ * act is [m,k] row-major T, out is [m,n] row-major T, weight / sz come from ksq_w4a16_repack.
+ * The workspace holds split-K partial sums; with workspace == NULL or too small the call still succeeds
+ * without split-K.  Calls that may overlap in time on one device must use different streams' worth of
+ * workspace: the workspace is scratch for the duration of one call only and holds no state between calls. */
+int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
+
+int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                   size_t k, size_t group_size, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ FP8 e4m3 (OCP: bias 7, max 448, no inf)
+ *
+ * ksq_fp8_quantize replaces Fp8E4m3Quantize (KS/kernels/nvidia/kernel_wrapper.cpp:1015-1027) =
+ * InvokeComputeFP8QuantizeScale + InvokeQuantizeMatrix (LU/cuda_fp8_utils.cu:27-44, 85-127):
+ *   scale[c] = max(absmax(x[c,:]) / 448, 1/(448*512));  q = e4m3(clamp(x / scale[c], +-448)).
+ * act is [m,k] T; act_q is [m,k] bytes; act_scale holds 1 float (per-tensor) or m floats (per-token). */
+int ksq_fp8_quantize(int dtype, const void* act, size_t m, size_t k, int mode, void* act_q, float* act_scale,
+                     void* stream);
+
+/* Replaces RescaleFp8E4m3 (KS/kernels/nvidia/kernel_wrapper.cpp:1043-1046, LU/cuda_fp8_utils.cu:140-155):
+ * out[i] = e4m3(float(in[i]) * (*scale_in / *scale_out)); in-place allowed. */
+int ksq_fp8_rescale(const void* in, void* out, size_t count, const float* scale_in, const float* scale_out,
+                    void* stream);
+
+/* On-the-fly weight conversion, replaces the device work of ConvertFp8E4m3Tensor
+ * (KS/models/quant/quant_weight.cpp:685-726): w is [k,n] T; w_q becomes [n,k] e4m3 (k contiguous) with a single
+ * scale written to w_scale[0]. */
+int ksq_fp8_convert_weight(int dtype, const void* w, size_t k, size_t n, void* w_q, float* w_scale, void* stream);
+
+/* Replaces Fp8QuantizedMatMul (KS/kernels/nvidia/kernel_wrapper.cpp:1033-1041, cuBLASLt FP8 matmul through
+ * LK/gemm_wrapper/gemm_wrapper.cc:39-107), extended to the per-token x per-channel scales of
+ * LK/asymmetric_gemm/fp8_rowwise_gemm/fp8_rowwise_gemm_kernel_template_sm90.h:119-131:
+ *   out[m,n] = T( (sum_k a[m,k] * w[n,k]) * w_scale[n or 0] * act_scale[m or 0] ),  fp32 accumulation.
+ * act_q is [m,k] e4m3, w_q is [n,k] e4m3 (k contiguous), scale counts are 1 or m / 1 or n. */
+int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
+
+int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                 const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KSQ_H_ */

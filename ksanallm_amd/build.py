@@ -1,0 +1,68 @@
+"""Builds libksq.so (the HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libksq.so")
+
+SOURCES = ["ksq_api.hip", "ksq_repack.hip", "ksq_w4a16_stream.hip", "ksq_w4a16_prefill.hip", "ksq_fp8.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-function",
+    "-I" + os.path.join(ROOT, "include"),
+    "-I" + CSRC,
+]
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; libksq.so cannot be built")
+    return exe
+
+
+def build_library(verbose=False, jobs=5):
+    """Compile every HIP source to an object (in parallel) and link libksq.so next to this file."""
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    cc = hipcc()
+    procs = []
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = [cc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        if len(procs) >= jobs:
+            _drain(procs)
+    _drain(procs)
+    link = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    subprocess.check_call(link)
+    return LIB
+
+
+def _drain(procs):
+    while procs:
+        src, p = procs.pop(0)
+        out, _ = p.communicate()
+        lines = [ln for ln in out.splitlines() if "packed-fp32-ops" not in ln]
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n" + "\n".join(lines))
+        if lines:
+            print("\n".join(lines), file=sys.stderr)
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

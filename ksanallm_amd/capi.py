@@ -1,0 +1,142 @@
+"""ctypes binding of libksq.so (the C ABI declared in include/ksq.h).
+
+Every wrapper takes raw device (or host) addresses as Python ints, or objects with ``data_ptr()`` (torch tensors)
+/ ``ctypes.data`` (numpy arrays), and raises :class:`KsqError` on a non-zero status.  Nothing here computes: a
+missing or unloadable library is an ImportError-like failure, never a fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libksq.so")
+
+# enums of include/ksq.h
+F16, BF16 = 0, 1
+W4_GPTQ_INT32_KPACK, W4_AWQ_INT32_NPACK, W4_ROWMAJOR_INT4_SIGNED = 0, 1, 2
+ZERO_NONE, ZERO_AWQ_INT32, ZERO_UINT8, ZERO_ADDITIVE = 0, 1, 2, 3
+FP8_PER_TENSOR_DYNAMIC, FP8_PER_TENSOR_STATIC, FP8_PER_TOKEN_DYNAMIC = 0, 1, 2
+OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, -1, -2, -3, -4
+
+EXPORTS = [
+    "ksq_version", "ksq_last_error_string", "ksq_device_compute_units",
+    "ksq_w4a16_repack_sizes", "ksq_w4a16_repack", "ksq_w4a16_repack_host",
+    "ksq_w4a16_workspace_bytes", "ksq_w4a16_gemm",
+    "ksq_fp8_quantize", "ksq_fp8_rescale", "ksq_fp8_convert_weight",
+    "ksq_fp8_workspace_bytes", "ksq_fp8_gemm",
+]
+
+
+class KsqError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"ksq error {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Load libksq.so; raises if it has not been built (there is no fallback path)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise KsqError(ERR_HIP, f"{LIB_PATH} is missing: build it with `python -m ksanallm_amd.build`")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+        psz = ctypes.POINTER(ctypes.c_size_t)
+        L.ksq_version.restype = ci
+        L.ksq_last_error_string.restype = ctypes.c_char_p
+        L.ksq_device_compute_units.restype = ci
+        L.ksq_w4a16_repack_sizes.argtypes = [sz, sz, sz, psz, psz]
+        L.ksq_w4a16_repack.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, vp, vp]
+        L.ksq_w4a16_repack_host.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, vp]
+        L.ksq_w4a16_workspace_bytes.argtypes = [sz, sz, sz, psz]
+        L.ksq_w4a16_gemm.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, sz, vp]
+        L.ksq_fp8_quantize.argtypes = [ci, vp, sz, sz, ci, vp, vp, vp]
+        L.ksq_fp8_rescale.argtypes = [vp, vp, sz, vp, vp, vp]
+        L.ksq_fp8_convert_weight.argtypes = [ci, vp, sz, sz, vp, vp, vp]
+        L.ksq_fp8_workspace_bytes.argtypes = [sz, sz, sz, psz]
+        L.ksq_fp8_gemm.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, vp, sz, vp]
+        for name in EXPORTS:
+            if name not in ("ksq_last_error_string",):
+                getattr(L, name).restype = ci
+        _lib = L
+    return _lib
+
+
+def _addr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    if hasattr(x, "ctypes"):
+        return x.ctypes.data
+    raise TypeError(f"cannot take the address of {type(x)}")
+
+
+def _check(code):
+    if code != OK:
+        raise KsqError(code, lib().ksq_last_error_string().decode())
+
+
+def version():
+    return lib().ksq_version()
+
+
+def device_compute_units():
+    return lib().ksq_device_compute_units()
+
+
+def w4a16_repack_sizes(k, n, group_size):
+    wb, sb = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    _check(lib().ksq_w4a16_repack_sizes(k, n, group_size, ctypes.byref(wb), ctypes.byref(sb)))
+    return wb.value, sb.value
+
+
+def w4a16_repack(src_layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, group_size, dst_weight, dst_sz,
+                 stream=None):
+    _check(lib().ksq_w4a16_repack(src_layout, _addr(qweight), zero_kind, _addr(zeros), _addr(scales), scale_dtype, k,
+                                  n, group_size, _addr(dst_weight), _addr(dst_sz), stream))
+
+
+def w4a16_repack_host(src_layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, group_size, dst_weight,
+                      dst_sz):
+    _check(lib().ksq_w4a16_repack_host(src_layout, _addr(qweight), zero_kind, _addr(zeros), _addr(scales),
+                                       scale_dtype, k, n, group_size, _addr(dst_weight), _addr(dst_sz)))
+
+
+def w4a16_workspace_bytes(max_m, n, k):
+    b = ctypes.c_size_t(0)
+    _check(lib().ksq_w4a16_workspace_bytes(max_m, n, k, ctypes.byref(b)))
+    return b.value
+
+
+def w4a16_gemm(dtype, out, act, weight, sz, m, n, k, group_size, workspace=None, workspace_bytes=0, stream=None):
+    _check(lib().ksq_w4a16_gemm(dtype, _addr(out), _addr(act), _addr(weight), _addr(sz), m, n, k, group_size,
+                                _addr(workspace), workspace_bytes, stream))
+
+
+def fp8_quantize(dtype, act, m, k, mode, act_q, act_scale, stream=None):
+    _check(lib().ksq_fp8_quantize(dtype, _addr(act), m, k, mode, _addr(act_q), _addr(act_scale), stream))
+
+
+def fp8_rescale(src, dst, count, scale_in, scale_out, stream=None):
+    _check(lib().ksq_fp8_rescale(_addr(src), _addr(dst), count, _addr(scale_in), _addr(scale_out), stream))
+
+
+def fp8_convert_weight(dtype, w, k, n, w_q, w_scale, stream=None):
+    _check(lib().ksq_fp8_convert_weight(dtype, _addr(w), k, n, _addr(w_q), _addr(w_scale), stream))
+
+
+def fp8_workspace_bytes(max_m, n, k):
+    b = ctypes.c_size_t(0)
+    _check(lib().ksq_fp8_workspace_bytes(max_m, n, k, ctypes.byref(b)))
+    return b.value
+
+
+def fp8_gemm(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k, workspace=None,
+             workspace_bytes=0, stream=None):
+    _check(lib().ksq_fp8_gemm(out_dtype, _addr(out), _addr(act_q), _addr(act_scale), act_scale_count, _addr(w_q),
+                              _addr(w_scale), w_scale_count, m, n, k, _addr(workspace), workspace_bytes, stream))

@@ -1,0 +1,227 @@
+// C-ABI entry points of libksq.so: argument validation, launch planning, error plumbing.
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+
+#include "ksq_internal.h"
+
+namespace ksq {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// ---- per-device state -----------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned g_splitk_counters[kCounterSlots * kCountersPerSlot];
+
+namespace {
+constexpr int kMaxDevices = 16;
+struct PerDevice {
+  std::once_flag once;
+  bool ok = false;
+  DeviceInfo info{};
+  unsigned* counters = nullptr;
+  std::atomic<unsigned> next_slot{0};
+};
+PerDevice g_dev[kMaxDevices];
+
+PerDevice* current_device_state() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(KSQ_ERR_HIP, "hipGetDevice failed or device index out of range");
+    return nullptr;
+  }
+  PerDevice* pd = &g_dev[dev];
+  std::call_once(pd->once, [pd, dev]() {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return;
+    pd->info.cus = prop.multiProcessorCount;
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_splitk_counters)) != hipSuccess || p == nullptr) return;
+    pd->counters = static_cast<unsigned*>(p);
+    pd->ok = true;
+  });
+  if (!pd->ok) {
+    fail(KSQ_ERR_HIP, "device %d: could not query properties or resolve the split-K counters", dev);
+    return nullptr;
+  }
+  return pd;
+}
+}  // namespace
+
+const DeviceInfo* device_info() {
+  PerDevice* pd = current_device_state();
+  return pd ? &pd->info : nullptr;
+}
+
+unsigned* counter_slot_device_ptr() {
+  PerDevice* pd = current_device_state();
+  if (!pd) return nullptr;
+  unsigned slot = pd->next_slot.fetch_add(1, std::memory_order_relaxed) % kCounterSlots;
+  return pd->counters + (size_t)slot * kCountersPerSlot;
+}
+
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  if (!v || !*v) return dflt;
+  return atoi(v);
+}
+
+// ---- launch planning ------------------------------------------------------------------------------------------
+// The streaming kernel gives every wave NT column tiles x a contiguous range of k tiles.  Split-K buys
+// parallelism for narrow N at the price of fp32 partial tiles written and read once each, so it is bounded both
+// by the workspace and by a traffic budget relative to the weight bytes.
+W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  W4Plan p{};
+  const size_t ntiles = n / kTileN, ktiles = k / kTileK;
+  p.prefill = false;
+  if (m <= 64) {
+    p.MT = (int)((m + 15) / 16);
+    p.mblocks = 1;
+    p.NT = 1;
+  } else {
+    p.MT = 4;
+    p.mblocks = (int)((m + 63) / 64);
+    p.NT = 2;
+  }
+  int nt_env = env_int("KSQ_W4_NT", 0);
+  if (nt_env == 1 || nt_env == 2) p.NT = nt_env;
+  const size_t ngroups = (ntiles + p.NT - 1) / p.NT;
+  const size_t wgs = ((ngroups + 3) / 4) * (size_t)p.mblocks;
+  size_t ksplit = 1;
+  if (m <= 64) {
+    const size_t target = (size_t)cus * 4;
+    ksplit = (target + wgs / 2) / wgs;
+    const size_t mpad = (size_t)p.MT * 16;
+    size_t traffic_cap = k / (64 * mpad);  // partial write+read <= 25% of the weight bytes
+    if (ksplit > traffic_cap) ksplit = traffic_cap;
+    if (ksplit > ktiles / 2) ksplit = ktiles / 2;
+    if (ksplit > 16) ksplit = 16;
+    if (ksplit < 1) ksplit = 1;
+    int ks_env = env_int("KSQ_W4_KSPLIT", 0);
+    if (ks_env >= 1 && (size_t)ks_env <= ktiles) ksplit = (size_t)ks_env;
+    if (ngroups * (size_t)p.mblocks > (size_t)kCountersPerSlot) ksplit = 1;
+  }
+  auto need = [&](size_t ks) { return ks <= 1 ? (size_t)0 : ks * (size_t)p.mblocks * ntiles * p.MT * 64 * 16; };
+  while (ksplit > 1 && need(ksplit) > workspace_bytes) --ksplit;
+  p.ksplit = (int)ksplit;
+  p.partial_bytes = need(ksplit);
+  return p;
+}
+
+Fp8Plan fp8_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  Fp8Plan p{};
+  const size_t ntiles = (n + 15) / 16, kblocks = k / 64;
+  p.prefill = false;
+  if (m <= 64) {
+    p.MT = (int)((m + 15) / 16);
+    p.mblocks = 1;
+  } else {
+    p.MT = 4;
+    p.mblocks = (int)((m + 63) / 64);
+  }
+  const size_t wgs = ((ntiles + 3) / 4) * (size_t)p.mblocks;
+  size_t ksplit = 1;
+  if (m <= 64) {
+    const size_t target = (size_t)cus * 4;
+    ksplit = (target + wgs / 2) / wgs;
+    const size_t mpad = (size_t)p.MT * 16;
+    size_t traffic_cap = k / (32 * mpad);  // partial write+read <= 25% of the weight bytes
+    if (ksplit > traffic_cap) ksplit = traffic_cap;
+    if (ksplit > kblocks / 4) ksplit = kblocks / 4;
+    if (ksplit > 16) ksplit = 16;
+    if (ksplit < 1) ksplit = 1;
+    int ks_env = env_int("KSQ_FP8_KSPLIT", 0);
+    if (ks_env >= 1 && (size_t)ks_env <= kblocks) ksplit = (size_t)ks_env;
+    if (ntiles * (size_t)p.mblocks > (size_t)kCountersPerSlot) ksplit = 1;
+  }
+  auto need = [&](size_t ks) { return ks <= 1 ? (size_t)0 : ks * (size_t)p.mblocks * ntiles * p.MT * 64 * 16; };
+  while (ksplit > 1 && need(ksplit) > workspace_bytes) --ksplit;
+  p.ksplit = (int)ksplit;
+  p.partial_bytes = need(ksplit);
+  return p;
+}
+
+}  // namespace ksq
+
+using namespace ksq;
+
+extern "C" {
+
+int ksq_version(void) { return 100; }
+
+const char* ksq_last_error_string(void) { return g_error; }
+
+int ksq_device_compute_units(void) {
+  const DeviceInfo* di = device_info();
+  return di ? di->cus : 0;
+}
+
+static int check_w4_shape(size_t k, size_t n, size_t g) {
+  KSQ_REQUIRE(k > 0 && n > 0, KSQ_ERR_INVALID_ARGUMENT, "k and n must be positive (k=%zu n=%zu)", k, n);
+  // the reference kernels accept group sizes 64 and 128 only (LK/asymmetric_gemm/fpA_intB_gemm/
+  // fpA_intB_gemm_template.h:130) and k % 64 == 0 (:168-171); the fragment order needs whole 128 x 16 tiles
+  KSQ_REQUIRE(g == 64 || g == 128, KSQ_ERR_UNSUPPORTED, "group size %zu not supported (64 or 128)", g);
+  KSQ_REQUIRE(k % kTileK == 0, KSQ_ERR_UNSUPPORTED, "k=%zu must be a multiple of %d", k, kTileK);
+  KSQ_REQUIRE(n % kTileN == 0, KSQ_ERR_UNSUPPORTED, "n=%zu must be a multiple of %d", n, kTileN);
+  KSQ_REQUIRE(k < (1u << 30) && n < (1u << 30), KSQ_ERR_UNSUPPORTED, "k or n too large");
+  return KSQ_OK;
+}
+
+int ksq_w4a16_repack_sizes(size_t k, size_t n, size_t g, size_t* weight_bytes, size_t* sz_bytes) {
+  int rc = check_w4_shape(k, n, g);
+  if (rc != KSQ_OK) return rc;
+  KSQ_REQUIRE(weight_bytes && sz_bytes, KSQ_ERR_INVALID_ARGUMENT, "null output pointer");
+  *weight_bytes = k * n / 2;
+  *sz_bytes = (k / g) * n * 4;
+  return KSQ_OK;
+}
+
+int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
+  KSQ_REQUIRE(bytes, KSQ_ERR_INVALID_ARGUMENT, "null output pointer");
+  KSQ_REQUIRE(max_m > 0, KSQ_ERR_INVALID_ARGUMENT, "max_m must be positive");
+  int rc = check_w4_shape(k, n, 128);
+  if (rc != KSQ_OK) return rc;
+  const DeviceInfo* di = device_info();
+  const int cus = di ? di->cus : 256;  // sizing only; without a device assume a full MI355X
+  size_t best = 0;
+  const size_t ms[4] = {16, 32, 48, 64};
+  for (size_t mm : ms) {
+    if (mm - 15 > max_m) break;
+    W4Plan p = w4a16_plan(mm, n, k, cus, (size_t)-1);
+    if (p.partial_bytes > best) best = p.partial_bytes;
+  }
+  *bytes = best;
+  return KSQ_OK;
+}
+
+int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                   size_t k, size_t g, void* workspace, size_t workspace_bytes, void* stream) {
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(out && act && weight && sz, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  int rc = check_w4_shape(k, n, g);
+  if (rc != KSQ_OK) return rc;
+  if (m == 0) return KSQ_OK;
+  KSQ_REQUIRE(m < (1u << 24), KSQ_ERR_UNSUPPORTED, "m=%zu too large", m);
+  KSQ_REQUIRE((reinterpret_cast<uintptr_t>(act) & 15) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15) == 0 &&
+                  (reinterpret_cast<uintptr_t>(sz) & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 1) == 0,
+              KSQ_ERR_INVALID_ARGUMENT, "act and weight must be 16-byte aligned");
+  const DeviceInfo* di = device_info();
+  if (!di) return KSQ_ERR_HIP;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(m, n, k, g))
+    return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, s);
+  if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
+  W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
+  return w4a16_launch_stream(dtype, plan, out, act, weight, sz, m, n, k, g, workspace, s);
+}
+
+}  // extern "C"

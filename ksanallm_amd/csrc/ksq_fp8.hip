@@ -1,0 +1,427 @@
+// FP8 e4m3 (OCP) path: activation quantisation, rescale, on-the-fly weight conversion and the streaming GEMM.
+#include "ksq_internal.h"
+
+namespace ksq {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kE4m3Max = 448.0f;
+constexpr float kMinScale = 1.0f / 448.0f / 512.0f;  // FP8_E4M3_MIN_SCALE of the reference
+
+template <typename T>
+__device__ inline float load_as_float(const uint16_t* p, size_t i);
+template <>
+__device__ inline float load_as_float<_Float16>(const uint16_t* p, size_t i) {
+  return (float)__builtin_bit_cast(_Float16, p[i]);
+}
+template <>
+__device__ inline float load_as_float<__bf16>(const uint16_t* p, size_t i) {
+  return __builtin_bit_cast(float, (uint32_t)p[i] << 16);
+}
+
+template <typename T>
+__device__ inline uint16_t float_to_bits(float v);
+template <>
+__device__ inline uint16_t float_to_bits<_Float16>(float v) {
+  return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+template <>
+__device__ inline uint16_t float_to_bits<__bf16>(float v) {
+  return __builtin_bit_cast(uint16_t, (__bf16)v);
+}
+
+// clamp(x / scale, +-448) -> e4m3 code (round to nearest even in hardware)
+__device__ inline uint32_t quantize_pair(float a, float b, float scale) {
+  float x = fminf(fmaxf(a / scale, -kE4m3Max), kE4m3Max);
+  float y = fminf(fmaxf(b / scale, -kE4m3Max), kE4m3Max);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(x, y, 0, false) & 0xFFFFu;
+}
+
+__device__ inline uint8_t quantize_one(float a, float scale) { return (uint8_t)(quantize_pair(a, 0.0f, scale) & 0xFFu); }
+
+__device__ inline float block_max_256(float v, float* smem) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) smem[wave] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3]));
+  __syncthreads();
+  return v;
+}
+
+__global__ void fill_zero_kernel(float* p, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.0f;
+}
+
+// per-tensor abs-max -> scale, merged over blocks with an atomic max on the (non-negative) float bits
+template <typename T>
+__global__ __launch_bounds__(256) void absmax_scale_kernel(const uint16_t* x, size_t count, float* scale) {
+  __shared__ float smem[4];
+  float mx = 0.0f;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256)
+    mx = fmaxf(mx, fabsf(load_as_float<T>(x, i)));
+  mx = block_max_256(mx, smem);
+  if (threadIdx.x == 0) {
+    float s = fmaxf(mx / kE4m3Max, kMinScale);
+    atomicMax(reinterpret_cast<unsigned int*>(scale), __builtin_bit_cast(unsigned int, s));
+  }
+}
+
+// elementwise quantisation with a given scale per channel (channel = row of length channel_size)
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* x, const float* scale, size_t num_channels,
+                                                       size_t channel_size, uint8_t* q) {
+  const size_t ch = blockIdx.y;
+  const float s = scale[ch];
+  const uint16_t* xr = x + ch * channel_size;
+  uint8_t* qr = q + ch * channel_size;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < channel_size; i += (size_t)gridDim.x * 256)
+    qr[i] = quantize_one(load_as_float<T>(xr, i), s);
+}
+
+// per-token: one block per row computes the row's scale and quantises the row
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_per_token_kernel(const uint16_t* x, size_t k, uint8_t* q,
+                                                                 float* scale) {
+  __shared__ float smem[4];
+  const size_t row = blockIdx.x;
+  const uint16_t* xr = x + row * k;
+  uint8_t* qr = q + row * k;
+  float mx = 0.0f;
+  for (size_t i = threadIdx.x; i < k; i += 256) mx = fmaxf(mx, fabsf(load_as_float<T>(xr, i)));
+  mx = block_max_256(mx, smem);
+  const float s = fmaxf(mx / kE4m3Max, kMinScale);
+  if (threadIdx.x == 0) scale[row] = s;
+  for (size_t i = threadIdx.x; i < k; i += 256) qr[i] = quantize_one(load_as_float<T>(xr, i), s);
+}
+
+__device__ inline float e4m3_to_float(uint8_t c) {
+  return __builtin_amdgcn_cvt_f32_fp8((int)c, 0);
+}
+
+__global__ __launch_bounds__(256) void rescale_kernel(const uint8_t* in, uint8_t* out, size_t count,
+                                                      const float* s_in, const float* s_out) {
+  const float r = *s_in / *s_out;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256) {
+    float v = fminf(fmaxf(e4m3_to_float(in[i]) * r, -kE4m3Max), kE4m3Max);  // the cast saturates to +-448
+    out[i] = (uint8_t)((uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.0f, 0, false) & 0xFFu);
+  }
+}
+
+// [k,n] T -> [n,k] e4m3 through a 64x64 LDS tile
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_quantize_kernel(const uint16_t* w, size_t k, size_t n,
+                                                                 const float* scale, uint8_t* wq) {
+  __shared__ uint8_t tile[64][65];
+  const float s = *scale;
+  const size_t k0 = (size_t)blockIdx.y * 64, n0 = (size_t)blockIdx.x * 64;
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    int kk = i >> 6, nn = i & 63;
+    uint8_t v = 0;
+    if (k0 + kk < k && n0 + nn < n) v = quantize_one(load_as_float<T>(w, (k0 + kk) * n + n0 + nn), s);
+    tile[kk][nn] = v;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    int nn = i >> 6, kk = i & 63;
+    if (k0 + kk < k && n0 + nn < n) wq[(n0 + nn) * k + k0 + kk] = tile[kk][nn];
+  }
+}
+
+// ---- streaming GEMM ------------------------------------------------------------------------------------------
+struct Fp8Args {
+  const uint8_t* aq;  // [M][K]
+  const uint8_t* wq;  // [N][K]
+  const float* a_scale;
+  const float* w_scale;
+  void* out;  // [M][N] T
+  f32x4* partial;
+  unsigned* counters;
+  int M, N, K, KB /* 128-byte k blocks, rounded up */, ntiles, ksplit;
+  int a_scale_per_row, w_scale_per_col;
+};
+
+// Wave = one 16-column tile x a range of 128-k blocks.  Each lane reads 2 x 16 B of its weight row per block (the
+// B operands of four 16x16x32 fp8 MFMAs) and the matching 2 x 16 B of each activation row tile.
+template <typename T, int MT, int D>
+__global__ __launch_bounds__(256) void fp8_stream_kernel(Fp8Args p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, j = lane >> 4;
+  const int nt = blockIdx.x * 4 + wave;
+  if (nt >= p.ntiles) return;  // wave-uniform; no block-level barrier below
+  const int split = blockIdx.y, mblock = blockIdx.z;
+  const int kb_begin = (int)(((long)p.KB * split) / p.ksplit);
+  const int kb_end = (int)(((long)p.KB * (split + 1)) / p.ksplit);
+  const int m0 = mblock * 16 * MT;
+
+  int wrow = nt * 16 + c;
+  wrow = wrow < p.N ? wrow : p.N - 1;
+  const uint8_t* wptr = p.wq + (size_t)wrow * p.K + 16 * j;
+  const uint8_t* aptr[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int row = m0 + 16 * mt + c;
+    row = row < p.M ? row : p.M - 1;
+    aptr[mt] = p.aq + (size_t)row * p.K + 16 * j;
+  }
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 wq[D][2];
+  u32x4 aq[D][MT][2];
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  auto fetch = [&](int slot, int kb) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int koff = kb * 128 + 64 * h;
+      const bool ok = koff + 16 * j < p.K;  // K % 16 == 0, so a 16-byte chunk is inside or outside as a whole
+      wq[slot][h] = ok ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + koff)) : zero4;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        aq[slot][mt][h] = ok ? *reinterpret_cast<const u32x4*>(aptr[mt] + koff) : zero4;
+    }
+  };
+  auto consume = [&](int slot) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        u32x2 bw = {wq[slot][h][2 * q], wq[slot][h][2 * q + 1]};
+        const long b = __builtin_bit_cast(long, bw);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          u32x2 aw = {aq[slot][mt][h][2 * q], aq[slot][mt][h][2 * q + 1]};
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(__builtin_bit_cast(long, aw), b, acc[mt], 0, 0, 0);
+        }
+      }
+  };
+
+#pragma unroll
+  for (int i = 0; i < D; ++i)
+    if (kb_begin + i < kb_end) fetch(i, kb_begin + i);
+  for (int kb = kb_begin; kb < kb_end; kb += D) {
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      if (kb + i < kb_end) {
+        consume(i);
+        if (kb + i + D < kb_end) fetch(i, kb + i + D);
+      }
+    }
+  }
+
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int col = nt * 16 + c;
+  const float ws = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
+  auto store_out = [&](int mt, f32x4 v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = m0 + 16 * mt + 4 * j + i;
+      if (row < p.M && col < p.N) {
+        const float as = p.a_scale[p.a_scale_per_row ? row : 0];
+        out[(size_t)row * p.N + col] = float_to_bits<T>((v[i] * ws) * as);
+      }
+    }
+  };
+
+  if (p.ksplit == 1) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) store_out(mt, acc[mt]);
+    return;
+  }
+  const size_t split_stride = (size_t)gridDim.z * p.ntiles * MT * 64;
+  auto pidx = [&](int sp, int mt) {
+    return (size_t)sp * split_stride + (((size_t)mblock * p.ntiles + nt) * MT + mt) * 64 + lane;
+  };
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) p.partial[pidx(split, mt)] = acc[mt];
+  __threadfence();
+  unsigned* ctr = p.counters + (size_t)mblock * p.ntiles + nt;
+  unsigned arrived = 0;
+  if (lane == 0) arrived = atomicAdd(ctr, 1u);
+  arrived = __builtin_amdgcn_readfirstlane(arrived);
+  if (arrived != (unsigned)(p.ksplit - 1)) return;
+  __threadfence();
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < p.ksplit; ++sp) sum += p.partial[pidx(sp, mt)];
+    store_out(mt, sum);
+  }
+  if (lane == 0) atomicExch(ctr, 0u);
+}
+
+template <typename T>
+void launch_fp8_stream(int mt, const Fp8Args& a, dim3 grid, hipStream_t s) {
+  switch (mt) {
+    case 1: hipLaunchKernelGGL((fp8_stream_kernel<T, 1, 4>), grid, dim3(256), 0, s, a); break;
+    case 2: hipLaunchKernelGGL((fp8_stream_kernel<T, 2, 3>), grid, dim3(256), 0, s, a); break;
+    case 3: hipLaunchKernelGGL((fp8_stream_kernel<T, 3, 2>), grid, dim3(256), 0, s, a); break;
+    default: hipLaunchKernelGGL((fp8_stream_kernel<T, 4, 2>), grid, dim3(256), 0, s, a); break;
+  }
+}
+
+unsigned blocks_for(size_t count, unsigned cap) {
+  size_t b = (count + 255) / 256;
+  if (b < 1) b = 1;
+  return (unsigned)(b > cap ? cap : b);
+}
+
+}  // namespace
+}  // namespace ksq
+
+using namespace ksq;
+
+extern "C" {
+
+int ksq_fp8_quantize(int dtype, const void* act, size_t m, size_t k, int mode, void* act_q, float* act_scale,
+                     void* stream) {
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(mode >= KSQ_FP8_PER_TENSOR_DYNAMIC && mode <= KSQ_FP8_PER_TOKEN_DYNAMIC, KSQ_ERR_INVALID_ARGUMENT,
+              "bad quantisation mode %d", mode);
+  KSQ_REQUIRE(act && act_q && act_scale, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if (m == 0 || k == 0) return KSQ_OK;
+  KSQ_REQUIRE(m <= 65535u * 16u, KSQ_ERR_UNSUPPORTED, "m=%zu too large", m);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint16_t* x = static_cast<const uint16_t*>(act);
+  uint8_t* q = static_cast<uint8_t*>(act_q);
+  const bool f16 = dtype == KSQ_F16;
+  if (mode == KSQ_FP8_PER_TOKEN_DYNAMIC) {
+    KSQ_REQUIRE(m < (1ull << 31), KSQ_ERR_UNSUPPORTED, "m too large");
+    if (f16) hipLaunchKernelGGL(quantize_per_token_kernel<_Float16>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
+    else hipLaunchKernelGGL(quantize_per_token_kernel<__bf16>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
+  } else {
+    const size_t count = m * k;
+    if (mode == KSQ_FP8_PER_TENSOR_DYNAMIC) {
+      // a fill kernel rather than a memset node keeps the call safe to record into a HIP graph
+      hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, act_scale, 1);
+      const unsigned nb = blocks_for(count, 2048);
+      if (f16) hipLaunchKernelGGL(absmax_scale_kernel<_Float16>, dim3(nb), dim3(256), 0, s, x, count, act_scale);
+      else hipLaunchKernelGGL(absmax_scale_kernel<__bf16>, dim3(nb), dim3(256), 0, s, x, count, act_scale);
+    }
+    const unsigned nb = blocks_for(count, 4096);
+    if (f16) hipLaunchKernelGGL(quantize_kernel<_Float16>, dim3(nb, 1), dim3(256), 0, s, x, act_scale, (size_t)1, count, q);
+    else hipLaunchKernelGGL(quantize_kernel<__bf16>, dim3(nb, 1), dim3(256), 0, s, x, act_scale, (size_t)1, count, q);
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+int ksq_fp8_rescale(const void* in, void* out, size_t count, const float* scale_in, const float* scale_out,
+                    void* stream) {
+  KSQ_REQUIRE(in && out && scale_in && scale_out, KSQ_ERR_INVALID_ARGUMENT, "null pointer");
+  if (count == 0) return KSQ_OK;
+  hipLaunchKernelGGL(rescale_kernel, dim3(blocks_for(count, 4096)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), count, scale_in, scale_out);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+int ksq_fp8_convert_weight(int dtype, const void* w, size_t k, size_t n, void* w_q, float* w_scale, void* stream) {
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(w && w_q && w_scale, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  KSQ_REQUIRE(k > 0 && n > 0, KSQ_ERR_INVALID_ARGUMENT, "k and n must be positive");
+  KSQ_REQUIRE((k + 63) / 64 <= 65535, KSQ_ERR_UNSUPPORTED, "k too large");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint16_t* x = static_cast<const uint16_t*>(w);
+  const size_t count = k * n;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, w_scale, 1);
+  const unsigned nb = blocks_for(count, 2048);
+  dim3 grid((unsigned)((n + 63) / 64), (unsigned)((k + 63) / 64));
+  if (dtype == KSQ_F16) {
+    hipLaunchKernelGGL(absmax_scale_kernel<_Float16>, dim3(nb), dim3(256), 0, s, x, count, w_scale);
+    hipLaunchKernelGGL(transpose_quantize_kernel<_Float16>, grid, dim3(256), 0, s, x, k, n, w_scale,
+                       static_cast<uint8_t*>(w_q));
+  } else {
+    hipLaunchKernelGGL(absmax_scale_kernel<__bf16>, dim3(nb), dim3(256), 0, s, x, count, w_scale);
+    hipLaunchKernelGGL(transpose_quantize_kernel<__bf16>, grid, dim3(256), 0, s, x, k, n, w_scale,
+                       static_cast<uint8_t*>(w_q));
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+static int check_fp8_shape(size_t n, size_t k) {
+  KSQ_REQUIRE(k > 0 && n > 0, KSQ_ERR_INVALID_ARGUMENT, "k and n must be positive (k=%zu n=%zu)", k, n);
+  KSQ_REQUIRE(k % 16 == 0, KSQ_ERR_UNSUPPORTED, "k=%zu must be a multiple of 16", k);
+  KSQ_REQUIRE(k < (1u << 30) && n < (1u << 30), KSQ_ERR_UNSUPPORTED, "k or n too large");
+  return KSQ_OK;
+}
+
+int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
+  KSQ_REQUIRE(bytes, KSQ_ERR_INVALID_ARGUMENT, "null output pointer");
+  KSQ_REQUIRE(max_m > 0, KSQ_ERR_INVALID_ARGUMENT, "max_m must be positive");
+  int rc = check_fp8_shape(n, k);
+  if (rc != KSQ_OK) return rc;
+  const DeviceInfo* di = device_info();
+  const int cus = di ? di->cus : 256;
+  size_t best = 0;
+  const size_t ms[4] = {16, 32, 48, 64};
+  for (size_t mm : ms) {
+    if (mm - 15 > max_m) break;
+    Fp8Plan p = fp8_plan(mm, n, k, cus, (size_t)-1);
+    if (p.partial_bytes > best) best = p.partial_bytes;
+  }
+  *bytes = best;
+  return KSQ_OK;
+}
+
+int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                 const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                 void* workspace, size_t workspace_bytes, void* stream) {
+  KSQ_REQUIRE(out_dtype == KSQ_F16 || out_dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", out_dtype);
+  KSQ_REQUIRE(out && act_q && w_q, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  // the reference layer refuses a missing weight scale (KS/layers/nvidia/fp8_matmul_layer.cpp:49-51)
+  KSQ_REQUIRE(w_scale != nullptr, KSQ_ERR_INVALID_ARGUMENT, "weight scale is null");
+  KSQ_REQUIRE(act_scale != nullptr, KSQ_ERR_INVALID_ARGUMENT, "activation scale is null");
+  int rc = check_fp8_shape(n, k);
+  if (rc != KSQ_OK) return rc;
+  if (m == 0) return KSQ_OK;
+  KSQ_REQUIRE(act_scale_count == 1 || act_scale_count == m, KSQ_ERR_INVALID_ARGUMENT,
+              "act_scale_count must be 1 or m (got %zu)", act_scale_count);
+  KSQ_REQUIRE(w_scale_count == 1 || w_scale_count == n, KSQ_ERR_INVALID_ARGUMENT,
+              "w_scale_count must be 1 or n (got %zu)", w_scale_count);
+  KSQ_REQUIRE((reinterpret_cast<uintptr_t>(act_q) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_q) & 15) == 0,
+              KSQ_ERR_INVALID_ARGUMENT, "act_q and w_q must be 16-byte aligned");
+  const DeviceInfo* di = device_info();
+  if (!di) return KSQ_ERR_HIP;
+  if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
+  Fp8Plan plan = fp8_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
+  Fp8Args a{};
+  a.aq = static_cast<const uint8_t*>(act_q);
+  a.wq = static_cast<const uint8_t*>(w_q);
+  a.a_scale = act_scale;
+  a.w_scale = w_scale;
+  a.out = out;
+  a.partial = static_cast<f32x4*>(workspace);
+  a.M = (int)m;
+  a.N = (int)n;
+  a.K = (int)k;
+  a.KB = (int)((k + 127) / 128);
+  a.ntiles = (int)((n + 15) / 16);
+  a.ksplit = plan.ksplit;
+  a.a_scale_per_row = act_scale_count > 1 || (m == 1 && false);
+  a.w_scale_per_col = w_scale_count > 1;
+  if (act_scale_count == m && m == 1) a.a_scale_per_row = 0;  // one row: index 0 either way
+  if (w_scale_count == n && n == 1) a.w_scale_per_col = 0;
+  a.counters = nullptr;
+  if (plan.ksplit > 1) {
+    a.counters = counter_slot_device_ptr();
+    if (!a.counters) return KSQ_ERR_HIP;
+  }
+  KSQ_REQUIRE(plan.mblocks <= 65535, KSQ_ERR_UNSUPPORTED, "m too large");
+  dim3 grid((unsigned)((a.ntiles + 3) / 4), (unsigned)plan.ksplit, (unsigned)plan.mblocks);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (out_dtype == KSQ_F16) launch_fp8_stream<_Float16>(plan.MT, a, grid, s);
+  else launch_fp8_stream<__bf16>(plan.MT, a, grid, s);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+// Internal declarations shared by the HIP translation units of libksq.so (not installed).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "ksq.h"
+
+namespace ksq {
+
+// ---- error plumbing (thread-local message behind ksq_last_error_string) -------------------------------------
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define KSQ_HIP_TRY(expr)                                                                      \
+  do {                                                                                         \
+    hipError_t e__ = (expr);                                                                   \
+    if (e__ != hipSuccess) return ::ksq::fail(KSQ_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e__)); \
+  } while (0)
+
+#define KSQ_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) return ::ksq::fail((code), __VA_ARGS__); \
+  } while (0)
+
+// ---- fragment-order geometry -------------------------------------------------------------------------------
+constexpr int kTileN = 16;        // columns per weight tile
+constexpr int kTileK = 128;       // k per weight tile
+constexpr int kTileWords = 256;   // 32-bit words per tile (64 lanes x 4)
+
+// Position of logical element (k, n) in the fragment-order weight buffer: index of the 32-bit word and the
+// nibble inside it.  Tiles are [N/16][K/128]; see include/ksq.h for the definition this implements.
+__host__ __device__ inline void frag_position(size_t k, size_t n, size_t K, size_t* word, int* nibble) {
+  size_t nt = n / kTileN, kt = k / kTileK;
+  int c = (int)(n % kTileN);
+  int kk = (int)(k % kTileK);
+  int d = kk >> 5;        // which of the four MFMAs of the tile
+  int j = (kk >> 3) & 3;  // k sub-group = lane / 16
+  int e = kk & 7;
+  int lane = 16 * j + c;
+  *word = ((nt * (K / kTileK) + kt) * 64 + (size_t)lane) * 4 + (size_t)d;
+  *nibble = (e & 1) ? 4 + (e >> 1) : (e >> 1);
+}
+
+// Inverse for one output word: which (k0, n) the word's eight elements start at.
+__host__ __device__ inline void frag_word_origin(size_t word, size_t K, size_t* k0, size_t* n) {
+  size_t d = word & 3;
+  size_t lane = (word >> 2) & 63;
+  size_t tile = word >> 8;
+  size_t KT = K / kTileK;
+  size_t nt = tile / KT, kt = tile % KT;
+  *n = nt * kTileN + (lane & 15);
+  *k0 = kt * kTileK + 32 * d + 8 * (lane >> 4);
+}
+
+// element e (0..7) of a fragment word lives in this nibble
+__host__ __device__ inline int frag_nibble_of(int e) { return (e & 1) ? 4 + (e >> 1) : (e >> 1); }
+
+// ---- split-K bookkeeping -----------------------------------------------------------------------------------
+// Arrival counters of the split-K fix-up.  They live in library-owned device memory (zero at load, returned
+// to zero by the last-arriving wave of every tile), so no launch has to clear anything.  Launches rotate over
+// kCounterSlots regions so that calls in flight on different streams do not share counters unless more than
+// kCounterSlots overlap.
+constexpr int kCounterSlots = 16;
+constexpr int kCountersPerSlot = 4096;
+unsigned* counter_slot_device_ptr();  // next slot (device address), or nullptr on failure
+
+struct DeviceInfo {
+  int cus;
+};
+const DeviceInfo* device_info();  // of the current device; nullptr on failure
+
+// ---- launch plans ------------------------------------------------------------------------------------------
+struct W4Plan {
+  int MT;       // 16-row tiles per wave (1..4)
+  int NT;       // 16-column tiles per wave
+  int mblocks;  // grid.z
+  int ksplit;   // grid.y
+  size_t partial_bytes;  // workspace the plan needs (0 when ksplit == 1)
+  bool prefill;  // true: LDS-tiled MFMA kernel, false: streaming kernel
+};
+W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+
+int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
+                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
+                         size_t n, size_t k, size_t g, hipStream_t s);
+bool w4a16_prefill_supported(size_t m, size_t n, size_t k, size_t g);
+
+struct Fp8Plan {
+  int MT;
+  int mblocks;
+  int ksplit;
+  size_t partial_bytes;
+  bool prefill;
+};
+Fp8Plan fp8_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+
+}  // namespace ksq

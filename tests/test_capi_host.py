@@ -1,0 +1,135 @@
+"""CPU-side tests of the C ABI: the library loads, exports every declared symbol, validates arguments with the
+documented status codes, and the host repack produces the documented fragment order (checked against an
+independent pure-Python statement of the layout).  No compute entry point is called on a device here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from ksanallm_amd import capi
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "ksq.h")).read()
+    declared = set(re.findall(r"\b(ksq_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    L = capi.lib()
+    for name in sorted(declared):
+        assert hasattr(L, name), f"libksq.so does not export {name}"
+    assert set(capi.EXPORTS) == declared
+    assert capi.version() >= 100
+
+
+def _expected_words(u):
+    K, N = u.shape
+    words = np.zeros(K * N // 8, dtype=np.uint32)
+    for k in range(K):
+        for n in range(N):
+            nt, kt, c, kk = n // 16, k // 128, n % 16, k % 128
+            d, j, e = kk >> 5, (kk >> 3) & 3, kk & 7
+            w = ((nt * (K // 128) + kt) * 64 + 16 * j + c) * 4 + d
+            nib = 4 + e // 2 if e & 1 else e // 2
+            words[w] |= np.uint32(int(u[k, n]) << (4 * nib))
+    return words
+
+
+@pytest.mark.parametrize("g", [64, 128])
+def test_host_repack_fragment_order(g):
+    rng = np.random.default_rng(31)
+    K, N = 256, 48
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8)
+    s = orc.to_bits(np.abs(rng.standard_normal((K // g, N))) * 0.02 + 1e-3, orc.BF16)
+    want = _expected_words(u)
+    sources = [
+        (capi.W4_GPTQ_INT32_KPACK, orc.gptq_pack(u)),
+        (capi.W4_AWQ_INT32_NPACK, orc.awq_pack(u)),
+        (capi.W4_ROWMAJOR_INT4_SIGNED, orc.rowmajor_pack(u)),
+    ]
+    zero_forms = [
+        (capi.ZERO_UINT8, z, z),
+        (capi.ZERO_AWQ_INT32, orc.awq_pack(z), z),
+        (capi.ZERO_ADDITIVE, orc.awq_additive_zeros(s, orc.BF16, z), z),
+        (capi.ZERO_NONE, None, np.full_like(z, 8)),
+    ]
+    for layout, src in sources:
+        for zk, zsrc, zwant in zero_forms:
+            dw = np.zeros(K * N // 8, dtype=np.uint32)
+            dsz = np.zeros((K // g) * N, dtype=np.uint32)
+            capi.w4a16_repack_host(layout, src, zk, zsrc, s, capi.BF16, K, N, g, dw, dsz)
+            assert np.array_equal(dw, want)
+            szw = dsz.reshape(N // 16, K // g, 16).transpose(1, 0, 2).reshape(K // g, N)
+            assert np.array_equal((szw & 0xFFFF).astype(np.uint16), s)
+            assert np.array_equal((szw >> 16).astype(np.uint8), zwant)
+
+
+def test_additive_zero_recovery_fp16_all_values():
+    # every z in [0,15] against a spread of scales, including tiny and large ones
+    scales = np.array([1e-3, 0.0123, 0.02, 0.5, 1.0, 3.3, 6e-5, 100.0], dtype=np.float32)
+    K, g = 128, 128
+    N = 16 * len(scales)
+    sv = np.repeat(scales, 16)[None, :]
+    z = np.tile(np.arange(16, dtype=np.uint8), len(scales))[None, :]
+    s = orc.to_bits(sv, orc.F16)
+    za = orc.awq_additive_zeros(s, orc.F16, z)
+    u = np.zeros((K, N), dtype=np.uint8)
+    dw = np.zeros(K * N // 8, dtype=np.uint32)
+    dsz = np.zeros(N, dtype=np.uint32)
+    capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, orc.gptq_pack(u), capi.ZERO_ADDITIVE, za, s, capi.F16, K, N, g,
+                           dw, dsz)
+    got = (dsz.reshape(N // 16, 1, 16) >> 16).astype(np.uint8).transpose(1, 0, 2).reshape(1, N)
+    assert np.array_equal(got, z)
+
+
+def test_sizes_and_argument_validation():
+    assert capi.w4a16_repack_sizes(4096, 4096, 128) == (4096 * 4096 // 2, 32 * 4096 * 4)
+    for k, n, g in [(100, 64, 128), (256, 24, 128), (256, 64, 32), (0, 64, 128)]:
+        with pytest.raises(capi.KsqError) as ei:
+            capi.w4a16_repack_sizes(k, n, g)
+        assert ei.value.code in (capi.ERR_UNSUPPORTED, capi.ERR_INVALID_ARGUMENT)
+    buf = np.zeros(64, dtype=np.uint8)
+    with pytest.raises(capi.KsqError) as ei:  # null tensor
+        capi.w4a16_gemm(capi.F16, None, buf, buf, buf, 1, 16, 128, 128)
+    assert ei.value.code == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(capi.KsqError) as ei:  # the reference kernels also refuse other group sizes
+        capi.w4a16_gemm(capi.F16, buf, buf, buf, buf, 1, 16, 128, 32)
+    assert ei.value.code == capi.ERR_UNSUPPORTED
+    with pytest.raises(capi.KsqError) as ei:  # k not a multiple of the tile
+        capi.w4a16_gemm(capi.F16, buf, buf, buf, buf, 1, 16, 192, 64)
+    assert ei.value.code == capi.ERR_UNSUPPORTED
+    with pytest.raises(capi.KsqError) as ei:  # bad dtype
+        capi.w4a16_gemm(7, buf, buf, buf, buf, 1, 16, 128, 128)
+    assert ei.value.code == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(capi.KsqError) as ei:  # weight scale missing: the reference layer throws too
+        capi.fp8_gemm(capi.BF16, buf, buf, buf, 1, buf, None, 1, 1, 16, 64)
+    assert ei.value.code == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(capi.KsqError) as ei:
+        capi.fp8_gemm(capi.BF16, buf, buf, buf, 3, buf, buf, 1, 2, 16, 64)  # act_scale_count not 1 or m
+    assert ei.value.code == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(capi.KsqError) as ei:
+        capi.fp8_quantize(capi.F16, buf, 1, 16, 9, buf, buf)
+    assert ei.value.code == capi.ERR_INVALID_ARGUMENT
+    assert "mode" in str(ei.value)
+
+
+def test_empty_inputs_are_noops():
+    buf = np.zeros(64, dtype=np.uint8)
+    capi.w4a16_gemm(capi.F16, buf, buf, buf, buf, 0, 16, 128, 128)  # m = 0
+    capi.fp8_gemm(capi.F16, buf, buf, buf, 1, buf, buf, 1, 0, 16, 64)
+    capi.fp8_quantize(capi.F16, buf, 0, 16, capi.FP8_PER_TOKEN_DYNAMIC, buf, buf)
+    capi.fp8_rescale(buf, buf, 0, buf, buf)
+
+
+def test_workspace_sizes_are_monotone_and_bounded():
+    for n, k in [(4096, 4096), (12288, 4096), (22016, 4096), (4096, 11008), (57344, 8192)]:
+        w16 = capi.w4a16_workspace_bytes(16, n, k)
+        w64 = capi.w4a16_workspace_bytes(64, n, k)
+        w4096 = capi.w4a16_workspace_bytes(4096, n, k)
+        assert w16 <= w64 == w4096
+        assert w64 <= k * n // 2  # never more than the weights themselves
+    assert capi.fp8_workspace_bytes(64, 8192, 8192) <= 8192 * 8192

@@ -1,0 +1,176 @@
+"""W4A16 parity tests proper: the HIP path through the C ABI against the CPU oracle on the same seeded bytes.
+Bar: max relative error <= 1e-2 (denominator floored at RMS of the oracle output) and mean absolute error
+<= 2e-3 x RMS, fp32 accumulation; integer and one-hot cases must match bit for bit."""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as orc
+from tests.ksq_testlib import ORC_DT, W4Case, W4Device, bits_of
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print(f"\n[case] {request.node.nodeid}", flush=True)
+    yield
+
+
+def _env(**kv):
+    class _Ctx:
+        def __enter__(self):
+            self.old = {k: os.environ.get(k) for k in kv}
+            for k, v in kv.items():
+                os.environ[k] = str(v)
+
+        def __exit__(self, *a):
+            for k, v in self.old.items():
+                if v is None:
+                    os.environ.pop(k, None)
+                else:
+                    os.environ[k] = v
+
+    return _Ctx()
+
+
+@pytest.mark.parametrize("layout", ["gptq", "awq", "rowmajor"])
+def test_device_repack_matches_host_repack(gpu, layout):
+    from ksanallm_amd import capi
+
+    case = W4Case(100, 4, 512, 96, g=64, kind="awq", dtype="f16")
+    dev = W4Device(case, gpu, layout=layout)
+    wb, sb = capi.w4a16_repack_sizes(case.K, case.N, case.g)
+    hw = np.zeros(wb // 4, dtype=np.uint32)
+    hs = np.zeros(sb // 4, dtype=np.uint32)
+    capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, case.gptq_qweight(), capi.ZERO_UINT8, case.z, case.scales,
+                           capi.F16, case.K, case.N, case.g, hw, hs)
+    assert np.array_equal(dev.weight.cpu().numpy().view(np.uint32), hw)
+    assert np.array_equal(dev.sz.cpu().numpy().view(np.uint32), hs)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("kind,g", [("gptq", 128), ("awq", 128), ("awq", 64)])
+def test_one_hot_rows_return_dequantized_rows_exactly(gpu, dtype, kind, g):
+    K, N = 512, 128
+    rows = [0, 1, 7, 8, 31, 32, 63, 64, 127, 128, 255, 256, 300, 383, 510, 511]
+    act = np.zeros((len(rows), K), dtype=np.float32)
+    for i, k in enumerate(rows):
+        act[i, k] = 1.0
+    case = W4Case(101, len(rows), K, N, g=g, kind=kind, dtype=dtype, act=act)
+    out = W4Device(case, gpu).gemm()
+    want = orc.to_bits(case.dequantized()[rows], ORC_DT[dtype])
+    assert np.array_equal(bits_of(out), want)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_integer_case_is_exact(gpu, dtype):
+    M, K, N = 7, 256, 64
+    rng = np.random.default_rng(102)
+    act = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    case = W4Case(102, M, K, N, kind="awq", dtype=dtype, act=act, scales=np.ones((K // 128, N), dtype=np.float32))
+    got = W4Device(case, gpu).gemm_f32()
+    want = act.astype(np.int64) @ (case.u.astype(np.int64) - np.repeat(case.z, 128, axis=0).astype(np.int64))
+    # the fp32 sums are exact integers; the output rounding to T is the same round-to-nearest-even on both sides
+    want_bits = orc.to_bits(want.astype(np.float32), ORC_DT[dtype])
+    assert np.array_equal(orc.to_bits(got, ORC_DT[dtype]), want_bits)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 100, 128, 200])
+def test_m_sweep_small_shape(gpu, dtype, M):
+    case = W4Case(1000 + M, M, 1024, 320, kind="awq", dtype=dtype)
+    got = W4Device(case, gpu).gemm_f32()
+    orc.assert_parity(got, case.oracle(), f"M={M} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("kind,g", [("gptq", 128), ("gptq", 64), ("awq", 64)])
+def test_group_sizes_and_kinds(gpu, dtype, kind, g):
+    case = W4Case(1100, 9, 768, 208, g=g, kind=kind, dtype=dtype)
+    orc.assert_parity(W4Device(case, gpu).gemm_f32(), case.oracle(), f"{kind} g={g} {dtype}")
+
+
+@pytest.mark.parametrize("ksplit", [1, 2, 3, 5, 8])
+@pytest.mark.parametrize("nt", [1, 2])
+@pytest.mark.parametrize("dtype,M", [("f16", 16), ("bf16", 33)])
+def test_forced_split_k_and_tile_widths(gpu, dtype, M, ksplit, nt):
+    case = W4Case(1200 + ksplit, M, 1024, 272, kind="awq", dtype=dtype)  # 17 column tiles: ragged for nt = 2
+    dev = W4Device(case, gpu)
+    import torch
+
+    big = torch.empty(64 << 20, dtype=torch.uint8, device=gpu)
+    dev.workspace, dev.workspace_bytes = big, big.numel()
+    with _env(KSQ_W4_KSPLIT=ksplit, KSQ_W4_NT=nt):
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()  # counters must have returned to zero
+    want = case.oracle()
+    orc.assert_parity(got1, want, f"ksplit={ksplit} nt={nt}")
+    assert np.array_equal(got1, got2), "split-K result must be deterministic and repeatable"
+
+
+def test_no_workspace_still_correct(gpu):
+    case = W4Case(1300, 16, 4096, 512, kind="gptq", dtype="f16")
+    dev = W4Device(case, gpu)
+    a = dev.gemm_f32(use_workspace=True)
+    b = dev.gemm_f32(use_workspace=False)
+    want = case.oracle()
+    orc.assert_parity(a, want, "with workspace")
+    orc.assert_parity(b, want, "without workspace")
+
+
+def test_config0_gptq_m16_4096x4096(gpu):
+    case = W4Case(0, 16, 4096, 4096, kind="gptq", dtype="f16")
+    m = orc.assert_parity(W4Device(case, gpu).gemm_f32(), case.oracle(), "cfg0")
+    print("cfg0 metrics", m)
+
+
+SHAPES_7B = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
+
+
+@pytest.mark.parametrize("K,N", SHAPES_7B)
+def test_config1_awq_decode_sweep(gpu, K, N):
+    import torch
+
+    case = W4Case(1000 + K + N, 64, K, N, kind="awq", dtype="f16")
+    dev = W4Device(case, gpu)
+    want = case.oracle()
+    for M in (1, 4, 16, 64):
+        got = dev.gemm(act=dev.act[:M].contiguous()).float().cpu().numpy()
+        orc.assert_parity(got, want[:M], f"cfg1 K={K} N={N} M={M}")
+    del dev
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("K,N", [(4096, 4096), (11008, 4096)])
+def test_config2_awq_bf16_prefill_rows_subset(gpu, K, N):
+    """M = 512 through the product path; the oracle checks a seeded subset of rows (the full product is the
+    bench's job)."""
+    case = W4Case(2000 + K + N, 512, K, N, kind="awq", dtype="bf16")
+    got = W4Device(case, gpu).gemm_f32()
+    rows = np.random.default_rng(5).choice(512, size=24, replace=False)
+    rows.sort()
+    orc.assert_parity(got[rows], case.oracle(rows=rows), f"cfg2 K={K} N={N}")
+
+
+def test_linearity_at_full_size(gpu):
+    """Size-independent property at a full 7B shape: f(a + b) = f(a) + f(b) when a, b and a + b are exactly
+    representable and the fp16 results do not round differently (integer activations, unit scales)."""
+    K, N, M = 4096, 12288, 16
+    rng = np.random.default_rng(7)
+    # sparse {-1,0,1} activations keep every |sum| far below 2^11 units, where fp16 is exact
+    a = (rng.integers(-1, 2, size=(M, K)) * (rng.random((M, K)) < 0.25)).astype(np.float32)
+    b = (rng.integers(-1, 2, size=(M, K)) * (rng.random((M, K)) < 0.25)).astype(np.float32)
+    ones = np.full((K // 128, N), 2.0**-6, dtype=np.float32)
+    ca = W4Case(7, M, K, N, kind="awq", dtype="f16", act=a, scales=ones)
+    dev = W4Device(ca, gpu)
+    import torch
+
+    def run(x):
+        t = torch.from_numpy(orc.to_bits(x, orc.F16).view(np.int16)).to(gpu).view(torch.float16)
+        return dev.gemm(act=t).float().cpu().numpy().astype(np.float64)
+
+    fa, fb, fab = run(a), run(b), run(a + b)
+    # every value is an integer multiple of 2^-6 below 2^11 * 2^-6, so all three are exact
+    assert np.array_equal(fa + fb, fab)
