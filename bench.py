@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Roofline bench of the quantized linear-layer path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: the four W4A16 GEMMs of a Llama-2-7B
+decoder layer (qkv 4096x12288, o 4096x4096, gate_up 4096x22016, down 11008x4096; AWQ asymmetric int4, g = 128,
+fp16 activations N(0,1)) at M = 16 tokens.  Consecutive steps use different layers (8 distinct weight sets,
+~830 MB) so that no launch re-reads weights that are still resident in the 256 MB last-level cache.  All inputs
+are resident in HBM before the timed region; the K timed steps are one HIP graph on one stream, bracketed by
+events on that stream.
+
+Prints ONE JSON line: value = whole-job algorithmic GB/s, plus `roofline` for the dominant kernel (the W4A16
+streaming kernel) and `cpu_baseline` (the CPU oracle -- dequantize to fp32 + blocked OpenMP GEMM -- timed on the
+same workload on this machine's host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+METRIC = "W4A16 GEMM GB/s (M≤16) & TFLOP/s (M=4096), Llama-7B shapes, 1×MI355X"
+SHAPES_7B = [("qkv", 4096, 12288), ("o", 4096, 4096), ("gate_up", 4096, 22016), ("down", 11008, 4096)]
+GROUP = 128
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "w4a16_stream_cfg1_m16_pmc.txt")
+
+
+def w4a16_bytes(m, k, n, awq=True):
+    """Algorithmic bytes of one GEMM: int4 weights + scales + (AWQ) uint4 zeros + activations + output."""
+    g = k // GROUP
+    return k * n // 2 + g * n * 2 + (g * n // 2 if awq else 0) + m * k * 2 + m * n * 2
+
+
+class Layer:
+    """One decoder layer's four AWQ weights, generated on the GPU and repacked through the C ABI."""
+
+    def __init__(self, torch, capi, device, seed, dtype, keep_source=False):
+        self.weights = []
+        self.source = []
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed)
+        tdt = torch.float16 if dtype == capi.F16 else torch.bfloat16
+        for name, k, n in SHAPES_7B:
+            g = k // GROUP
+            qweight = torch.randint(-2**31, 2**31 - 1, (k, n // 8), dtype=torch.int32, device=device, generator=gen)
+            qzeros = torch.randint(-2**31, 2**31 - 1, (g, n // 8), dtype=torch.int32, device=device, generator=gen)
+            scales = (torch.randn((g, n), device=device, generator=gen).abs() * 0.02 + 1e-3).to(tdt)
+            wb, sb = capi.w4a16_repack_sizes(k, n, GROUP)
+            w = torch.empty(wb, dtype=torch.uint8, device=device)
+            sz = torch.empty(sb // 4, dtype=torch.int32, device=device)
+            capi.w4a16_repack(capi.W4_AWQ_INT32_NPACK, qweight, capi.ZERO_AWQ_INT32, qzeros, scales, dtype, k, n,
+                              GROUP, w, sz)
+            self.weights.append((name, k, n, w, sz))
+            if keep_source:
+                self.source.append((qweight.cpu().numpy(), qzeros.cpu().numpy(), scales))
+        torch.cuda.synchronize()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--m", type=int, default=16, help="tokens per step in the headline workload")
+    ap.add_argument("--layers", type=int, default=8, help="distinct weight sets rotated over")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
+
+    import numpy as np
+    import torch
+
+    from ksanallm_amd import capi
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    M = args.m
+    dtype = capi.F16
+    layers = [Layer(torch, capi, dev, 1000 + i, dtype, keep_source=(i == 0)) for i in range(args.layers)]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    acts = {k: torch.randn((M, k), device=dev, generator=gen).to(torch.float16) for k in (4096, 11008)}
+    outs = {n: torch.empty((M, n), dtype=torch.float16, device=dev) for n in (12288, 4096, 22016)}
+    ws_bytes = max(capi.w4a16_workspace_bytes(M, n, k) for _, k, n in SHAPES_7B)
+    workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+
+    stream = torch.cuda.Stream(device=dev)
+    sp = stream.cuda_stream
+
+    def step(i):
+        for _, k, n, w, sz in layers[i % len(layers)].weights:
+            capi.w4a16_gemm(dtype, outs[n], acts[k], w, sz, M, n, k, GROUP, workspace, ws_bytes, sp)
+
+    with torch.cuda.stream(stream):
+        for i in range(args.warmup):
+            step(i)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(args.steps):
+                step(i)
+        graph.replay()  # untimed: first replay uploads the graph
+        stream.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record(stream)
+        graph.replay()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        gpu_ms = ev0.elapsed_time(ev1)
+
+    step_bytes = sum(w4a16_bytes(M, k, n) for _, k, n in SHAPES_7B)
+    ms_per_step = wall_ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launches = args.steps * len(SHAPES_7B)
+    avg_launch_us = gpu_ms * 1e3 / launches
+    achieved = (step_bytes / len(SHAPES_7B)) / (avg_launch_us * 1e-6) / 1e9
+    traffic = None
+    if os.path.exists(TRAFFIC_FILE):
+        for line in open(TRAFFIC_FILE):
+            if line.startswith("traffic_bytes_per_launch:"):
+                traffic = float(line.split(":")[1])
+
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"configs[1]: Llama-2-7B decode, AWQ int4 g=128, fp16 act, M={M}; step = qkv+o+gate_up+down "
+                        f"GEMMs of one layer, {args.layers} layers rotated",
+            "bytes_per_step": step_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "w4a16_stream_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "avg_launch_us": round(avg_launch_us, 3),
+            "launches": launches,
+        },
+    }
+
+    extra = {}
+    if not args.no_extra:
+        extra["per_shape"] = per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, dtype)
+        extra["prefill_m4096"] = prefill(torch, capi, layers[0], dev, stream)
+    if not args.no_cpu:
+        result["cpu_baseline"], extra["parity_vs_cpu"] = cpu_baseline(np, torch, capi, layers[0], acts, outs,
+                                                                      workspace, ws_bytes, M, dtype, step_bytes)
+    if extra:
+        result["extra"] = extra
+    print(json.dumps(result), flush=True)
+
+
+def time_graph(torch, stream, launch, count):
+    """Average device time per launch (us) of `count` back-to-back launches replayed as one graph."""
+    with torch.cuda.stream(stream):
+        for i in range(min(count, 4)):
+            launch(i)
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(count):
+                launch(i)
+        g.replay()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        g.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / count
+
+
+def per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, dtype):
+    table = {}
+    for idx, (name, k, n) in enumerate(SHAPES_7B):
+        def launch(i, idx=idx, k=k, n=n):
+            _, _, _, w, sz = layers[i % len(layers)].weights[idx]
+            capi.w4a16_gemm(dtype, outs[n], acts[k], w, sz, M, n, k, GROUP, workspace, ws_bytes, stream.cuda_stream)
+
+        us = time_graph(torch, stream, launch, 64)
+        b = w4a16_bytes(M, k, n)
+        table[name] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 3)}
+    return table
+
+
+def prefill(torch, capi, layer, dev, stream):
+    """configs[2] at M = 4096 (bf16 activations): TFLOP/s per shape against the dense MFMA peak.  The weights are
+    the fp16-scaled set of layer 0 re-used with bf16 activations only for timing (the arithmetic is the same)."""
+    M = 4096
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    table = {}
+    for name, k, n, w, sz in layer.weights:
+        act = torch.randn((M, k), device=dev, generator=gen).to(torch.bfloat16)
+        out = torch.empty((M, n), dtype=torch.bfloat16, device=dev)
+
+        def launch(i):
+            capi.w4a16_gemm(capi.BF16, out, act, w, sz, M, n, k, GROUP, None, 0, stream.cuda_stream)
+
+        us = time_graph(torch, stream, launch, 4)
+        tf = 2.0 * M * k * n / us / 1e6
+        table[name] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        del act, out
+    return table
+
+
+def cpu_baseline(np, torch, capi, layer, acts, outs, workspace, ws_bytes, M, dtype, step_bytes):
+    """The CPU oracle on the same workload (one full step = the four GEMMs of layer 0), timed on this machine's
+    host cores; its output doubles as a parity check of the GPU result for that layer."""
+    from oracle import oracle as orc
+
+    cases = []
+    for (name, k, n, w, sz), (qw, qz, scales) in zip(layer.weights, layer.source):
+        u = orc.awq_unpack(qw)
+        z = orc.awq_unpack(qz)
+        s_bits = scales.view(torch.int16).cpu().numpy().view(np.uint16)
+        a_bits = acts[k].view(torch.int16).cpu().numpy().view(np.uint16)
+        scratch = (np.empty((k, n), dtype=np.float32), np.empty((M, k), dtype=np.float32))
+        cases.append((name, k, n, u, z, s_bits, a_bits, scratch, w, sz))
+
+    def one_step():
+        return [orc.w4a16_forward(a, orc.F16, u, s, orc.F16, z, GROUP, scratch)
+                for (_, _, _, u, z, s, a, scratch, _, _) in cases]
+
+    one_step()  # warm-up (page-faults the scratch buffers)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        cpu_out = one_step()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    worst = {"max_rel": 0.0, "mean_abs_over_rms": 0.0}
+    for (name, k, n, u, z, s, a, scratch, w, sz), want in zip(cases, cpu_out):
+        capi.w4a16_gemm(dtype, outs[n], acts[k], w, sz, M, n, k, GROUP, workspace, ws_bytes, None)
+        torch.cuda.synchronize()
+        m = orc.error_metrics(outs[n].float().cpu().numpy(), want)
+        worst = {key: max(worst[key], m[key]) for key in worst}
+    base = {
+        "value": round(step_bytes / t / 1e9, 3),
+        "unit": "GB/s",
+        "cores": orc.num_threads(),
+        "kind": "port",
+        "sample": f"one full step (4 GEMMs, M={M}), median of 3 runs, {t:.3f} s per step; dequantize to fp32 + blocked "
+                  f"OpenMP GEMM",
+    }
+    return base, {k: float(f"{v:.3e}") for k, v in worst.items()}
+
+
+if __name__ == "__main__":
+    main()

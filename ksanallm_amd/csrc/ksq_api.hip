@@ -76,36 +76,44 @@ static int env_int(const char* name, int dflt) {
 }
 
 // ---- launch planning ------------------------------------------------------------------------------------------
-// The streaming kernel gives every wave NT column tiles x a contiguous range of k tiles.  Split-K buys
-// parallelism for narrow N at the price of fp32 partial tiles written and read once each, so it is bounded both
-// by the workspace and by a traffic budget relative to the weight bytes.
+// The streaming kernel gives every wave NT column tiles x a contiguous range of k tiles and keeps D tiles per
+// column tile in flight.  What bounds it on narrow N is the number of bytes in flight, i.e. the number of waves:
+// about one wave per SIMD (4 per CU) is needed before HBM latency is covered.  Splitting k across workgroups
+// (grid.y) buys those waves at the price of fp32 partial tiles written and read once each plus three dependent
+// trips to device memory (~3 us measured), so it is used only when the column tiles alone give fewer than one wave
+// per SIMD, and it is bounded by the workspace and by a traffic budget relative to the weight bytes.  k can also
+// be sliced inside a workgroup (reduced through LDS); measured slower than one slice on MI355X for the decode
+// shapes, so it is off by default (KSQ_W4_SLICES selects it).
 W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   W4Plan p{};
   const size_t ntiles = n / kTileN, ktiles = k / kTileK;
+  const size_t simds = (size_t)cus * 4;
   p.prefill = false;
   if (m <= 64) {
     p.MT = (int)((m + 15) / 16);
     p.mblocks = 1;
-    p.NT = 1;
+    p.NT = (p.MT >= 2 || ntiles >= simds) ? 2 : 1;
   } else {
     p.MT = 4;
     p.mblocks = (int)((m + 63) / 64);
     p.NT = 2;
   }
   int nt_env = env_int("KSQ_W4_NT", 0);
-  if (nt_env == 1 || nt_env == 2) p.NT = nt_env;
+  if (nt_env == 1 || nt_env == 2 || nt_env == 4) p.NT = nt_env;
+  p.slices = 1;
+  int sl_env = env_int("KSQ_W4_SLICES", 0);
+  const int max_slices = m <= 64 ? w4a16_stream_max_slices(p.MT, p.NT) : 1;
+  if (sl_env == 1 || (sl_env == 2 && max_slices >= 2) || (sl_env == 4 && max_slices >= 4)) p.slices = sl_env;
   const size_t ngroups = (ntiles + p.NT - 1) / p.NT;
-  const size_t wgs = ((ngroups + 3) / 4) * (size_t)p.mblocks;
   size_t ksplit = 1;
   if (m <= 64) {
-    const size_t target = (size_t)cus * 4;
-    ksplit = (target + wgs / 2) / wgs;
+    size_t wanted = simds / ngroups;  // waves per split = ngroups
     const size_t mpad = (size_t)p.MT * 16;
-    size_t traffic_cap = k / (64 * mpad);  // partial write+read <= 25% of the weight bytes
-    if (ksplit > traffic_cap) ksplit = traffic_cap;
-    if (ksplit > ktiles / 2) ksplit = ktiles / 2;
-    if (ksplit > 16) ksplit = 16;
-    if (ksplit < 1) ksplit = 1;
+    size_t cap = k / (32 * mpad);  // partial write + read <= 50% of the weight bytes
+    if (cap > ktiles / 4) cap = ktiles / 4;  // at least four k tiles per wave
+    if (wanted > cap) wanted = cap;
+    if (wanted < 1) wanted = 1;
+    ksplit = wanted;
     int ks_env = env_int("KSQ_W4_KSPLIT", 0);
     if (ks_env >= 1 && (size_t)ks_env <= ktiles) ksplit = (size_t)ks_env;
     if (ngroups * (size_t)p.mblocks > (size_t)kCountersPerSlot) ksplit = 1;

@@ -240,21 +240,21 @@ __global__ __launch_bounds__(256) void fp8_stream_kernel(Fp8Args p) {
     return (size_t)sp * split_stride + (((size_t)mblock * p.ntiles + nt) * MT + mt) * 64 + lane;
   };
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) p.partial[pidx(split, mt)] = acc[mt];
-  __threadfence();
+  for (int mt = 0; mt < MT; ++mt) store_agent(p.partial + pidx(split, mt), acc[mt]);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores are acknowledged
   unsigned* ctr = p.counters + (size_t)mblock * p.ntiles + nt;
   unsigned arrived = 0;
-  if (lane == 0) arrived = atomicAdd(ctr, 1u);
+  if (lane == 0) arrived = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   arrived = __builtin_amdgcn_readfirstlane(arrived);
   if (arrived != (unsigned)(p.ksplit - 1)) return;
-  __threadfence();
+  asm volatile("" ::: "memory");
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < p.ksplit; ++sp) sum += p.partial[pidx(sp, mt)];
+    for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + pidx(sp, mt));
     store_out(mt, sum);
   }
-  if (lane == 0) atomicExch(ctr, 0u);
+  if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <typename T>

@@ -65,6 +65,29 @@ constexpr int kCounterSlots = 16;
 constexpr int kCountersPerSlot = 4096;
 unsigned* counter_slot_device_ptr();  // next slot (device address), or nullptr on failure
 
+#if defined(__HIPCC__)
+// Split-K partial tiles cross workgroups (and XCDs, each with its own L2) through agent-scope relaxed atomics:
+// the stores write through and the loads miss the non-coherent caches, so no whole-cache write-back or
+// invalidate is needed around the arrival counter.
+typedef float ksq_f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long ksq_u64x2 __attribute__((ext_vector_type(2)));
+
+__device__ inline void store_agent(ksq_f32x4* p, ksq_f32x4 v) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+  ksq_u64x2 w = __builtin_bit_cast(ksq_u64x2, v);
+  __hip_atomic_store(q, w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 1, w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ inline ksq_f32x4 load_agent(const ksq_f32x4* p) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(const_cast<ksq_f32x4*>(p));
+  ksq_u64x2 w;
+  w[0] = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  w[1] = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __builtin_bit_cast(ksq_f32x4, w);
+}
+#endif
+
 struct DeviceInfo {
   int cus;
 };
@@ -76,6 +99,7 @@ struct W4Plan {
   int NT;       // 16-column tiles per wave
   int mblocks;  // grid.z
   int ksplit;   // grid.y
+  int slices;   // k slices inside one workgroup (4 waves each)
   size_t partial_bytes;  // workspace the plan needs (0 when ksplit == 1)
   bool prefill;  // true: LDS-tiled MFMA kernel, false: streaming kernel
 };
@@ -86,6 +110,7 @@ int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* ac
 int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
                          size_t n, size_t k, size_t g, hipStream_t s);
 bool w4a16_prefill_supported(size_t m, size_t n, size_t k, size_t g);
+int w4a16_stream_max_slices(int mt, int nt);
 
 struct Fp8Plan {
   int MT;

@@ -1,33 +1,41 @@
 // W4A16 streaming kernel (decode regime, M <= 64; also the fallback for shapes the prefill kernel does not take).
 //
-// HBM-bound: every wave streams 1 KiB weight tiles (one 128-bit load per lane = the B operands of four
-// 16x16x32 MFMAs), unpacks nibbles to exact small integers in registers, multiplies on the matrix cores and
-// applies the group scale to the fp32 group sum.  Weights are read exactly once; activations come from L2.
+// HBM-bound.  A workgroup is KS k-slices x 4 waves: the four waves of a slice own 4 x NT column tiles and share
+// the slice's range of k tiles.  Every wave streams its 1 KiB weight tiles straight from HBM into a register ring
+// D tiles deep (one 128-bit buffer load per lane is the B operand of four 16x16x32 MFMAs), while the activations
+// of the slice's k range are staged once per slice into LDS in MFMA fragment order (double-buffered chunks of KCT
+// tiles) and read back with conflict-free ds_read_b128.  Weights are read exactly once.
 //
-//   fp16: B = (u - z) exactly, built with two bit operations and one packed subtract per register.
-//   bf16: gfx950 has no packed bf16 arithmetic, so B = 128 + u (pure bit operations) and the bias is removed
-//         per group in fp32:  acc += s * (P - (128 + z) * R),  R = row sums of the activations over the group,
-//         obtained from one extra MFMA against a vector of ones (exact products, fp32 sums).
-#include <type_traits>
-
+// Arithmetic: nibble u becomes the 16-bit pattern of bias + u with bit operations only (fp16: 1024 + u for
+// nibbles at bits 0-3 of a half, 64 + u for nibbles at bits 4-7; bf16: 128 + u), which is exact.  A second MFMA per
+// 32-k step multiplies the same activations with the per-column constant -(bias + z), so the accumulator holds the
+// exact-integer group sum  sum_k a[m,k] * (u[k,n] - z[g,n])  (exact products, fp32 sums); the group scale is then
+// applied in fp32:  acc += s[g,n] * P.  No floating-point VALU work is spent per weight.
+//
+// The k slices of a workgroup are reduced through LDS; a further split of k across workgroups (grid.y) is reduced
+// by the last-arriving workgroup through a device-memory workspace.
+//
+// All global reads are range-checked buffer loads whose resource covers exactly the wave's k range of one column
+// tile: tiles past the end of the range and padding column tiles read as zero without touching memory, which
+// keeps the pipeline free of branches (the hardware retires loads in order, and the compiler can only leave later
+// prefetches in flight across a wait when the number of loads issued after it is known statically).
 #include "ksq_internal.h"
 
 namespace ksq {
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 struct StreamArgs {
-  const u32x4* weight;  // [ntiles][KT][64]
-  const uint32_t* sz;   // [ntiles][G][16]
-  const void* act;      // [M][K]
-  void* out;            // [M][N]
-  f32x4* partial;       // [ksplit][mblocks][ntiles][MT][64]
-  unsigned* counters;   // [mblocks * ngroups]
+  const void* weight;  // [ntiles][KT][64] x 16 B
+  const void* sz;      // [ntiles][G][16] x 4 B
+  const void* act;     // [M][K] T
+  void* out;           // [M][N] T
+  f32x4* partial;      // [ksplit][mblocks][ntiles][MT][64]
+  unsigned* counters;  // [mblocks * ngroups]
   int M, N, K, KT, G, ntiles, ngroups, ksplit;
 };
 
@@ -36,27 +44,27 @@ struct Ops;
 
 template <>
 struct Ops<_Float16> {
-  static constexpr bool kBias = false;
-  // word -> eight fp16 values u - z (exact); zc = z replicated as 0x000z000z
-  static __device__ inline half8 unpack(uint32_t x, uint32_t zc) {
-    const uint32_t c_lo = 0x64006400u | zc;         // 1024 + z
-    const uint32_t c_hi = 0x54005400u | (zc << 4);  // 64 + z
-    uint32_t y = x >> 8;
-    uint32_t v0 = (x & 0x000F000Fu) | 0x64006400u;  // 1024 + u   (elements 0,1)
-    uint32_t v1 = (x & 0x00F000F0u) | 0x54005400u;  // 64 + u     (elements 2,3)
-    uint32_t v2 = (y & 0x000F000Fu) | 0x64006400u;  // elements 4,5
-    uint32_t v3 = (y & 0x00F000F0u) | 0x54005400u;  // elements 6,7
-    half2v r0 = __builtin_bit_cast(half2v, v0) - __builtin_bit_cast(half2v, c_lo);
-    half2v r1 = __builtin_bit_cast(half2v, v1) - __builtin_bit_cast(half2v, c_hi);
-    half2v r2 = __builtin_bit_cast(half2v, v2) - __builtin_bit_cast(half2v, c_lo);
-    half2v r3 = __builtin_bit_cast(half2v, v3) - __builtin_bit_cast(half2v, c_hi);
-    half8 o;
-    o[0] = r0[0]; o[1] = r0[1]; o[2] = r1[0]; o[3] = r1[1];
-    o[4] = r2[0]; o[5] = r2[1]; o[6] = r3[0]; o[7] = r3[1];
-    return o;
+  // word of eight nibbles -> four registers of two biased fp16 each.  Element 2p sits in nibble p and element
+  // 2p + 1 in nibble p + 4; nibbles 0/4 and 2/6 take the 1024 + u form, nibbles 1/5 and 3/7 the 64 + u form.
+  static __device__ inline u32x4 unpack(uint32_t x, uint32_t m_lo, uint32_t m_hi, uint32_t c_lo, uint32_t c_hi) {
+    const uint32_t y = x >> 8;
+    u32x4 v;
+    v[0] = (x & m_lo) | c_lo;
+    v[1] = (x & m_hi) | c_hi;
+    v[2] = (y & m_lo) | c_lo;
+    v[3] = (y & m_hi) | c_hi;
+    return v;
   }
-  static __device__ inline f32x4 mfma(u32x4 a, half8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), b, c, 0, 0, 0);
+  static constexpr uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x00F000F0u;
+  static constexpr uint32_t kMagicLo = 0x64006400u, kMagicHi = 0x54005400u;
+  // -(bias + z) per element for the correction MFMA; zc = z replicated into both halves
+  static __device__ inline u32x4 correction(uint32_t zc) {
+    const uint32_t lo = 0xE400E400u | zc, hi = 0xD400D400u | (zc << 4);
+    return u32x4{lo, hi, lo, hi};
+  }
+  static __device__ inline f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0,
+                                                  0, 0);
   }
   static __device__ inline float scale_to_float(uint32_t szw) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(szw & 0xFFFFu));
@@ -66,63 +74,84 @@ struct Ops<_Float16> {
 
 template <>
 struct Ops<__bf16> {
-  static constexpr bool kBias = true;
-  typedef bf16x8 frag;
-  // word -> eight bf16 values 128 + u (exact)
-  static __device__ inline bf16x8 unpack(uint32_t x, uint32_t) {
+  // bf16 has 7 mantissa bits: only nibbles at bits 0-3 of a half can be or-ed in, as 128 + u
+  static __device__ inline u32x4 unpack(uint32_t x, uint32_t m_lo, uint32_t, uint32_t c_lo, uint32_t) {
     u32x4 v;
-    v[0] = (x & 0x000F000Fu) | 0x43004300u;
-    v[1] = ((x >> 4) & 0x000F000Fu) | 0x43004300u;
-    v[2] = ((x >> 8) & 0x000F000Fu) | 0x43004300u;
-    v[3] = ((x >> 12) & 0x000F000Fu) | 0x43004300u;
-    return __builtin_bit_cast(bf16x8, v);
+    v[0] = (x & m_lo) | c_lo;
+    v[1] = ((x >> 4) & m_lo) | c_lo;
+    v[2] = ((x >> 8) & m_lo) | c_lo;
+    v[3] = ((x >> 12) & m_lo) | c_lo;
+    return v;
   }
-  static __device__ inline f32x4 mfma(u32x4 a, bf16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), b, c, 0, 0, 0);
+  static constexpr uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x000F000Fu;
+  static constexpr uint32_t kMagicLo = 0x43004300u, kMagicHi = 0x43004300u;
+  static __device__ inline u32x4 correction(uint32_t zc) {
+    const uint32_t v = 0xC300C300u | zc;
+    return u32x4{v, v, v, v};
   }
-  static __device__ inline bf16x8 ones() {
-    u32x4 v = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    return __builtin_bit_cast(bf16x8, v);
+  static __device__ inline f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
   }
   static __device__ inline float scale_to_float(uint32_t szw) { return __builtin_bit_cast(float, szw << 16); }
   static __device__ inline uint16_t to_bits(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
 };
 
-template <typename T, int MT, int NT, int GPT, int D>
-__global__ __launch_bounds__(256) void w4a16_stream_kernel(StreamArgs p) {
+template <typename T, int MT, int NT, int GPT, int D, int KCT, int KS>
+__global__ __launch_bounds__(256 * KS) __attribute__((amdgpu_waves_per_eu(KS >= 4 ? 4 : 2))) void
+w4a16_stream_kernel(StreamArgs p) {
   using O = Ops<T>;
-  constexpr int DPG = 4 / GPT;  // MFMAs (32-k steps) per quantisation group inside one tile
+  static_assert(D % KCT == 0 && ((D / KCT) % 2) == 0, "a ring round must span an even number of LDS chunks");
+  constexpr int DPG = 4 / GPT;                       // MFMAs (32-k steps) per quantisation group inside one tile
+  constexpr int kBuf = MT * KCT * 4 * 64;            // 16-byte elements per LDS buffer
+  constexpr int kRed = (KS - 1) * 4 * MT * NT * 64;  // 16-byte elements of the slice reduction
+  constexpr int kLds = KS * 2 * kBuf > kRed ? KS * 2 * kBuf : kRed;
+  __shared__ u32x4 lds_a[kLds];
+
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, kept in a scalar register
+  const int wcol = wave & 3, slice = wave >> 2;
   const int c = lane & 15, j = lane >> 4;
-  const int grp = blockIdx.x * 4 + wave;  // column-tile group of this wave
-  if (grp >= p.ngroups) return;           // wave-uniform; the kernel has no block-level barrier
+  const int grp = blockIdx.x * 4 + wcol;  // column-tile group of this wave
   const int nt0 = grp * NT;
   const int split = blockIdx.y, mblock = blockIdx.z;
-  const int kt_begin = (int)(((long)p.KT * split) / p.ksplit);
-  const int kt_end = (int)(((long)p.KT * (split + 1)) / p.ksplit);
+  // k range of the workgroup, then of this wave's slice; every slice runs the same number of ring rounds
+  const int wg_begin = (int)(((long)p.KT * split) / p.ksplit);
+  const int wg_end = (int)(((long)p.KT * (split + 1)) / p.ksplit);
+  const int wg_tiles = wg_end - wg_begin;
+  const int kt_begin = wg_begin + (wg_tiles * slice) / KS;
+  const int kt_end = wg_begin + (wg_tiles * (slice + 1)) / KS;
+  const int ntile = kt_end - kt_begin;
+  const int rounds = ((wg_tiles + KS - 1) / KS + D - 1) / D;
   const int m0 = mblock * (16 * MT);
 
-  // per-lane base pointers
-  const uint16_t* act = static_cast<const uint16_t*>(p.act);
-  const uint16_t* arow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int row = m0 + 16 * mt + c;
-    row = row < p.M ? row : p.M - 1;  // padding rows re-read the last row; their results are never stored
-    arow[mt] = act + (size_t)row * p.K + 8 * j;
-  }
-  const u32x4* wbase[NT];
-  const uint32_t* szbase[NT];
+  __amdgpu_buffer_rsrc_t rs_w[NT], rs_sz[NT];
   bool tile_ok[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    int nt = nt0 + t;
+    const int nt = nt0 + t;
     tile_ok[t] = nt < p.ntiles;
-    nt = tile_ok[t] ? nt : p.ntiles - 1;
-    wbase[t] = p.weight + (size_t)nt * p.KT * 64 + lane;
-    szbase[t] = p.sz + (size_t)nt * p.G * 16 + c;
+    const size_t ntc = tile_ok[t] ? (size_t)nt : 0;
+    const char* wb = static_cast<const char*>(p.weight) + (ntc * p.KT + kt_begin) * 1024;
+    const char* sb = static_cast<const char*>(p.sz) + (ntc * p.G + (size_t)kt_begin * GPT) * 64;
+    rs_w[t] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(wb), 0, tile_ok[t] ? ntile * 1024 : 0, 0x00020000);
+    rs_sz[t] =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(sb), 0, tile_ok[t] ? ntile * GPT * 64 : 0, 0x00020000);
   }
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
+  // staging role of this thread inside its slice: fragment (MFMA index d = wcol, lane) of every tile of a chunk.
+  // Padding rows sit at an offset that stays out of range for every k (k * 2 < 2^31); tiles past the k range read
+  // real activations of the neighbouring range (or zeros past the end of the tensor), which meet zero weights and
+  // a zero scale.
+  unsigned a_off[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int row = m0 + 16 * mt + c;
+    a_off[mt] = row < p.M ? ((unsigned)row * p.K + kt_begin * kTileK + 32 * wcol + 8 * j) * 2u : 0x80000000u;
+  }
+  const unsigned w_voff = lane * 16u, sz_voff = c * 4u;
+  u32x4* const lds_s = lds_a + slice * (2 * kBuf);  // this slice's two activation buffers
 
   f32x4 acc[MT][NT];
 #pragma unroll
@@ -130,118 +159,130 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(StreamArgs p) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // register ring of D k-tiles: weights, scale/zero words and activation fragments are fetched D tiles ahead
   u32x4 wq[D][NT];
   uint32_t szq[D][NT][GPT];
-  u32x4 aq[D][MT][4];
+  u32x4 a_stage[2][MT][KCT];  // two chunks in flight: a chunk is fetched a full ring round before it is committed
 
-  auto fetch = [&](int slot, int kt) {
+  auto fetch = [&](int slot, int tile) {  // tile = index inside this wave's k range
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      wq[slot][t] = __builtin_nontemporal_load(wbase[t] + (size_t)kt * 64);
+      wq[slot][t] =
+          __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[t], w_voff + tile * 1024u, 0, 2));
 #pragma unroll
-      for (int gi = 0; gi < GPT; ++gi) szq[slot][t][gi] = szbase[t][(size_t)(kt * GPT + gi) * 16];
+      for (int gi = 0; gi < GPT; ++gi)
+        szq[slot][t][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[t], sz_voff + (tile * GPT + gi) * 64u, 0, 0);
     }
+  };
+  auto stage_a = [&](int set, int chunk) {  // global -> registers
+#pragma unroll
+    for (int i = 0; i < KCT; ++i) {
+      const unsigned tile = (unsigned)(chunk * KCT + i);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        a_stage[set][mt][i] =
+            __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, a_off[mt] + tile * 256u, 0, 0));
+    }
+  };
+  auto commit_a = [&](int set, int buf) {  // registers -> LDS, fragment order: [mt][tile][d][lane]
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int d = 0; d < 4; ++d)
-        aq[slot][mt][d] = *reinterpret_cast<const u32x4*>(arow[mt] + (size_t)kt * kTileK + 32 * d);
+      for (int i = 0; i < KCT; ++i)
+        lds_s[buf * kBuf + ((mt * KCT + i) * 4 + wcol) * 64 + lane] = a_stage[set][mt][i];
   };
 
-  auto consume = [&](int slot) {
-    f32x4 R[MT][GPT];
-    if constexpr (O::kBias) {
+  // constants of the unpack kept in registers so that each output register costs one v_and_or_b32
+  uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
+  asm volatile("" : "+s"(m_lo));
+  asm volatile("" : "+v"(c_lo));
+  asm volatile("" : "+v"(c_hi));
+  asm volatile("" : "+v"(m_hi));
+
+  auto consume = [&](int slot, int buf, int il) {
+    u32x4 af[MT][4];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int gi = 0; gi < GPT; ++gi) {
-          f32x4 r = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int dd = 0; dd < DPG; ++dd) r = O::mfma(aq[slot][mt][gi * DPG + dd], Ops<__bf16>::ones(), r);
-          R[mt][gi] = r;
-        }
-    }
+      for (int d = 0; d < 4; ++d) af[mt][d] = lds_s[buf * kBuf + ((mt * KCT + il) * 4 + d) * 64 + lane];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
       for (int gi = 0; gi < GPT; ++gi) {
         const uint32_t szw = szq[slot][t][gi];
         const uint32_t z = szw >> 16;
-        const uint32_t zc = z | (z << 16);
+        const u32x4 corr = O::correction(z | (z << 16));
         const float s = O::scale_to_float(szw);
         f32x4 P[MT];
 #pragma unroll
         for (int dd = 0; dd < DPG; ++dd) {
           const int d = gi * DPG + dd;
-          auto b = O::unpack(wq[slot][t][d], zc);
+          const u32x4 b = O::unpack(wq[slot][t][d], m_lo, m_hi, c_lo, c_hi);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            P[mt] = O::mfma(aq[slot][mt][d], b, dd == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : P[mt]);
+          for (int mt = 0; mt < MT; ++mt) {
+            P[mt] = O::mfma(af[mt][d], corr, dd == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : P[mt]);
+            P[mt] = O::mfma(af[mt][d], b, P[mt]);
+          }
         }
-        if constexpr (O::kBias) {
-          const float cz = -(128.0f + (float)z);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[mt][t][i] += s * (cz * R[mt][gi][i] + P[mt][i]);
-        } else {
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[mt][t][i] += s * P[mt][i];
-        }
+          for (int i = 0; i < 4; ++i) acc[mt][t][i] += s * P[mt][i];
       }
     }
   };
 
-  // Software pipeline.  The hardware retires loads in order and the compiler can only keep later prefetches in
-  // flight across a wait when the number of loads issued after it is known statically, so every stage below is
-  // straight-line code: a steady-state loop whose D fetches are all unconditional, and a tail specialised at
-  // compile time on the remainder.
-  const int ntile = kt_end - kt_begin;
-  auto tail = [&](auto rc, int kt) {  // D tiles in flight in slots 0..D-1, R more to fetch from kt + D
-    constexpr int R = decltype(rc)::value;
+  // ---- pipeline: every wave of the workgroup runs the same number of rounds (uniform barriers)
+  stage_a(0, 0);
+  stage_a(1, 1);
+  __builtin_amdgcn_sched_barrier(0);  // issue order = consumption order: loads retire in order
+#pragma unroll
+  for (int i = 0; i < D; ++i) {
+    fetch(i, i);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  commit_a(0, 0);
+  stage_a(0, 2);
+  __syncthreads();
+  __builtin_amdgcn_sched_barrier(0);
+  for (int r = 0; r < rounds; ++r) {
 #pragma unroll
     for (int i = 0; i < D; ++i) {
-      consume(i);
-      if (i < R) fetch(i, kt + D + i);  // i and R are constants after unrolling
-    }
-#pragma unroll
-    for (int i = 0; i < R; ++i) consume(i);
-  };
-  auto small = [&](auto nc) {  // fewer than D tiles in total
-    constexpr int NS = decltype(nc)::value;
-#pragma unroll
-    for (int i = 0; i < NS; ++i) fetch(i, kt_begin + i);
-#pragma unroll
-    for (int i = 0; i < NS; ++i) consume(i);
-  };
-  if (ntile >= D) {
-#pragma unroll
-    for (int i = 0; i < D; ++i) fetch(i, kt_begin + i);
-    int kt = kt_begin;
-    for (int rounds = ntile / D; rounds >= 2; --rounds, kt += D) {
-#pragma unroll
-      for (int i = 0; i < D; ++i) {
-        consume(i);
-        fetch(i, kt + D + i);
+      const int buf = (i / KCT) & 1;  // D / KCT is even, so the chunk parity is static inside a round
+      const int il = i % KCT;
+      consume(i, buf, il);
+      fetch(i, r * D + i + D);
+      __builtin_amdgcn_sched_barrier(0);  // keep one tile's registers live at a time
+      if (il == KCT - 1) {
+        const int chunk = r * (D / KCT) + i / KCT;  // chunk just finished; its parity is that of buf
+        commit_a(buf ^ 1, buf ^ 1);                 // chunk + 1, fetched a ring round ago
+        stage_a(buf ^ 1, chunk + 3);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    switch (ntile % D) {
-      case 0: tail(std::integral_constant<int, 0>{}, kt); break;
-      case 1: tail(std::integral_constant<int, (1 < D ? 1 : 0)>{}, kt); break;
-      case 2: tail(std::integral_constant<int, (2 < D ? 2 : 0)>{}, kt); break;
-      default: tail(std::integral_constant<int, (3 < D ? 3 : 0)>{}, kt); break;
-    }
-  } else {
-    switch (ntile) {
-      case 0: break;
-      case 1: small(std::integral_constant<int, 1>{}); break;
-      case 2: small(std::integral_constant<int, (2 < D ? 2 : 1)>{}); break;
-      default: small(std::integral_constant<int, (3 < D ? 3 : 1)>{}); break;
-    }
   }
+
+  // ---- reduce the k slices of the workgroup through LDS (the activation buffers are free now)
+  if constexpr (KS > 1) {
+    f32x4* red = reinterpret_cast<f32x4*>(lds_a);
+    if (slice > 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          red[((((slice - 1) * 4 + wcol) * MT + mt) * NT + t) * 64 + lane] = acc[mt][t];
+    }
+    __syncthreads();
+    if (slice > 0) return;
+#pragma unroll
+    for (int sl = 1; sl < KS; ++sl)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[mt][t] += red[((((sl - 1) * 4 + wcol) * MT + mt) * NT + t) * 64 + lane];
+  }
+
+  if (grp >= p.ngroups) return;  // no barrier below this line
 
   // ---- epilogue: lane (c, j) holds column 16*nt + c, rows m0 + 16*mt + 4*j + i
   uint16_t* out = static_cast<uint16_t*>(p.out);
@@ -263,8 +304,8 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(StreamArgs p) {
     return;
   }
 
-  // split-K fix-up: every split parks its fp32 tiles, the last one to arrive adds them in split order
-  // (deterministic) and writes the result.  Counters return to zero for the next launch.
+  // split-K fix-up across workgroups: every split parks its fp32 tiles, the last one to arrive adds them in split
+  // order (deterministic) and writes the result.  Counters return to zero for the next launch.
   const size_t split_stride = (size_t)gridDim.z * p.ntiles * MT * 64;
   auto pidx = [&](int sp, int mt, int t) {
     int nt = nt0 + t;
@@ -275,64 +316,85 @@ __global__ __launch_bounds__(256) void w4a16_stream_kernel(StreamArgs p) {
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < NT; ++t)
-      if (tile_ok[t]) p.partial[pidx(split, mt, t)] = acc[mt][t];
-  __threadfence();
+      if (tile_ok[t]) store_agent(p.partial + pidx(split, mt, t), acc[mt][t]);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores are acknowledged
   unsigned* ctr = p.counters + (size_t)mblock * p.ngroups + grp;
   unsigned arrived = 0;
-  if (lane == 0) arrived = atomicAdd(ctr, 1u);
+  if (lane == 0) arrived = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   arrived = __builtin_amdgcn_readfirstlane(arrived);
   if (arrived != (unsigned)(p.ksplit - 1)) return;
-  __threadfence();
+  asm volatile("" ::: "memory");
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if (!tile_ok[t]) continue;
       f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-      for (int sp = 0; sp < p.ksplit; ++sp) {
-        f32x4 v = p.partial[pidx(sp, mt, t)];
-        sum += v;
-      }
+      for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + pidx(sp, mt, t));
       store_out(mt, t, sum);
     }
-  if (lane == 0) atomicExch(ctr, 0u);
+  if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T, int MT, int NT, int GPT, int KS>
+void launch_ks(const StreamArgs& a, dim3 grid, hipStream_t s) {
+  constexpr int D = (NT == 4 || MT >= 3) ? 4 : 8;
+  constexpr int KCT = (KS >= 2 || MT >= 3 || NT == 4) ? 2 : 4;
+  hipLaunchKernelGGL((w4a16_stream_kernel<T, MT, NT, GPT, D, KCT, KS>), grid, dim3(256 * KS), 0, s, a);
 }
 
 template <typename T, int MT, int NT, int GPT>
-void launch_one(const StreamArgs& a, dim3 grid, hipStream_t s) {
-  constexpr int D = MT == 1 ? 4 : (MT == 2 ? 3 : 2);
-  hipLaunchKernelGGL((w4a16_stream_kernel<T, MT, NT, GPT, D>), grid, dim3(256), 0, s, a);
+void launch_one(int ks, const StreamArgs& a, dim3 grid, hipStream_t s) {
+  if constexpr (MT == 1 && NT == 1) {
+    if (ks == 4) return launch_ks<T, MT, NT, GPT, 4>(a, grid, s);
+  }
+  if constexpr (MT <= 2 && NT <= 2) {
+    if (ks >= 2) return launch_ks<T, MT, NT, GPT, 2>(a, grid, s);
+  }
+  launch_ks<T, MT, NT, GPT, 1>(a, grid, s);
 }
 
 template <typename T, int MT, int NT>
-void launch_gpt(int gpt, const StreamArgs& a, dim3 grid, hipStream_t s) {
-  if (gpt == 1) launch_one<T, MT, NT, 1>(a, grid, s);
-  else launch_one<T, MT, NT, 2>(a, grid, s);
+void launch_gpt(int gpt, int ks, const StreamArgs& a, dim3 grid, hipStream_t s) {
+  if (gpt == 1) launch_one<T, MT, NT, 1>(ks, a, grid, s);
+  else launch_one<T, MT, NT, 2>(ks, a, grid, s);
 }
 
 template <typename T, int MT>
-void launch_nt(int nt, int gpt, const StreamArgs& a, dim3 grid, hipStream_t s) {
-  if (nt == 1) launch_gpt<T, MT, 1>(gpt, a, grid, s);
-  else launch_gpt<T, MT, 2>(gpt, a, grid, s);
+void launch_nt(int nt, int gpt, int ks, const StreamArgs& a, dim3 grid, hipStream_t s) {
+  if (nt == 1) launch_gpt<T, MT, 1>(gpt, ks, a, grid, s);
+  else if (nt == 2) launch_gpt<T, MT, 2>(gpt, ks, a, grid, s);
+  else launch_gpt<T, MT, 4>(gpt, ks, a, grid, s);
 }
 
 template <typename T>
-void launch_mt(int mt, int nt, int gpt, const StreamArgs& a, dim3 grid, hipStream_t s) {
+void launch_mt(int mt, int nt, int gpt, int ks, const StreamArgs& a, dim3 grid, hipStream_t s) {
   switch (mt) {
-    case 1: launch_nt<T, 1>(nt, gpt, a, grid, s); break;
-    case 2: launch_nt<T, 2>(nt, gpt, a, grid, s); break;
-    case 3: launch_nt<T, 3>(nt, gpt, a, grid, s); break;
-    default: launch_nt<T, 4>(nt, gpt, a, grid, s); break;
+    case 1: launch_nt<T, 1>(nt, gpt, ks, a, grid, s); break;
+    case 2: launch_nt<T, 2>(nt, gpt, ks, a, grid, s); break;
+    case 3: launch_nt<T, 3>(nt, gpt, ks, a, grid, s); break;
+    default: launch_nt<T, 4>(nt, gpt, ks, a, grid, s); break;
   }
 }
 
 }  // namespace
 
+// in-workgroup k slices the kernel is instantiated with for a given wave tile
+int w4a16_stream_max_slices(int mt, int nt) {
+  if (mt == 1 && nt == 1) return 4;
+  if (mt <= 2 && nt <= 2) return 2;
+  return 1;
+}
+
 int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
                         const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
+  // activations are addressed with 32-bit range-checked offsets
+  KSQ_REQUIRE(m * k * 2 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED, "activation tensor larger than 2 GiB (m=%zu k=%zu)",
+              m, k);
+  KSQ_REQUIRE(plan.NT == 1 || plan.NT == 2 || plan.NT == 4, KSQ_ERR_INVALID_ARGUMENT, "bad plan");
   StreamArgs a{};
-  a.weight = static_cast<const u32x4*>(weight);
-  a.sz = static_cast<const uint32_t*>(sz);
+  a.weight = weight;
+  a.sz = sz;
   a.act = act;
   a.out = out;
   a.partial = static_cast<f32x4*>(workspace);
@@ -355,8 +417,8 @@ int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* ac
   KSQ_REQUIRE(plan.mblocks <= 65535 && plan.ksplit <= 65535, KSQ_ERR_UNSUPPORTED, "grid too large");
   dim3 grid((unsigned)((a.ngroups + 3) / 4), (unsigned)plan.ksplit, (unsigned)plan.mblocks);
   const int gpt = (int)(kTileK / g);
-  if (dtype == KSQ_F16) launch_mt<_Float16>(plan.MT, plan.NT, gpt, a, grid, s);
-  else launch_mt<__bf16>(plan.MT, plan.NT, gpt, a, grid, s);
+  if (dtype == KSQ_F16) launch_mt<_Float16>(plan.MT, plan.NT, gpt, plan.slices, a, grid, s);
+  else launch_mt<__bf16>(plan.MT, plan.NT, gpt, plan.slices, a, grid, s);
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

@@ -93,20 +93,20 @@ def test_group_sizes_and_kinds(gpu, dtype, kind, g):
 
 
 @pytest.mark.parametrize("ksplit", [1, 2, 3, 5, 8])
-@pytest.mark.parametrize("nt", [1, 2])
-@pytest.mark.parametrize("dtype,M", [("f16", 16), ("bf16", 33)])
-def test_forced_split_k_and_tile_widths(gpu, dtype, M, ksplit, nt):
-    case = W4Case(1200 + ksplit, M, 1024, 272, kind="awq", dtype=dtype)  # 17 column tiles: ragged for nt = 2
+@pytest.mark.parametrize("nt,slices", [(1, 1), (1, 2), (1, 4), (2, 1), (2, 2), (4, 1)])
+@pytest.mark.parametrize("dtype,M", [("f16", 16), ("bf16", 33), ("bf16", 7)])
+def test_forced_split_k_and_tile_widths(gpu, dtype, M, ksplit, nt, slices):
+    case = W4Case(1200 + ksplit, M, 1408, 272, kind="awq", dtype=dtype)  # 11 k tiles, 17 column tiles: ragged
     dev = W4Device(case, gpu)
     import torch
 
     big = torch.empty(64 << 20, dtype=torch.uint8, device=gpu)
     dev.workspace, dev.workspace_bytes = big, big.numel()
-    with _env(KSQ_W4_KSPLIT=ksplit, KSQ_W4_NT=nt):
+    with _env(KSQ_W4_KSPLIT=ksplit, KSQ_W4_NT=nt, KSQ_W4_SLICES=slices):
         got1 = dev.gemm_f32()
         got2 = dev.gemm_f32()  # counters must have returned to zero
     want = case.oracle()
-    orc.assert_parity(got1, want, f"ksplit={ksplit} nt={nt}")
+    orc.assert_parity(got1, want, f"ksplit={ksplit} nt={nt} slices={slices}")
     assert np.array_equal(got1, got2), "split-K result must be deterministic and repeatable"
 
 
