@@ -207,6 +207,8 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     W4Plan p = w4a16_plan(mm, n, k, cus, (size_t)-1);
     if (p.partial_bytes > best) best = p.partial_bytes;
   }
+  KstatPlan kp = w4a16_kstat_plan(1, n, k, cus, (size_t)-1);
+  if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   *bytes = best;
   return KSQ_OK;
 }
@@ -228,6 +230,10 @@ int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, co
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(m, n, k, g))
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, s);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
+  if (m <= 16 && env_int("KSQ_W4_KSTAT", 1) != 0) {
+    KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
+    if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s);
+  }
   W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
   return w4a16_launch_stream(dtype, plan, out, act, weight, sz, m, n, k, g, workspace, s);
 }

@@ -112,6 +112,19 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
 bool w4a16_prefill_supported(size_t m, size_t n, size_t k, size_t g);
 int w4a16_stream_max_slices(int mt, int nt);
 
+struct KstatPlan {
+  bool ok;       // the k-stationary decode kernel takes this shape
+  int tpw;       // k tiles per wave (16 waves per workgroup)
+  int ksplit;    // grid.y
+  int nt_per_wg; // column tiles per workgroup
+  int grid_x;
+  int nb;        // column tiles per batch (= ring depth / tpw)
+  size_t partial_bytes;
+};
+KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
+                       const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+
 struct Fp8Plan {
   int MT;
   int mblocks;

@@ -1,0 +1,259 @@
+// W4A16 decode kernel for M <= 16: k-stationary.
+//
+// A workgroup is 16 waves.  Wave w keeps the activation fragments of its own TPW k tiles in registers for the
+// whole kernel (the activations of a decode step are tiny: 16 x K) and streams the weight tiles (n tile, its k
+// tiles) of the workgroup's column range straight from HBM into a register ring, one batch of NB column tiles
+// ahead.  Nothing is re-read: no activation traffic per weight tile, no LDS on the streaming path.  After every
+// batch the 16 partial tiles of a column tile (one per wave = per k slice) are summed through LDS in a fixed
+// order.  Because k is covered inside the workgroup, narrow N needs no split across workgroups; only K > 48
+// tiles x 16 waves is split over grid.y and finished by the last-arriving workgroup through the workspace.
+//
+// Arithmetic as in the streaming kernel: biased nibbles by bit operations, a correction MFMA with -(bias + z),
+// fp32 group sums scaled by s[g,n].
+#include <cstdlib>
+
+#include "ksq_internal.h"
+#include "ksq_w4a16_ops.h"
+
+namespace ksq {
+namespace {
+
+using namespace w4;
+
+struct KstatArgs {
+  const void* weight;  // [ntiles][KT][64] x 16 B
+  const void* sz;      // [ntiles][G][16] x 4 B
+  const void* act;     // [M][K] T
+  void* out;           // [M][N] T
+  f32x4* partial;      // [ksplit][ntiles][64]
+  unsigned* counters;  // [ntiles]
+  int M, N, K, KT, G, ntiles, ksplit, nt_per_wg;
+};
+
+template <typename T, int GPT, int TPW, int NB>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void w4a16_kstat_kernel(KstatArgs p) {
+  using O = Ops<T>;
+  constexpr int DPG = 4 / GPT;
+  constexpr int D = NB * TPW;  // ring depth = one batch
+  __shared__ f32x4 red[NB * 16 * 64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, j = lane >> 4;
+  const int split = blockIdx.y;
+  const int wg_begin = (int)(((long)p.KT * split) / p.ksplit);
+  const int wg_end = (int)(((long)p.KT * (split + 1)) / p.ksplit);
+  const int kt0 = wg_begin + wave * TPW;  // first k tile of this wave
+  const int nt_begin = blockIdx.x * p.nt_per_wg;
+  int count = p.ntiles - nt_begin;
+  count = count < p.nt_per_wg ? count : p.nt_per_wg;
+  const int nbatches = (p.nt_per_wg + NB - 1) / NB;  // same for every workgroup
+
+  // Resources start at (nt_begin, kt0) and end with the wave's tiles of the last column tile of the workgroup, so
+  // column tiles past the range read as zero; k tiles past the end of the split are parked at an offset that stays
+  // out of range for every column tile (the range is far below 2^31 bytes).
+  const size_t kt0c = kt0 < p.KT ? (size_t)kt0 : (size_t)p.KT - 1;
+  const char* wb = static_cast<const char*>(p.weight) + ((size_t)nt_begin * p.KT + kt0c) * 1024;
+  const char* sb = static_cast<const char*>(p.sz) + ((size_t)nt_begin * p.G + kt0c * GPT) * 64;
+  const bool any = count > 0 && kt0 < wg_end;
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(wb), 0, any ? ((count - 1) * p.KT + TPW) * 1024 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_sz = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(sb), 0, any ? ((count - 1) * p.G + TPW * GPT) * 64 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
+  unsigned w_off[TPW], sz_off[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) {
+    const bool ok = kt0 + t < wg_end;
+    w_off[t] = ok ? t * 1024u + lane * 16u : 0x80000000u;
+    sz_off[t] = ok ? t * GPT * 64u + c * 4u : 0x80000000u;
+  }
+  const unsigned w_stride = (unsigned)p.KT * 1024u, sz_stride = (unsigned)p.G * 64u;
+
+  // activation fragments of this wave's k tiles: registers for the whole kernel
+  u32x4 af[TPW][4];
+#pragma unroll
+  for (int t = 0; t < TPW; ++t)
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const bool ok = c < p.M && kt0 + t < wg_end;
+      const unsigned ao = ok ? ((unsigned)c * p.K + (kt0 + t) * kTileK + 32 * d + 8 * j) * 2u : 0x80000000u;
+      af[t][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+    }
+
+  u32x4 wq[D];
+  uint32_t szq[D][GPT];
+  auto fetch = [&](int slot, int i /* column tile inside the workgroup */, int t) {
+    wq[slot] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_off[t] + i * w_stride, 0, 2));
+#pragma unroll
+    for (int gi = 0; gi < GPT; ++gi)
+      szq[slot][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, sz_off[t] + gi * 64u + i * sz_stride, 0, 0);
+  };
+
+  uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
+  asm volatile("" : "+s"(m_lo));
+  asm volatile("" : "+v"(c_lo));
+  asm volatile("" : "+v"(c_hi));
+  asm volatile("" : "+v"(m_hi));
+
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int q = 0; q < D; ++q) {
+    fetch(q, q / TPW, q % TPW);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  for (int b = 0; b < nbatches; ++b) {
+    f32x4 accb[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      accb[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) {
+        const int slot = i * TPW + t;
+#pragma unroll
+        for (int gi = 0; gi < GPT; ++gi) {
+          const uint32_t szw = szq[slot][gi];
+          const uint32_t z = szw >> 16;
+          const u32x4 corr = O::correction(z | (z << 16));
+          const float s = O::scale_to_float(szw);
+          f32x4 P = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int dd = 0; dd < DPG; ++dd) {
+            const int d = gi * DPG + dd;
+            const u32x4 bw = O::unpack(wq[slot][d], m_lo, m_hi, c_lo, c_hi);
+            P = O::mfma(af[t][d], corr, P);
+            P = O::mfma(af[t][d], bw, P);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) accb[i][e] += s * P[e];
+        }
+        fetch(slot, (b + 1) * NB + i, t);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- sum the 16 k slices of every column tile of the batch (fixed order: deterministic)
+#pragma unroll
+    for (int i = 0; i < NB; ++i) red[(i * 16 + wave) * 64 + lane] = accb[i];
+    __syncthreads();
+    if (wave < NB) {
+      const int nt = nt_begin + b * NB + wave;
+      const bool valid = b * NB + wave < count;
+      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ww = 0; ww < 16; ++ww) sum += red[(wave * 16 + ww) * 64 + lane];
+      bool store = valid;
+      if (p.ksplit > 1 && valid) {
+        // split across workgroups: park the fp32 tile, the last split to arrive adds them in split order
+        const size_t stride = (size_t)p.ntiles * 64;
+        store_agent(p.partial + (size_t)split * stride + (size_t)nt * 64 + lane, sum);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned arrived = 0;
+        if (lane == 0)
+          arrived = __hip_atomic_fetch_add(p.counters + nt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        store = arrived == (unsigned)(p.ksplit - 1);
+        if (store) {
+          asm volatile("" ::: "memory");
+          sum = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + (size_t)sp * stride + (size_t)nt * 64 + lane);
+          if (lane == 0) __hip_atomic_store(p.counters + nt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      if (store) {
+        const int col = nt * 16 + c;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int row = 4 * j + e;
+          if (row < p.M) out[(size_t)row * p.N + col] = O::to_bits(sum[e]);
+        }
+      }
+    }
+    __syncthreads();  // the reduction buffer is reused by the next batch
+  }
+}
+
+template <typename T, int GPT, int TPW>
+void launch_nb(int nb, const KstatArgs& a, dim3 grid, hipStream_t s) {
+  if (nb >= 4) hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, TPW, 4>), grid, dim3(1024), 0, s, a);
+  else if (nb >= 2) hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, TPW, 2>), grid, dim3(1024), 0, s, a);
+  else hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, TPW, 1>), grid, dim3(1024), 0, s, a);
+}
+
+template <typename T, int GPT>
+void launch_tpw(int tpw, int nb, const KstatArgs& a, dim3 grid, hipStream_t s) {
+  if (tpw <= 1) launch_nb<T, GPT, 1>(nb, a, grid, s);
+  else if (tpw == 2) launch_nb<T, GPT, 2>(nb, a, grid, s);
+  else launch_nb<T, GPT, 3>(nb, a, grid, s);
+}
+
+}  // namespace
+
+// Plan of the k-stationary kernel: k tiles per wave (at most 3, i.e. 48 per workgroup), split count, column tiles
+// per workgroup and batch size.
+KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  KstatPlan p{};
+  const size_t ntiles = n / kTileN, ktiles = k / kTileK;
+  p.ok = m >= 1 && m <= 16 && ntiles <= (size_t)kCountersPerSlot;
+  size_t ksplit = (ktiles + 47) / 48;
+  if (const char* e = getenv("KSQ_W4_KSPLIT")) {  // tuning / test override; never below what the registers need
+    const size_t v = (size_t)atoi(e);
+    if (v > ksplit && v <= ktiles) ksplit = v;
+  }
+  if (ksplit > 1 && ksplit * ntiles * 64 * 16 > workspace_bytes) p.ok = false;
+  if (!p.ok) return p;
+  const size_t per_split = (ktiles + ksplit - 1) / ksplit;
+  p.ksplit = (int)ksplit;
+  p.tpw = (int)((per_split + 15) / 16);
+  size_t wgs = (size_t)cus / ksplit;
+  if (wgs < 1) wgs = 1;
+  if (wgs > ntiles) wgs = ntiles;
+  p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
+  p.grid_x = (int)((ntiles + p.nt_per_wg - 1) / p.nt_per_wg);
+  p.nb = p.nt_per_wg >= 3 ? 4 : (p.nt_per_wg >= 2 ? 2 : 1);  // ring depth = nb * tpw tiles in flight per wave
+  if (p.tpw >= 3 && p.nb > 2) p.nb = 2;  // register budget of 16 waves per workgroup
+  p.partial_bytes = ksplit > 1 ? ksplit * ntiles * 64 * 16 : 0;
+  return p;
+}
+
+int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
+                       const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
+  KSQ_REQUIRE(m * k * 2 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED, "activation tensor larger than 2 GiB");
+  KSQ_REQUIRE((size_t)plan.nt_per_wg * (k / kTileK) * 1024 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED,
+              "column range of one workgroup larger than 2 GiB");
+  KstatArgs a{};
+  a.weight = weight;
+  a.sz = sz;
+  a.act = act;
+  a.out = out;
+  a.partial = static_cast<f32x4*>(workspace);
+  a.M = (int)m;
+  a.N = (int)n;
+  a.K = (int)k;
+  a.KT = (int)(k / kTileK);
+  a.G = (int)(k / g);
+  a.ntiles = (int)(n / kTileN);
+  a.ksplit = plan.ksplit;
+  a.nt_per_wg = plan.nt_per_wg;
+  a.counters = nullptr;
+  if (plan.ksplit > 1) {
+    KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
+    a.counters = counter_slot_device_ptr();
+    if (!a.counters) return KSQ_ERR_HIP;
+  }
+  dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
+  const int gpt = (int)(kTileK / g);
+  if (dtype == KSQ_F16) {
+    if (gpt == 1) launch_tpw<_Float16, 1>(plan.tpw, plan.nb, a, grid, s);
+    else launch_tpw<_Float16, 2>(plan.tpw, plan.nb, a, grid, s);
+  } else {
+    if (gpt == 1) launch_tpw<__bf16, 1>(plan.tpw, plan.nb, a, grid, s);
+    else launch_tpw<__bf16, 2>(plan.tpw, plan.nb, a, grid, s);
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+}  // namespace ksq

@@ -20,14 +20,12 @@
 // keeps the pipeline free of branches (the hardware retires loads in order, and the compiler can only leave later
 // prefetches in flight across a wait when the number of loads issued after it is known statically).
 #include "ksq_internal.h"
+#include "ksq_w4a16_ops.h"
 
 namespace ksq {
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+using namespace w4;
 
 struct StreamArgs {
   const void* weight;  // [ntiles][KT][64] x 16 B
@@ -39,70 +37,14 @@ struct StreamArgs {
   int M, N, K, KT, G, ntiles, ngroups, ksplit;
 };
 
-template <typename T>
-struct Ops;
-
-template <>
-struct Ops<_Float16> {
-  // word of eight nibbles -> four registers of two biased fp16 each.  Element 2p sits in nibble p and element
-  // 2p + 1 in nibble p + 4; nibbles 0/4 and 2/6 take the 1024 + u form, nibbles 1/5 and 3/7 the 64 + u form.
-  static __device__ inline u32x4 unpack(uint32_t x, uint32_t m_lo, uint32_t m_hi, uint32_t c_lo, uint32_t c_hi) {
-    const uint32_t y = x >> 8;
-    u32x4 v;
-    v[0] = (x & m_lo) | c_lo;
-    v[1] = (x & m_hi) | c_hi;
-    v[2] = (y & m_lo) | c_lo;
-    v[3] = (y & m_hi) | c_hi;
-    return v;
-  }
-  static constexpr uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x00F000F0u;
-  static constexpr uint32_t kMagicLo = 0x64006400u, kMagicHi = 0x54005400u;
-  // -(bias + z) per element for the correction MFMA; zc = z replicated into both halves
-  static __device__ inline u32x4 correction(uint32_t zc) {
-    const uint32_t lo = 0xE400E400u | zc, hi = 0xD400D400u | (zc << 4);
-    return u32x4{lo, hi, lo, hi};
-  }
-  static __device__ inline f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0,
-                                                  0, 0);
-  }
-  static __device__ inline float scale_to_float(uint32_t szw) {
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)(szw & 0xFFFFu));
-  }
-  static __device__ inline uint16_t to_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
-};
-
-template <>
-struct Ops<__bf16> {
-  // bf16 has 7 mantissa bits: only nibbles at bits 0-3 of a half can be or-ed in, as 128 + u
-  static __device__ inline u32x4 unpack(uint32_t x, uint32_t m_lo, uint32_t, uint32_t c_lo, uint32_t) {
-    u32x4 v;
-    v[0] = (x & m_lo) | c_lo;
-    v[1] = ((x >> 4) & m_lo) | c_lo;
-    v[2] = ((x >> 8) & m_lo) | c_lo;
-    v[3] = ((x >> 12) & m_lo) | c_lo;
-    return v;
-  }
-  static constexpr uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x000F000Fu;
-  static constexpr uint32_t kMagicLo = 0x43004300u, kMagicHi = 0x43004300u;
-  static __device__ inline u32x4 correction(uint32_t zc) {
-    const uint32_t v = 0xC300C300u | zc;
-    return u32x4{v, v, v, v};
-  }
-  static __device__ inline f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
-  }
-  static __device__ inline float scale_to_float(uint32_t szw) { return __builtin_bit_cast(float, szw << 16); }
-  static __device__ inline uint16_t to_bits(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
-};
-
 template <typename T, int MT, int NT, int GPT, int D, int KCT, int KS>
-__global__ __launch_bounds__(256 * KS) __attribute__((amdgpu_waves_per_eu(KS >= 4 ? 4 : 2))) void
+__global__ __launch_bounds__(256 * KS)
+    __attribute__((amdgpu_waves_per_eu(KS >= 4 ? 4 : (MT * NT >= 4 ? 1 : 2)))) void
 w4a16_stream_kernel(StreamArgs p) {
   using O = Ops<T>;
   static_assert(D % KCT == 0 && ((D / KCT) % 2) == 0, "a ring round must span an even number of LDS chunks");
   constexpr int DPG = 4 / GPT;                       // MFMAs (32-k steps) per quantisation group inside one tile
+  constexpr int NACC = (MT * NT <= 2 && DPG >= 2) ? 2 : 1;  // accumulators one group sum is spread over
   constexpr int kBuf = MT * KCT * 4 * 64;            // 16-byte elements per LDS buffer
   constexpr int kRed = (KS - 1) * 4 * MT * NT * 64;  // 16-byte elements of the slice reduction
   constexpr int kLds = KS * 2 * kBuf > kRed ? KS * 2 * kBuf : kRed;
@@ -198,12 +140,47 @@ w4a16_stream_kernel(StreamArgs p) {
   asm volatile("" : "+v"(c_hi));
   asm volatile("" : "+v"(m_hi));
 
-  auto consume = [&](int slot, int buf, int il) {
-    u32x4 af[MT][4];
+  // Software pipeline inside the wave.  A step issues the MFMAs of tile i from activation fragments that were
+  // read from LDS at the end of step i - 1, and only then folds the group sums of tile i - 1 into the
+  // accumulators, so neither the LDS latency nor the matrix-core latency is waited for.  Each group sum is kept in
+  // two accumulators (alternating 32-k steps) to halve the dependent MFMA chain.
+  u32x4 af[MT][4];
+  f32x4 pend[MT][NT][GPT][NACC];
+  float pend_s[NT][GPT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int gi = 0; gi < GPT; ++gi) {
+      pend_s[t][gi] = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int h = 0; h < NACC; ++h) pend[mt][t][gi][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  auto load_frags = [&](int buf, int il) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int d = 0; d < 4; ++d) af[mt][d] = lds_s[buf * kBuf + ((mt * KCT + il) * 4 + d) * 64 + lane];
+  };
+  auto flush = [&]() {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if constexpr (NACC == 2)
+              acc[mt][t][i] += pend_s[t][gi] * (pend[mt][t][gi][0][i] + pend[mt][t][gi][1][i]);
+            else
+              acc[mt][t][i] += pend_s[t][gi] * pend[mt][t][gi][0][i];
+          }
+  };
+  auto consume = [&](int slot) {
+    f32x4 cur[MT][NT][GPT][NACC];
+    float cur_s[NT][GPT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -211,24 +188,32 @@ w4a16_stream_kernel(StreamArgs p) {
         const uint32_t szw = szq[slot][t][gi];
         const uint32_t z = szw >> 16;
         const u32x4 corr = O::correction(z | (z << 16));
-        const float s = O::scale_to_float(szw);
-        f32x4 P[MT];
+        cur_s[t][gi] = O::scale_to_float(szw);
 #pragma unroll
         for (int dd = 0; dd < DPG; ++dd) {
           const int d = gi * DPG + dd;
+          const int h = dd % NACC;
           const u32x4 b = O::unpack(wq[slot][t][d], m_lo, m_hi, c_lo, c_hi);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            P[mt] = O::mfma(af[mt][d], corr, dd == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : P[mt]);
-            P[mt] = O::mfma(af[mt][d], b, P[mt]);
+            f32x4 pacc = dd < NACC ? f32x4{0.f, 0.f, 0.f, 0.f} : cur[mt][t][gi][h];
+            pacc = O::mfma(af[mt][d], corr, pacc);
+            cur[mt][t][gi][h] = O::mfma(af[mt][d], b, pacc);
           }
         }
+      }
+    }
+    flush();  // previous tile, while this tile's MFMAs are in flight
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi) {
+        pend_s[t][gi] = cur_s[t][gi];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[mt][t][i] += s * P[mt][i];
+          for (int h = 0; h < NACC; ++h) pend[mt][t][gi][h] = cur[mt][t][gi][h];
       }
-    }
   };
 
   // ---- pipeline: every wave of the workgroup runs the same number of rounds (uniform barriers)
@@ -243,13 +228,14 @@ w4a16_stream_kernel(StreamArgs p) {
   commit_a(0, 0);
   stage_a(0, 2);
   __syncthreads();
+  load_frags(0, 0);
   __builtin_amdgcn_sched_barrier(0);
   for (int r = 0; r < rounds; ++r) {
 #pragma unroll
     for (int i = 0; i < D; ++i) {
       const int buf = (i / KCT) & 1;  // D / KCT is even, so the chunk parity is static inside a round
       const int il = i % KCT;
-      consume(i, buf, il);
+      consume(i);
       fetch(i, r * D + i + D);
       __builtin_amdgcn_sched_barrier(0);  // keep one tile's registers live at a time
       if (il == KCT - 1) {
@@ -257,10 +243,14 @@ w4a16_stream_kernel(StreamArgs p) {
         commit_a(buf ^ 1, buf ^ 1);                 // chunk + 1, fetched a ring round ago
         stage_a(buf ^ 1, chunk + 3);
         __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
+        load_frags(buf ^ 1, 0);  // first tile of the next chunk
+      } else {
+        load_frags(buf, il + 1);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
+  flush();
 
   // ---- reduce the k slices of the workgroup through LDS (the activation buffers are free now)
   if constexpr (KS > 1) {
