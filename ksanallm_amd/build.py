@@ -53,6 +53,20 @@ def build_library(verbose=False, jobs=5):
     return LIB
 
 
+def build_layer_driver():
+    """Compile the C++ layer shims (host code over the C ABI) and their test driver next to libksq.so."""
+    cc = hipcc()
+    layers = os.path.join(CSRC, "layers")
+    out = os.path.join(HERE, "layer_driver")
+    cmd = [cc, "-std=c++17", "-O2", "-Wall", "-Wno-unused-parameter", "-I" + os.path.join(ROOT, "include"),
+           "-I" + layers, os.path.join(ROOT, "tests", "cpp", "layer_driver.cpp"), os.path.join(layers, "layers.cpp"),
+           "-L" + HERE, "-lksq", "-Wl,-rpath,$ORIGIN", "-o", out]
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("layer driver build failed:\n" + p.stdout)
+    return out
+
+
 def _drain(procs):
     while procs:
         src, p = procs.pop(0)
@@ -66,3 +80,4 @@ def _drain(procs):
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_layer_driver())

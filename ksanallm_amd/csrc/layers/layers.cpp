@@ -1,0 +1,242 @@
+// Implementation of the layer shims over the C ABI (ksq.h).  Error conventions follow the reference: success is
+// Status(); misuse and device errors raise std::runtime_error through KLLM_THROW (KS/utils/logger.h:123), the way
+// KS/layers/nvidia/{group_matmul,fp8_matmul}_layer.cpp and the kernel library do.
+#include <hip/hip_runtime_api.h>
+
+#include <sstream>
+
+#include "fp8_matmul_layer.h"
+#include "group_matmul_layer.h"
+#include "ksq.h"
+#include "matmul_layer_factory.h"
+
+namespace ksana_llm {
+
+namespace {
+
+void ThrowOnKsqError(int code, const char* what) {
+  if (code == KSQ_OK) return;
+  std::ostringstream os;
+  os << what << " failed (" << code << "): " << ksq_last_error_string();
+  KLLM_THROW(os.str());
+}
+
+template <typename T>
+int KsqDtype() {
+  return TypeTraits<T>::kDataType == TYPE_FP16 ? KSQ_F16 : KSQ_BF16;
+}
+
+constexpr size_t kFp8GemmWorkspaceBytes = 32ull << 20;  // the reference reserves 32 MiB for cuBLASLt here
+
+}  // namespace
+
+Status CreateTensor(Tensor& tensor, const std::vector<size_t>& shape, DataType dtype, int rank, MemoryDevice device) {
+  (void)rank;
+  tensor.device = device;
+  tensor.dtype = dtype;
+  tensor.shape = shape;
+  const size_t bytes = tensor.GetTotalBytes();
+  void* ptr = nullptr;
+  if (bytes > 0) {
+    hipError_t e = device == MEMORY_DEVICE ? hipMalloc(&ptr, bytes) : hipHostMalloc(&ptr, bytes, 0);
+    if (e != hipSuccess) KLLM_THROW(std::string("CreateTensor: ") + hipGetErrorString(e));
+  }
+  tensor.refer_ptr = ptr;
+  return Status();
+}
+
+Status DestroyTensor(Tensor& tensor, int rank) {
+  (void)rank;
+  if (tensor.refer_ptr) {
+    if (tensor.device == MEMORY_DEVICE) (void)hipFree(tensor.refer_ptr);
+    else (void)hipHostFree(tensor.refer_ptr);
+  }
+  tensor.refer_ptr = nullptr;
+  return Status();
+}
+
+// ---------------------------------------------------------------------------------------------- GroupMatMulLayer
+template <typename T, DataType WT>
+Status GroupMatMulLayer<T, WT>::Init(const std::vector<std::any>& parameters, std::shared_ptr<Context> context,
+                                     int rank) {
+  context_ = context;
+  rank_ = rank;
+
+  int parameter_index = 0;
+  is_awq_ = std::any_cast<const bool>(parameters[parameter_index++]);
+  is_gptq_desc_ = std::any_cast<const bool>(parameters[parameter_index++]);
+  is_k_full_ = std::any_cast<const bool>(parameters[parameter_index++]);
+  backend_ = std::any_cast<const GroupQuantBackend>(parameters[parameter_index++]);
+  max_m_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  max_n_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  max_k_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  groupsize_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  cutlass_use_gemv_cuda_core_ = std::any_cast<const bool>(parameters[parameter_index++]);
+
+  is_k_full_ = is_gptq_desc_ ? is_k_full_ : true;
+  return Status();
+}
+
+template <typename T, DataType WT>
+size_t GroupMatMulLayer<T, WT>::GetWorkSpaceSize() {
+  if constexpr (WT == TYPE_I4_GROUP) {
+    size_t bytes = 0;
+    ThrowOnKsqError(ksq_w4a16_workspace_bytes(max_m_, max_n_, max_k_, &bytes), "ksq_w4a16_workspace_bytes");
+    return bytes;
+  } else {
+    KLLM_THROW("Not supported weight data type. GroupMatMul only supports TYPE_I4_GROUP.");
+  }
+}
+
+template <typename T, DataType WT>
+Status GroupMatMulLayer<T, WT>::Preprocess(const ModelConfig& model_config_) {
+  (void)model_config_;
+  if constexpr (WT != TYPE_I4_GROUP) {
+    KLLM_THROW("Not supported weight data type. GroupMatMul only supports TYPE_I4_GROUP.");
+  }
+  return Status();
+}
+
+template <typename T, DataType WT>
+Status GroupMatMulLayer<T, WT>::Forward(const std::vector<Tensor>& input_tensors,
+                                        std::vector<Tensor>& output_tensors) {
+  if constexpr (WT == TYPE_I4_GROUP) {
+    if (is_gptq_desc_) {
+      // the reference serves desc_act through its Marlin backend only (KS/utils/environment.cpp:105-106)
+      KLLM_THROW("GroupMatMulLayer: desc_act (g_idx / perm) weights are not supported by this backend.");
+    }
+    const Tensor& weight_tensor = input_tensors[1];
+    if (weight_tensor.scales == nullptr) {
+      KLLM_THROW("GroupMatMulLayer: weight tensor has no scales bound.");
+    }
+    void* p_qweight_tensor = weight_tensor.GetPtr<void>();
+    void* p_sz_tensor = weight_tensor.scales->GetPtr<void>();
+
+    const size_t m = input_tensors[0].shape[0];
+    const size_t n = max_n_;
+    const size_t k = max_k_;
+
+    void* ws = workspace_buffer_ ? workspace_buffer_->GetPtr<void>() : nullptr;
+    const size_t ws_bytes = workspace_buffer_ ? workspace_buffer_->GetTotalBytes() : 0;
+    ThrowOnKsqError(ksq_w4a16_gemm(KsqDtype<T>(), output_tensors[0].GetPtr<void>(), input_tensors[0].GetPtr<void>(),
+                                   p_qweight_tensor, p_sz_tensor, m, n, k, groupsize_, ws, ws_bytes,
+                                   context_->GetComputeStreams()[rank_].Get()),
+                    "ksq_w4a16_gemm");
+
+    output_tensors[0].shape = {m, n};
+    output_tensors[0].dtype = input_tensors[0].dtype;
+    return Status();
+  } else {
+    KLLM_THROW("Not supported weight data type. GroupMatMul only supports TYPE_I4_GROUP.");
+  }
+}
+
+template class GroupMatMulLayer<float16, TYPE_I4_GROUP>;
+template class GroupMatMulLayer<bfloat16, TYPE_I4_GROUP>;
+
+Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, const Tensor* qzeros,
+                              bool zeros_additive, const Tensor& scales, size_t k, size_t n, size_t groupsize,
+                              Tensor& weight, Tensor& weight_sz, int rank, Stream& stream) {
+  size_t weight_bytes = 0, sz_bytes = 0;
+  ThrowOnKsqError(ksq_w4a16_repack_sizes(k, n, groupsize, &weight_bytes, &sz_bytes), "ksq_w4a16_repack_sizes");
+  if (scales.dtype != TYPE_FP16 && scales.dtype != TYPE_BF16) KLLM_THROW("RepackGroupQuantWeight: scales must be fp16 or bf16.");
+  CreateTensor(weight, {k, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);  // same shape as ksana's "*.weight"
+  CreateTensor(weight_sz, {k / groupsize, n}, TYPE_UINT32, rank, MEMORY_DEVICE);
+  int src = layout == GROUP_WEIGHT_GPTQ_INT32 ? KSQ_W4_GPTQ_INT32_KPACK
+            : layout == GROUP_WEIGHT_AWQ_INT32 ? KSQ_W4_AWQ_INT32_NPACK
+                                               : KSQ_W4_ROWMAJOR_INT4_SIGNED;
+  int zero_kind = KSQ_ZERO_NONE;
+  if (qzeros != nullptr) {
+    if (zeros_additive) zero_kind = KSQ_ZERO_ADDITIVE;
+    else if (qzeros->dtype == TYPE_INT32 || qzeros->dtype == TYPE_UINT32) zero_kind = KSQ_ZERO_AWQ_INT32;
+    else zero_kind = KSQ_ZERO_UINT8;
+  }
+  ThrowOnKsqError(
+      ksq_w4a16_repack(src, qweight.GetPtr<void>(), zero_kind, qzeros ? qzeros->GetPtr<void>() : nullptr,
+                       scales.GetPtr<void>(), scales.dtype == TYPE_FP16 ? KSQ_F16 : KSQ_BF16, k, n, groupsize,
+                       weight.GetPtr<void>(), weight_sz.GetPtr<void>(), stream.Get()),
+      "ksq_w4a16_repack");
+  weight.dtype = TYPE_I4_GROUP;
+  weight.scales = &weight_sz;
+  return Status();
+}
+
+// ------------------------------------------------------------------------------------------------ Fp8MatMulLayer
+template <typename T>
+Status Fp8MatMulLayer<T>::Init(const std::vector<std::any>& parameters, std::shared_ptr<Context> context, int rank) {
+  STATUS_CHECK_FAILURE(BaseLayer::Init(parameters, context, rank));
+  int parameter_index = 0;
+  max_m_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  max_k_ = std::any_cast<const size_t>(parameters[parameter_index++]);
+  return Status();
+}
+
+template <typename T>
+size_t Fp8MatMulLayer<T>::GetWorkSpaceSize(const int m, const int k) {
+  // [ GEMM split-K workspace | m*k e4m3 activations | m float scales ]; the reference's layout with one scale
+  // slot per token instead of one in total (KS/layers/nvidia/fp8_matmul_layer.cpp:22-28, 45-46, 60)
+  size_t input_size = (size_t)m * k * GetTypeSize(TYPE_FP8_E4M3);
+  input_size = (input_size + 15) / 16 * 16;
+  size_t scale_size = (size_t)m * GetTypeSize(TYPE_FP32);
+  return input_size + scale_size + kFp8GemmWorkspaceBytes;
+}
+
+template <typename T>
+size_t Fp8MatMulLayer<T>::GetWorkSpaceSize() {
+  return GetWorkSpaceSize(max_m_, max_k_);
+}
+
+template <typename T>
+Status Fp8MatMulLayer<T>::Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) {
+  int m = input_tensors[0].shape[0];
+  int k = input_tensors[0].shape[1];
+  int n = input_tensors[1].shape[0];
+  const void* input = input_tensors[0].GetPtr<const void>();
+  size_t workspace_size = GetWorkSpaceSize(m, k);
+  if (!workspace_buffer_ || workspace_size > workspace_buffer_->GetTotalBytes()) {
+    std::ostringstream os;
+    os << "workspace size " << workspace_size << " > buffer size "
+       << (workspace_buffer_ ? workspace_buffer_->GetTotalBytes() : 0);
+    KLLM_THROW(os.str());
+  }
+  char* gemm_workspace = workspace_buffer_->GetPtr<char>();
+  char* input_quant = gemm_workspace + kFp8GemmWorkspaceBytes;
+  const void* weight_quant = input_tensors[1].GetPtr<const void>();
+  const float* weight_scale =
+      input_tensors[1].weight_scales ? input_tensors[1].weight_scales->GetPtr<const float>() : nullptr;
+  if (weight_scale == nullptr) {
+    KLLM_THROW("Cannot load weight_scale. Weight_scale is nullptr.");
+  }
+  const size_t weight_scale_count = input_tensors[1].weight_scales->GetElementNumber() == (size_t)n && n > 1 ? n : 1;
+  void* output = output_tensors[0].GetPtr<void>();
+  output_tensors[0].shape = {static_cast<size_t>(m), static_cast<size_t>(n)};
+  output_tensors[0].dtype = input_tensors[0].dtype;
+  void* stream = context_->GetComputeStreams()[rank_].Get();
+  float* input_scale = nullptr;
+  size_t input_scale_count = 1;
+  size_t quant_bytes = ((size_t)m * k + 15) / 16 * 16;
+  if (input_tensors[1].input_scales) {
+    input_scale = input_tensors[1].input_scales->GetPtr<float>();
+    ThrowOnKsqError(ksq_fp8_quantize(KsqDtype<T>(), input, m, k, KSQ_FP8_PER_TENSOR_STATIC, input_quant, input_scale,
+                                     stream), "ksq_fp8_quantize");
+  } else {
+    input_scale = reinterpret_cast<float*>(input_quant + quant_bytes);
+    const bool per_token = weight_scale_count > 1;
+    input_scale_count = per_token ? m : 1;
+    ThrowOnKsqError(ksq_fp8_quantize(KsqDtype<T>(), input, m, k,
+                                     per_token ? KSQ_FP8_PER_TOKEN_DYNAMIC : KSQ_FP8_PER_TENSOR_DYNAMIC, input_quant,
+                                     input_scale, stream), "ksq_fp8_quantize");
+  }
+  ThrowOnKsqError(ksq_fp8_gemm(KsqDtype<T>(), output, input_quant, input_scale, input_scale_count, weight_quant,
+                               weight_scale, weight_scale_count, m, n, k, gemm_workspace, kFp8GemmWorkspaceBytes,
+                               stream), "ksq_fp8_gemm");
+  return Status();
+}
+
+template class Fp8MatMulLayer<float16>;
+template class Fp8MatMulLayer<bfloat16>;
+
+template class MatMulLayerFactory<float16>;
+template class MatMulLayerFactory<bfloat16>;
+
+}  // namespace ksana_llm

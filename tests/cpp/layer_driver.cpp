@@ -1,0 +1,272 @@
+// Test driver of the C++ layer shims: builds the layers through MatMulLayerFactory exactly as CommonModel does
+// (AutoCreateLayer by weight name), runs Forward on the device and writes the result for the Python parity tests.
+//
+//   layer_driver w4a16 <dir> <f16|bf16> <m> <k> <n> <g> <gptq|awq> <gptq|awq|rowmajor> <none|awq|uint8|additive>
+//       reads <dir>/qweight.bin, qzeros.bin (unless none), scales.bin, act.bin; writes <dir>/out.bin
+//   layer_driver fp8 <dir> <f16|bf16> <m> <k> <n> <wscales: 1|n> <static: 0|1>
+//       reads <dir>/wq.bin, wscale.bin, act.bin, iscale.bin (static); writes <dir>/out.bin
+//   layer_driver errors
+//       exercises the error conventions; prints one line per check
+// Prints "OK <m> <n> <dtype>" or "THROW <message>".
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "matmul_layer_factory.h"
+
+using namespace ksana_llm;
+
+static std::vector<char> ReadFile(const std::string& path) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) throw std::runtime_error("cannot open " + path);
+  return std::vector<char>((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+}
+
+static Tensor Upload(const std::vector<char>& bytes, DataType dtype, const std::vector<size_t>& shape) {
+  Tensor t;
+  CreateTensor(t, shape, dtype, 0, MEMORY_DEVICE);
+  if (t.GetTotalBytes() != bytes.size())
+    throw std::runtime_error("size mismatch: file has " + std::to_string(bytes.size()) + " bytes, tensor " +
+                             std::to_string(t.GetTotalBytes()));
+  if (hipMemcpy(t.GetPtr<void>(), bytes.data(), bytes.size(), hipMemcpyHostToDevice) != hipSuccess)
+    throw std::runtime_error("hipMemcpy H2D failed");
+  return t;
+}
+
+static void Download(const Tensor& t, const std::string& path) {
+  std::vector<char> host(t.GetTotalBytes());
+  if (hipDeviceSynchronize() != hipSuccess) throw std::runtime_error("device error after Forward");
+  if (hipMemcpy(host.data(), t.GetPtr<void>(), host.size(), hipMemcpyDeviceToHost) != hipSuccess)
+    throw std::runtime_error("hipMemcpy D2H failed");
+  std::ofstream f(path, std::ios::binary);
+  f.write(host.data(), host.size());
+}
+
+struct OneWeight : public BaseWeight {
+  Tensor t;
+  Tensor GetModelWeights(const std::string&) override { return t; }
+};
+
+template <typename T>
+static int RunW4(int argc, char** argv) {
+  const std::string dir = argv[2];
+  const size_t m = atol(argv[4]), k = atol(argv[5]), n = atol(argv[6]), g = atol(argv[7]);
+  const std::string method = argv[8], layout = argv[9], zeros = argv[10];
+  const DataType dt = TypeTraits<T>::kDataType;
+  auto context = std::make_shared<Context>(1);
+
+  Tensor scales = Upload(ReadFile(dir + "/scales.bin"), dt, {k / g, n});
+  Tensor qweight, qzeros, weight, weight_sz;
+  GroupWeightLayout lay;
+  if (layout == "gptq") {
+    lay = GROUP_WEIGHT_GPTQ_INT32;
+    qweight = Upload(ReadFile(dir + "/qweight.bin"), TYPE_INT32, {k / 8, n});
+  } else if (layout == "awq") {
+    lay = GROUP_WEIGHT_AWQ_INT32;
+    qweight = Upload(ReadFile(dir + "/qweight.bin"), TYPE_INT32, {k, n / 8});
+  } else {
+    lay = GROUP_WEIGHT_ROWMAJOR_INT4;
+    qweight = Upload(ReadFile(dir + "/qweight.bin"), TYPE_INT8, {k, n / 2});
+  }
+  const Tensor* zp = nullptr;
+  bool additive = false;
+  if (zeros == "awq") {
+    qzeros = Upload(ReadFile(dir + "/qzeros.bin"), TYPE_INT32, {k / g, n / 8});
+    zp = &qzeros;
+  } else if (zeros == "uint8") {
+    qzeros = Upload(ReadFile(dir + "/qzeros.bin"), TYPE_UINT8, {k / g, n});
+    zp = &qzeros;
+  } else if (zeros == "additive") {
+    qzeros = Upload(ReadFile(dir + "/qzeros.bin"), dt, {k / g, n});
+    zp = &qzeros;
+    additive = true;
+  }
+  RepackGroupQuantWeight(lay, qweight, zp, additive, scales, k, n, g, weight, weight_sz, 0,
+                         context->GetComputeStreams()[0]);
+
+  ModelConfig cfg;
+  cfg.is_quant = true;
+  cfg.quant_config.method = method == "awq" ? QUANT_AWQ : QUANT_GPTQ;
+  cfg.quant_config.group_size = g;
+  cfg.hidden_units = k;
+  cfg.size_per_head = n;  // query_key_value: k = hidden_units, n = size_per_head * (head_num + 2 * kv heads)
+  cfg.head_num = 1;
+  cfg.num_key_value_heads = 0;
+  cfg.max_scheduler_token_num = m;
+  std::shared_ptr<Tensor> workspace;
+  MatMulLayerFactory<T> factory(workspace, cfg, 0, context);
+  auto holder = std::make_shared<OneWeight>();
+  holder->t = weight;
+  auto layer = factory.AutoCreateLayer(holder, "model.layers.0.self_attn.query_key_value.weight", TYPE_I4_GROUP, dt, dt, {});
+
+  Tensor act = Upload(ReadFile(dir + "/act.bin"), dt, {m, k});
+  Tensor out;
+  CreateTensor(out, {m, n}, dt, 0, MEMORY_DEVICE);
+  out.shape = {0};
+  std::vector<Tensor> outputs = {out};
+  Status st = layer->Forward({act, weight}, outputs);
+  if (!st.OK()) throw std::runtime_error("Forward returned " + st.GetMessage());
+  Download(outputs[0], dir + "/out.bin");
+  std::cout << "OK " << outputs[0].shape[0] << " " << outputs[0].shape[1] << " " << outputs[0].dtype << std::endl;
+  return 0;
+}
+
+template <typename T>
+static int RunFp8(int argc, char** argv) {
+  const std::string dir = argv[2];
+  const size_t m = atol(argv[4]), k = atol(argv[5]), n = atol(argv[6]);
+  const size_t nws = std::string(argv[7]) == "n" ? n : 1;
+  const bool is_static = atoi(argv[8]) != 0;
+  const DataType dt = TypeTraits<T>::kDataType;
+  auto context = std::make_shared<Context>(1);
+  Tensor wq = Upload(ReadFile(dir + "/wq.bin"), TYPE_FP8_E4M3, {n, k});
+  Tensor wscale = Upload(ReadFile(dir + "/wscale.bin"), TYPE_FP32, {nws});
+  Tensor iscale;
+  wq.weight_scales = &wscale;
+  if (is_static) {
+    iscale = Upload(ReadFile(dir + "/iscale.bin"), TYPE_FP32, {1});
+    wq.input_scales = &iscale;
+  }
+  ModelConfig cfg;
+  cfg.max_scheduler_token_num = m;
+  std::shared_ptr<Tensor> workspace;
+  MatMulLayerFactory<T> factory(workspace, cfg, 0, context);
+  auto holder = std::make_shared<OneWeight>();
+  holder->t = wq;
+  auto layer = factory.AutoCreateLayer(holder, "model.layers.0.mlp.down_proj.weight", TYPE_FP8_E4M3, dt, dt, {});
+  Tensor act = Upload(ReadFile(dir + "/act.bin"), dt, {m, k});
+  Tensor out;
+  CreateTensor(out, {m, n}, dt, 0, MEMORY_DEVICE);
+  std::vector<Tensor> outputs = {out};
+  Status st = layer->Forward({act, wq}, outputs);
+  if (!st.OK()) throw std::runtime_error("Forward returned " + st.GetMessage());
+  Download(outputs[0], dir + "/out.bin");
+  std::cout << "OK " << outputs[0].shape[0] << " " << outputs[0].shape[1] << " " << outputs[0].dtype << std::endl;
+  return 0;
+}
+
+template <typename F>
+static void Expect(const char* name, bool want_throw, F f) {
+  bool threw = false;
+  std::string msg;
+  try {
+    f();
+  } catch (const std::runtime_error& e) {
+    threw = true;
+    msg = e.what();
+  } catch (const std::bad_any_cast& e) {
+    threw = true;
+    msg = std::string("bad_any_cast: ") + e.what();
+  }
+  std::cout << (threw == want_throw ? "PASS " : "FAIL ") << name << (threw ? " :: " + msg : "") << std::endl;
+}
+
+static int RunErrors() {
+  auto context = std::make_shared<Context>(1);
+  ModelConfig cfg;
+  cfg.is_quant = true;
+  cfg.quant_config.method = QUANT_GPTQ;
+  std::shared_ptr<Tensor> workspace;
+  MatMulLayerFactory<float16> factory(workspace, cfg, 0, context);
+  std::vector<std::any> good = {false, false, true, CUTLASS_BACKEND, size_t(16), size_t(256), size_t(256), size_t(128), true};
+
+  Expect("unregistered (weight,input,output,quant) key throws", true,
+         [&] { factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP32, TYPE_FP32, good, QUANT_GPTQ); });
+  Expect("parameter pack in the wrong order throws", true, [&] {
+    std::vector<std::any> bad = {size_t(16), false, true};
+    factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, bad, QUANT_GPTQ);
+  });
+  Expect("group size 32 is refused when the workspace is sized", true, [&] {
+    std::vector<std::any> p = good;
+    p[7] = size_t(32);
+    auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
+    Tensor a, w, s, o;
+    CreateTensor(a, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    CreateTensor(w, {256, 128}, TYPE_UINT8, 0, MEMORY_DEVICE);
+    CreateTensor(s, {8, 256}, TYPE_UINT32, 0, MEMORY_DEVICE);
+    CreateTensor(o, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    w.scales = &s;
+    std::vector<Tensor> outs = {o};
+    l->Forward({a, w}, outs);
+  });
+  Expect("k not a multiple of 128 is refused", true, [&] {
+    std::vector<std::any> p = good;
+    p[6] = size_t(192);
+    factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
+  });
+  Expect("desc_act weights are refused at Forward", true, [&] {
+    std::vector<std::any> p = good;
+    p[1] = true;
+    auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
+    Tensor a, w, s, o;
+    CreateTensor(a, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    CreateTensor(w, {256, 128}, TYPE_UINT8, 0, MEMORY_DEVICE);
+    CreateTensor(s, {2, 256}, TYPE_UINT32, 0, MEMORY_DEVICE);
+    CreateTensor(o, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    w.scales = &s;
+    std::vector<Tensor> outs = {o};
+    l->Forward({a, w}, outs);
+  });
+  Expect("weight without bound scales throws", true, [&] {
+    auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, good, QUANT_GPTQ);
+    Tensor a, w, o;
+    CreateTensor(a, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    CreateTensor(w, {256, 128}, TYPE_UINT8, 0, MEMORY_DEVICE);
+    CreateTensor(o, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    std::vector<Tensor> outs = {o};
+    l->Forward({a, w}, outs);
+  });
+  Expect("fp8: null weight scale throws", true, [&] {
+    std::vector<std::any> p = {size_t(4), size_t(256)};
+    auto l = factory.CreateLayer(TYPE_FP8_E4M3, TYPE_FP16, TYPE_FP16, p, QUANT_FP8_E4M3);
+    Tensor a, w, o;
+    CreateTensor(a, {4, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
+    CreateTensor(w, {64, 256}, TYPE_FP8_E4M3, 0, MEMORY_DEVICE);
+    CreateTensor(o, {4, 64}, TYPE_FP16, 0, MEMORY_DEVICE);
+    std::vector<Tensor> outs = {o};
+    l->Forward({a, w}, outs);
+  });
+  Expect("fp8: workspace smaller than the request throws", true, [&] {
+    std::vector<std::any> p = {size_t(4), size_t(256)};
+    auto l = factory.CreateLayer(TYPE_FP8_E4M3, TYPE_FP16, TYPE_FP16, p, QUANT_FP8_E4M3);
+    Tensor a, w, o, sc;
+    CreateTensor(a, {64, 256}, TYPE_FP16, 0, MEMORY_DEVICE);  // m = 64 > max_m = 4
+    CreateTensor(w, {64, 256}, TYPE_FP8_E4M3, 0, MEMORY_DEVICE);
+    CreateTensor(sc, {1}, TYPE_FP32, 0, MEMORY_DEVICE);
+    CreateTensor(o, {64, 64}, TYPE_FP16, 0, MEMORY_DEVICE);
+    w.weight_scales = &sc;
+    std::vector<Tensor> outs = {o};
+    l->Forward({a, w}, outs);
+  });
+  Expect("well-formed group layer builds and shares one workspace", false, [&] {
+    auto l1 = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, good, QUANT_GPTQ);
+    std::vector<std::any> big = good;
+    big[5] = size_t(4096);
+    big[6] = size_t(4096);
+    auto l2 = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, big, QUANT_AWQ);
+    if (!factory.GetWorkSpaceBuffer() || factory.GetWorkSpaceBuffer()->GetTotalBytes() < l2->GetWorkSpaceSize())
+      throw std::runtime_error("shared workspace was not grown to the largest request");
+  });
+  return 0;
+}
+
+int main(int argc, char** argv) {
+  try {
+    if (argc >= 2 && std::string(argv[1]) == "errors") return RunErrors();
+    if (argc == 11 && std::string(argv[1]) == "w4a16")
+      return std::string(argv[3]) == "f16" ? RunW4<float16>(argc, argv) : RunW4<bfloat16>(argc, argv);
+    if (argc == 9 && std::string(argv[1]) == "fp8")
+      return std::string(argv[3]) == "f16" ? RunFp8<float16>(argc, argv) : RunFp8<bfloat16>(argc, argv);
+    std::cerr << "usage: see the header of layer_driver.cpp" << std::endl;
+    return 2;
+  } catch (const std::exception& e) {
+    std::cout << "THROW " << e.what() << std::endl;
+    return 1;
+  }
+}
