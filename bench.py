@@ -174,6 +174,7 @@ def main():
     if not args.no_extra:
         extra["per_shape"] = per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, dtype)
         extra["prefill_m4096"] = prefill(torch, capi, layers[0], dev, stream)
+        extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], dev, stream, "f16")
     if not args.no_cpu:
         result["cpu_baseline"], extra["parity_vs_cpu"] = cpu_baseline(np, torch, capi, layers[0], acts, outs,
                                                                       workspace, ws_bytes, M, dtype, step_bytes)
@@ -215,7 +216,7 @@ def per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, d
     return table
 
 
-def prefill(torch, capi, layer, dev, stream):
+def prefill(torch, capi, layer, dev, stream, dtype_name="bf16"):
     """configs[2] at M = 4096 (bf16 activations): TFLOP/s per shape against the dense MFMA peak.  The weights are
     the fp16-scaled set of layer 0 re-used with bf16 activations only for timing (the arithmetic is the same)."""
     M = 4096
@@ -223,16 +224,20 @@ def prefill(torch, capi, layer, dev, stream):
     gen.manual_seed(11)
     table = {}
     for name, k, n, w, sz in layer.weights:
-        act = torch.randn((M, k), device=dev, generator=gen).to(torch.bfloat16)
-        out = torch.empty((M, n), dtype=torch.bfloat16, device=dev)
+        tdt = torch.bfloat16 if dtype_name == "bf16" else torch.float16
+        cdt = capi.BF16 if dtype_name == "bf16" else capi.F16
+        act = torch.randn((M, k), device=dev, generator=gen).to(tdt)
+        out = torch.empty((M, n), dtype=tdt, device=dev)
+        wsb = capi.w4a16_workspace_bytes(M, n, k)
+        ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
 
         def launch(i):
-            capi.w4a16_gemm(capi.BF16, out, act, w, sz, M, n, k, GROUP, None, 0, stream.cuda_stream)
+            capi.w4a16_gemm(cdt, out, act, w, sz, M, n, k, GROUP, ws, wsb, stream.cuda_stream)
 
         us = time_graph(torch, stream, launch, 4)
         tf = 2.0 * M * k * n / us / 1e6
         table[name] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-        del act, out
+        del act, out, ws
     return table
 
 

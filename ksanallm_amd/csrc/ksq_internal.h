@@ -108,8 +108,9 @@ W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes)
 int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
                         const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
 int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, hipStream_t s);
-bool w4a16_prefill_supported(size_t m, size_t n, size_t k, size_t g);
+                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k);
+bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g);
 int w4a16_stream_max_slices(int mt, int nt);
 
 struct KstatPlan {

@@ -1,13 +1,329 @@
-// W4A16 prefill kernel (large M, MFMA-bound): LDS-tiled activations, weights dequantised in registers.
+// W4A16 prefill kernel (large M, MFMA-bound).
+//
+// Workgroup tile 128 rows x 256 columns, four waves side by side: every wave owns a 128 x 64 output tile
+// (8 x 4 MFMA tiles of 16 x 16, fp32 accumulators in registers).  Activations are staged through LDS in MFMA
+// fragment order, 64 k at a time, double-buffered, one barrier per stage.  Weights never touch LDS: each wave
+// reads its own column tiles straight from the fragment-order buffer (one 128-bit load per lane = the B operands of
+// four 16x16x32 MFMAs), one k tile ahead, and dequantises them in registers once per 128 rows:
+//   w = T((u - z) * s), rounded once -- the reference's dequantise-then-MMA semantics
+//   (LK/cutlass_extensions/gemm/warp/mma_tensorop_dequantizer.h:206-245, 368-394), with no second rounding.
+//   bit operations to 1024 + u / 64 + u, packed fp16 subtract of (bias + z) (exact), packed multiply by s.
+// The matrix cores always run in fp16.  Rounding a dequantised weight to bf16 (8 significant bits) would cost up to
+// 2^-8 per weight -- together with the bf16 rounding of the output more than the 1e-2 bound on the maximum relative
+// error allows -- so bf16 activations are first re-encoded, exactly, as fp16 with one power-of-two exponent per row
+// (a bf16 significand fits into fp16; the row exponent keeps every row inside the fp16 range whatever its
+// magnitude); the row factor 2^e is applied to the fp32 accumulators in the epilogue, and the bf16 group scales
+// are converted to fp16.
+// Workgroups are numbered so that those sharing a row block of the activations run on the same XCD (own L2).
 #include "ksq_internal.h"
+#include "ksq_w4a16_ops.h"
 
 namespace ksq {
+namespace {
 
-bool w4a16_prefill_supported(size_t, size_t, size_t, size_t) { return false; }
+using namespace w4;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-int w4a16_launch_prefill(int, void*, const void*, const void*, const void*, size_t, size_t, size_t, size_t,
-                         hipStream_t) {
-  return fail(KSQ_ERR_UNSUPPORTED, "prefill kernel not built");
+struct PrefillArgs {
+  const void* weight;
+  const void* sz;
+  const void* act;
+  void* out;
+  const float* row_scale;  // bf16 route: 2^e per row of the re-encoded activations
+  int M, N, K, KT, G, ntiles, mblocks, nblocks;
+};
+
+constexpr int kBM = 128, kBNT = 16;  // rows and column tiles (of 16) per workgroup
+constexpr int kMT = 8, kNT = 4;      // MFMA tiles per wave: 8 x 4
+
+template <typename T>
+struct Dequant;
+
+template <>
+struct Dequant<_Float16> {
+  // per (group, column): packed (s, s), packed (1024 + z), packed (64 + z)
+  struct Consts {
+    uint32_t s2, c_lo, c_hi;
+  };
+  static __device__ inline Consts prepare(uint32_t szw) {
+    const uint32_t z = szw >> 16, zc = z | (z << 16);
+    Consts k;
+    k.s2 = (szw & 0xFFFFu) | (szw << 16);
+    k.c_lo = 0x64006400u | zc;
+    k.c_hi = 0x54005400u | (zc << 4);
+    return k;
+  }
+  static __device__ inline u32x4 run(uint32_t x, const Consts& k, uint32_t m_lo, uint32_t m_hi, uint32_t g_lo,
+                                     uint32_t g_hi) {
+    const uint32_t y = x >> 8;
+    const half2v s = __builtin_bit_cast(half2v, k.s2);
+    const half2v clo = __builtin_bit_cast(half2v, k.c_lo), chi = __builtin_bit_cast(half2v, k.c_hi);
+    half2v r0 = (__builtin_bit_cast(half2v, (x & m_lo) | g_lo) - clo) * s;
+    half2v r1 = (__builtin_bit_cast(half2v, (x & m_hi) | g_hi) - chi) * s;
+    half2v r2 = (__builtin_bit_cast(half2v, (y & m_lo) | g_lo) - clo) * s;
+    half2v r3 = (__builtin_bit_cast(half2v, (y & m_hi) | g_hi) - chi) * s;
+    return u32x4{__builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1), __builtin_bit_cast(uint32_t, r2),
+                 __builtin_bit_cast(uint32_t, r3)};
+  }
+};
+
+template <>
+struct Dequant<__bf16> : Dequant<_Float16> {
+  // scales arrive as bf16 bits; the arithmetic is the fp16 one
+  static __device__ inline Consts prepare(uint32_t szw) {
+    const _Float16 sh = (_Float16)__builtin_bit_cast(float, szw << 16);
+    const uint32_t sb = __builtin_bit_cast(uint16_t, sh);
+    return Dequant<_Float16>::prepare((szw & 0xFFFF0000u) | sb);
+  }
+};
+
+// bf16 [M][K] -> fp16 [M][K] * 2^-e[row] (exact: power-of-two shift of an 8-bit significand into 11 bits), with
+// e[row] chosen so that the row maximum lands at 2^14; row_scale[row] = 2^e.  One workgroup per row.
+__global__ __launch_bounds__(256) void bf16_rows_to_f16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                               float* __restrict__ row_scale, int K) {
+  __shared__ float smem[4];
+  const size_t row = blockIdx.x;
+  const uint16_t* s = src + row * K;
+  uint16_t* d = dst + row * K;
+  float mx = 0.f;
+  for (int i = threadIdx.x; i < K; i += 256) {
+    const float v = __builtin_fabsf(__builtin_bit_cast(float, (uint32_t)s[i] << 16));
+    mx = (v == v && v < __builtin_inff()) ? __builtin_fmaxf(mx, v) : mx;  // NaN / Inf do not set the exponent
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off));
+  if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = __builtin_fmaxf(__builtin_fmaxf(smem[0], smem[1]), __builtin_fmaxf(smem[2], smem[3]));
+  int e = 0;
+  if (mx > 0.f) e = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFF) - 127 - 14;
+  const float down = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);  // 2^-e, e in [-163, 113]: clamp below
+  const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+  if (threadIdx.x == 0) row_scale[row] = up;
+  for (int i = threadIdx.x; i < K; i += 256) {
+    const float v = __builtin_bit_cast(float, (uint32_t)s[i] << 16) * down;
+    d[i] = __builtin_bit_cast(uint16_t, (_Float16)v);
+  }
+}
+
+template <typename T, int GPT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
+  using O = Ops<_Float16>;  // the matrix cores run in fp16 for both element types
+  using DQ = Dequant<T>;
+  constexpr bool kBF16 = sizeof(T) == 2 && !__is_same(T, _Float16);
+  constexpr int kStage = kMT * 2 * 64;  // 16-byte elements per activation stage (128 rows x 64 k)
+  constexpr int kEpiStride = 68;        // floats per row of the epilogue transpose (2-way conflicts at worst)
+  __shared__ u32x4 lds[2 * kStage];     // 32 KiB: two activation stages; reused by the epilogue
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, j = lane >> 4;
+
+  // XCD-aware numbering: hardware hands consecutive workgroup ids to the 8 XCDs in turn; give every XCD a
+  // contiguous run of (row block, column block) pairs so that the workgroups sharing activations share an L2
+  const int total = gridDim.x, per_xcd = total >> 3;
+  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int mb = lid / p.nblocks, nb = lid - mb * p.nblocks;
+  if (mb >= p.mblocks) return;  // padding workgroups (grid is rounded up to a multiple of 8)
+  const int m0 = mb * kBM;
+  const int nt0 = nb * kBNT + wave * kNT;
+
+  __amdgpu_buffer_rsrc_t rs_w[kNT], rs_sz[kNT];
+  bool tile_ok[kNT];
+#pragma unroll
+  for (int t = 0; t < kNT; ++t) {
+    const int nt = nt0 + t;
+    tile_ok[t] = nt < p.ntiles;
+    const size_t ntc = tile_ok[t] ? (size_t)nt : 0;
+    rs_w[t] = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(static_cast<const char*>(p.weight) + ntc * p.KT * 1024), 0, tile_ok[t] ? p.KT * 1024 : 0,
+        0x00020000);
+    rs_sz[t] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(static_cast<const char*>(p.sz) + ntc * p.G * 64), 0,
+                                                 tile_ok[t] ? p.G * 64 : 0, 0x00020000);
+  }
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
+  // staging role: fragments f = 4 * wave + i, i < 4, of a stage; f = (row tile mt, 32-k step ks)
+  unsigned a_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int f = 4 * wave + i, mt = f >> 1, ks = f & 1;
+    const int row = m0 + 16 * mt + c;
+    a_off[i] = row < p.M ? ((unsigned)row * p.K + 32 * ks + 8 * j) * 2u : 0x80000000u;
+  }
+  const unsigned w_voff = lane * 16u, sz_voff = c * 4u;
+
+  f32x4 acc[kMT][kNT];
+#pragma unroll
+  for (int mt = 0; mt < kMT; ++mt)
+#pragma unroll
+    for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 a_reg[4];
+  u32x4 b_cur[kNT], b_nxt[kNT];
+  uint32_t sz_cur[kNT][GPT], sz_nxt[kNT][GPT];
+
+  auto load_a = [&](int stage) {  // stage = 64-k slice index; beyond K reads as zero
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      a_reg[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                               rs_a, (unsigned)stage * 128u < (unsigned)p.K * 2u ? a_off[i] + stage * 128u
+                                                                                               : 0x80000000u,
+                                               0, 0));
+  };
+  auto write_a = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds[buf * kStage + (4 * wave + i) * 64 + lane] = a_reg[i];
+  };
+  auto load_b = [&](int kt) {  // past the last k tile the resource returns zero
+#pragma unroll
+    for (int t = 0; t < kNT; ++t) {
+      b_nxt[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[t], w_voff + kt * 1024u, 0, 0));
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi)
+        sz_nxt[t][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[t], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
+    }
+  };
+
+  uint32_t m_lo = Ops<_Float16>::kMaskLo, m_hi = Ops<_Float16>::kMaskHi, g_lo = Ops<_Float16>::kMagicLo,
+           g_hi = Ops<_Float16>::kMagicHi;
+  asm volatile("" : "+s"(m_lo));
+  asm volatile("" : "+v"(g_lo));
+  asm volatile("" : "+v"(g_hi));
+  asm volatile("" : "+v"(m_hi));
+
+  auto compute_half = [&](int buf, int half) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int d = 2 * half + ks;
+      u32x4 b[kNT];
+#pragma unroll
+      for (int t = 0; t < kNT; ++t) {
+        const typename DQ::Consts k = DQ::prepare(sz_cur[t][GPT == 2 ? half : 0]);
+        b[t] = DQ::run(b_cur[t][d], k, m_lo, m_hi, g_lo, g_hi);
+      }
+#pragma unroll
+      for (int mt = 0; mt < kMT; ++mt) {
+        const u32x4 af = lds[buf * kStage + (mt * 2 + ks) * 64 + lane];
+#pragma unroll
+        for (int t = 0; t < kNT; ++t) acc[mt][t] = O::mfma(af, b[t], acc[mt][t]);
+      }
+    }
+  };
+
+  // ---- main loop over k tiles; two activation stages (64 k each) per tile
+  load_b(0);
+  load_a(0);
+  write_a(0);
+  load_a(1);
+#pragma unroll
+  for (int t = 0; t < kNT; ++t) {
+    b_cur[t] = b_nxt[t];
+#pragma unroll
+    for (int gi = 0; gi < GPT; ++gi) sz_cur[t][gi] = sz_nxt[t][gi];
+  }
+  for (int kt = 0; kt < p.KT; ++kt) {
+    // stage 2*kt
+    __syncthreads();  // stage 2*kt is visible; everyone has finished reading the other buffer
+    write_a(1);       // stage 2*kt + 1
+    load_a(2 * kt + 2);
+    load_b(kt + 1);
+    compute_half(0, 0);
+    // stage 2*kt + 1
+    __syncthreads();
+    write_a(0);  // stage 2*kt + 2
+    load_a(2 * kt + 3);
+    compute_half(1, 1);
+#pragma unroll
+    for (int t = 0; t < kNT; ++t) {
+      b_cur[t] = b_nxt[t];
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi) sz_cur[t][gi] = sz_nxt[t][gi];
+    }
+  }
+
+  // ---- epilogue: transpose each 16-row slab through LDS so that every lane stores 16 contiguous bytes
+  __syncthreads();
+  float* epi = reinterpret_cast<float*>(lds) + wave * (16 * kEpiStride);  // 4352 B per wave
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int ncol0 = nt0 * 16;
+#pragma unroll
+  for (int mt = 0; mt < kMT; ++mt) {
+#pragma unroll
+    for (int t = 0; t < kNT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) epi[(4 * j + i) * kEpiStride + 16 * t + c] = acc[mt][t][i];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int r = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
+      const float* src = epi + r * kEpiStride + cc;
+      const int row = m0 + 16 * mt + r, col = ncol0 + cc;
+      float rs = 1.f;
+      if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
+      u32x4 packed;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        packed[q] = (uint32_t)Ops<T>::to_bits(src[2 * q] * rs) | ((uint32_t)Ops<T>::to_bits(src[2 * q + 1] * rs) << 16);
+      if (row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+}
+
+}  // namespace
+
+bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g) {
+  (void)g;
+  (void)dtype;
+  return m >= 128 && n % 16 == 0 && m * k * 2 < 0x7FFFFF00ull && (k / kTileK) * 1024 < 0x7FFFFF00ull;
+}
+
+// bf16 route: fp16 copy of the activations + one float per row
+size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k) {
+  if (dtype != KSQ_BF16) return 0;
+  return (m * k * 2 + 255) / 256 * 256 + m * 4;
+}
+
+int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
+                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
+  KSQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && n % 8 == 0, KSQ_ERR_INVALID_ARGUMENT,
+              "prefill output must be 16-byte aligned");
+  PrefillArgs a{};
+  a.weight = weight;
+  a.sz = sz;
+  a.act = act;
+  a.out = out;
+  a.row_scale = nullptr;
+  a.M = (int)m;
+  a.N = (int)n;
+  a.K = (int)k;
+  a.KT = (int)(k / kTileK);
+  a.G = (int)(k / g);
+  a.ntiles = (int)(n / kTileN);
+  a.mblocks = (int)((m + kBM - 1) / kBM);
+  a.nblocks = (a.ntiles + kBNT - 1) / kBNT;
+  const size_t total = ((size_t)a.mblocks * a.nblocks + 7) / 8 * 8;
+  KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+  dim3 grid((unsigned)total);
+  const int gpt = (int)(kTileK / g);
+  if (dtype == KSQ_F16) {
+    if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<_Float16, 1>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((w4a16_prefill_kernel<_Float16, 2>), grid, dim3(256), 0, s, a);
+  } else {
+    KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "bf16 prefill needs its workspace");
+    uint16_t* a16 = static_cast<uint16_t*>(workspace);
+    float* row_scale = reinterpret_cast<float*>(static_cast<char*>(workspace) + (m * k * 2 + 255) / 256 * 256);
+    hipLaunchKernelGGL(bf16_rows_to_f16_kernel, dim3((unsigned)m), dim3(256), 0, s, static_cast<const uint16_t*>(act),
+                       a16, row_scale, (int)k);
+    a.act = a16;
+    a.row_scale = row_scale;
+    if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<__bf16, 1>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((w4a16_prefill_kernel<__bf16, 2>), grid, dim3(256), 0, s, a);
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
 }
 
 }  // namespace ksq
