@@ -391,6 +391,9 @@ int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_s
               KSQ_ERR_INVALID_ARGUMENT, "act_q and w_q must be 16-byte aligned");
   const DeviceInfo* di = device_info();
   if (!di) return KSQ_ERR_HIP;
+  if (fp8_prefill_supported(m, n, k) && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
+    return fp8_launch_prefill(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
+                              static_cast<hipStream_t>(stream));
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
   Fp8Plan plan = fp8_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
   Fp8Args a{};

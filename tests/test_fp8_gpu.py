@@ -183,6 +183,28 @@ def test_gemm_per_tensor_scales_and_ragged_shapes(gpu):
     orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), "fp8 ragged no workspace")
 
 
+@pytest.mark.parametrize("M,K,N", [(128, 1024, 256), (300, 1008, 264), (257, 2048, 520)])
+def test_gemm_large_m_ragged(gpu, M, K, N):
+    """M >= 128 takes the MFMA-tiled kernel: ragged M, K not a multiple of the 128-byte stage, N not of the tile."""
+    xq, xs, wq, ws = _fp8_case(410 + M, M, K, N)
+    got = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+    orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"fp8 large M={M} K={K} N={N}")
+    got1 = _run_gemm(gpu, xq, xs[:1].copy(), wq, ws[:1].copy(), "f16")
+    orc.assert_parity(got1, orc.fp8_gemm(xq, xs[:1].copy(), wq, ws[:1].copy()), f"fp8 large per-tensor M={M}")
+
+
+def test_gemm_large_m_small_integers_exact(gpu):
+    rng = np.random.default_rng(420)
+    M, K, N = 256, 384, 256
+    codes = orc.e4m3_encode(np.arange(-4, 5, dtype=np.float32))
+    xq = codes[rng.integers(0, 9, size=(M, K))]
+    wq = codes[rng.integers(0, 9, size=(N, K))]
+    one = np.ones(1, dtype=np.float32)
+    got = _run_gemm(gpu, xq, one, wq, one, "f16")
+    want = orc.e4m3_decode(xq).astype(np.int64) @ orc.e4m3_decode(wq).astype(np.int64).T
+    assert np.array_equal(orc.to_bits(got, orc.F16), orc.to_bits(want.astype(np.float32), orc.F16))
+
+
 def test_gemm_small_integers_exact(gpu):
     rng = np.random.default_rng(402)
     M, K, N = 16, 512, 64
