@@ -9,7 +9,7 @@ are resident in HBM before the timed region; the K timed steps are one HIP graph
 events on that stream.
 
 Prints ONE JSON line: value = whole-job algorithmic GB/s, plus `roofline` for the dominant kernel (the W4A16
-streaming kernel) and `cpu_baseline` (the CPU oracle -- dequantize to fp32 + blocked OpenMP GEMM -- timed on the
+k-stationary decode kernel) and `cpu_baseline` (the CPU oracle -- dequantize to fp32 + blocked OpenMP GEMM -- timed on the
 same workload on this machine's host cores).
 """
 import argparse

@@ -99,9 +99,12 @@ int ksq_w4a16_repack_host(int src_layout, const void* qweight_host, int zero_kin
  * FpAIntBGroupCutlassGemmWrapper::Gemm (LK/asymmetric_gemm/asymmetric_gemm_wrapper.cu:53-77):
  *   out[m,n] = T( sum_k act[m,k] * s[k/g,n] * (u[k,n] - z[k/g,n]) ),  fp32 accumulation.
  * act is [m,k] row-major T, out is [m,n] row-major T, weight / sz come from ksq_w4a16_repack.
- * The workspace holds split-K partial sums; with workspace == NULL or too small the call still succeeds
- * without split-K.  Calls that may overlap in time on one device must use different streams' worth of
- * workspace: the workspace is scratch for the duration of one call only and holds no state between calls. */
+ * The workspace (256-byte aligned, ksq_w4a16_workspace_bytes) holds split-K partial sums and, for bf16
+ * activations at m >= 128, the fp16 re-encoding of the activations.  With workspace == NULL, misaligned or too
+ * small the call still succeeds on a slower route that needs none.  The workspace is scratch for the duration
+ * of one call and holds no state between calls; calls that may overlap in time on one device need a workspace
+ * each, and at most 16 split-K launches of this library may be in flight on one device at a time (they share
+ * 16 rotating sets of arrival counters in library-owned device memory). */
 int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
 
 int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
