@@ -24,6 +24,7 @@ namespace {
 using namespace w4;
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
 
 struct PrefillArgs {
   const void* weight;
@@ -31,7 +32,7 @@ struct PrefillArgs {
   const void* act;
   void* out;
   const float* row_scale;  // bf16 route: 2^e per row of the re-encoded activations
-  int M, N, K, KT, G, ntiles, mblocks, nblocks;
+  int M, N, K, KT, G, ntiles, mblocks, nblocks, super_n;
 };
 
 constexpr int kBM = 128, kBNT = 16;  // rows and column tiles (of 16) per workgroup
@@ -112,45 +113,50 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   using O = Ops<_Float16>;  // the matrix cores run in fp16 for both element types
   using DQ = Dequant<T>;
   constexpr bool kBF16 = sizeof(T) == 2 && !__is_same(T, _Float16);
-  constexpr int kStage = kMT * 2 * 64;  // 16-byte elements per activation stage (128 rows x 64 k)
+  constexpr int kStage = kMT * 4 * 64;  // 16-byte elements per activation stage (128 rows x 128 k) = 32 KiB
   constexpr int kEpiStride = 68;        // floats per row of the epilogue transpose (2-way conflicts at worst)
-  __shared__ u32x4 lds[2 * kStage];     // 32 KiB: two activation stages; reused by the epilogue
+  // two activation stages as two separate objects: loads into one are then known not to alias reads of the other
+  __shared__ u32x4 lds_a0[kStage];
+  __shared__ u32x4 lds_a1[kStage];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
 
-  // XCD-aware numbering: hardware hands consecutive workgroup ids to the 8 XCDs in turn; give every XCD a
-  // contiguous run of (row block, column block) pairs so that the workgroups sharing activations share an L2
-  const int total = gridDim.x, per_xcd = total >> 3;
+  // Workgroup numbering.  Hardware hands consecutive workgroup ids to the 8 XCDs in turn; every XCD (own L2) gets a
+  // contiguous run of logical ids, and logical ids walk 8 x 8 super-tiles of (row block, column block) pairs, so the
+  // 64 workgroups resident on an XCD share 8 activation row blocks and 8 weight column blocks.
+  const int per_xcd = gridDim.x >> 3;
   const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int mb = lid / p.nblocks, nb = lid - mb * p.nblocks;
-  if (mb >= p.mblocks) return;  // padding workgroups (grid is rounded up to a multiple of 8)
+  const int st = lid >> 6, r = lid & 63;
+  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
+  const int mb = st_m * 8 + (r & 7), nb = st_n * 8 + (r >> 3);
+  if (mb >= p.mblocks || nb >= p.nblocks) return;  // padding of partial super-tiles
   const int m0 = mb * kBM;
   const int nt0 = nb * kBNT + wave * kNT;
 
   __amdgpu_buffer_rsrc_t rs_w[kNT], rs_sz[kNT];
-  bool tile_ok[kNT];
 #pragma unroll
   for (int t = 0; t < kNT; ++t) {
     const int nt = nt0 + t;
-    tile_ok[t] = nt < p.ntiles;
-    const size_t ntc = tile_ok[t] ? (size_t)nt : 0;
+    const bool ok = nt < p.ntiles;
+    const size_t ntc = ok ? (size_t)nt : 0;
     rs_w[t] = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<char*>(static_cast<const char*>(p.weight) + ntc * p.KT * 1024), 0, tile_ok[t] ? p.KT * 1024 : 0,
-        0x00020000);
+        const_cast<char*>(static_cast<const char*>(p.weight) + ntc * p.KT * 1024), 0, ok ? p.KT * 1024 : 0, 0x00020000);
     rs_sz[t] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(static_cast<const char*>(p.sz) + ntc * p.G * 64), 0,
-                                                 tile_ok[t] ? p.G * 64 : 0, 0x00020000);
+                                                 ok ? p.G * 64 : 0, 0x00020000);
   }
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
-  // staging role: fragments f = 4 * wave + i, i < 4, of a stage; f = (row tile mt, 32-k step ks)
-  unsigned a_off[4];
+  // Staging role of this wave: fragments f = 8 * wave + i of a stage, f = 4 * (row tile) + (32-k step); rows past M
+  // repeat row M - 1 (their results are never stored).  A fragment is 64 lanes x 16 bytes, lane (c, j) = row c,
+  // k = 8 j .. 8 j + 7 of the step, and goes from global memory straight into LDS at lane * 16.
+  unsigned a_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int f = 4 * wave + i, mt = f >> 1, ks = f & 1;
-    const int row = m0 + 16 * mt + c;
-    a_off[i] = row < p.M ? ((unsigned)row * p.K + 32 * ks + 8 * j) * 2u : 0x80000000u;
+  for (int h = 0; h < 2; ++h) {
+    int row = m0 + 16 * (2 * wave + h) + c;
+    row = row < p.M ? row : p.M - 1;
+    a_off[h] = ((unsigned)row * p.K + 8 * j) * 2u;
   }
   const unsigned w_voff = lane * 16u, sz_voff = c * 4u;
 
@@ -160,29 +166,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
     for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  u32x4 a_reg[4];
-  u32x4 b_cur[kNT], b_nxt[kNT];
-  uint32_t sz_cur[kNT][GPT], sz_nxt[kNT][GPT];
+  struct BTile {
+    u32x4 w[kNT];
+    uint32_t sz[kNT][GPT];
+  };
+  BTile b0, b1;
 
-  auto load_a = [&](int stage) {  // stage = 64-k slice index; beyond K reads as zero
+  auto load_a = [&](u32x4* buf, int kt) {  // k tile kt of the activations -> buf; past K the data is never used
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      a_reg[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                               rs_a, (unsigned)stage * 128u < (unsigned)p.K * 2u ? a_off[i] + stage * 128u
-                                                                                               : 0x80000000u,
-                                               0, 0));
+    for (int i = 0; i < 8; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (8 * wave + i) * 64), 16, a_off[i >> 2],
+                                               kt * 256 + (i & 3) * 64, 0, 0);
   };
-  auto write_a = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) lds[buf * kStage + (4 * wave + i) * 64 + lane] = a_reg[i];
-  };
-  auto load_b = [&](int kt) {  // past the last k tile the resource returns zero
+  auto load_b = [&](BTile& b, int kt) {  // past the last k tile the resource returns zero
 #pragma unroll
     for (int t = 0; t < kNT; ++t) {
-      b_nxt[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[t], w_voff + kt * 1024u, 0, 0));
+      b.w[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[t], w_voff + kt * 1024u, 0, 0));
 #pragma unroll
       for (int gi = 0; gi < GPT; ++gi)
-        sz_nxt[t][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[t], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
+        b.sz[t][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[t], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
     }
   };
 
@@ -193,59 +195,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   asm volatile("" : "+v"(g_hi));
   asm volatile("" : "+v"(m_hi));
 
-  auto compute_half = [&](int buf, int half) {
+  auto compute = [&](const u32x4* buf, const BTile& bt) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const int d = 2 * half + ks;
+    for (int ks = 0; ks < 4; ++ks) {
       u32x4 b[kNT];
 #pragma unroll
       for (int t = 0; t < kNT; ++t) {
-        const typename DQ::Consts k = DQ::prepare(sz_cur[t][GPT == 2 ? half : 0]);
-        b[t] = DQ::run(b_cur[t][d], k, m_lo, m_hi, g_lo, g_hi);
+        const typename DQ::Consts k = DQ::prepare(bt.sz[t][GPT == 2 ? (ks >> 1) : 0]);
+        b[t] = DQ::run(bt.w[t][ks], k, m_lo, m_hi, g_lo, g_hi);
       }
 #pragma unroll
       for (int mt = 0; mt < kMT; ++mt) {
-        const u32x4 af = lds[buf * kStage + (mt * 2 + ks) * 64 + lane];
+        const u32x4 af = buf[(mt * 4 + ks) * 64 + lane];
 #pragma unroll
         for (int t = 0; t < kNT; ++t) acc[mt][t] = O::mfma(af, b[t], acc[mt][t]);
       }
     }
   };
+  // One k tile: everything in flight (this tile's activations and weights) has landed and is visible to the whole
+  // workgroup, and every wave is done with the other buffer; then the next tile's loads go out before the math.
+  auto step = [&](u32x4* cur, u32x4* nxt, const BTile& bc, BTile& bn, int kt) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    load_a(nxt, kt + 1);
+    load_b(bn, kt + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(cur, bc);
+  };
 
-  // ---- main loop over k tiles; two activation stages (64 k each) per tile
-  load_b(0);
-  load_a(0);
-  write_a(0);
-  load_a(1);
-#pragma unroll
-  for (int t = 0; t < kNT; ++t) {
-    b_cur[t] = b_nxt[t];
-#pragma unroll
-    for (int gi = 0; gi < GPT; ++gi) sz_cur[t][gi] = sz_nxt[t][gi];
+  load_a(lds_a0, 0);
+  load_b(b0, 0);
+  int kt = 0;
+  for (; kt + 2 <= p.KT; kt += 2) {
+    step(lds_a0, lds_a1, b0, b1, kt);
+    step(lds_a1, lds_a0, b1, b0, kt + 1);
   }
-  for (int kt = 0; kt < p.KT; ++kt) {
-    // stage 2*kt
-    __syncthreads();  // stage 2*kt is visible; everyone has finished reading the other buffer
-    write_a(1);       // stage 2*kt + 1
-    load_a(2 * kt + 2);
-    load_b(kt + 1);
-    compute_half(0, 0);
-    // stage 2*kt + 1
-    __syncthreads();
-    write_a(0);  // stage 2*kt + 2
-    load_a(2 * kt + 3);
-    compute_half(1, 1);
-#pragma unroll
-    for (int t = 0; t < kNT; ++t) {
-      b_cur[t] = b_nxt[t];
-#pragma unroll
-      for (int gi = 0; gi < GPT; ++gi) sz_cur[t][gi] = sz_nxt[t][gi];
-    }
-  }
+  if (kt < p.KT) step(lds_a0, lds_a1, b0, b1, kt);
 
   // ---- epilogue: transpose each 16-row slab through LDS so that every lane stores 16 contiguous bytes
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
   __syncthreads();
-  float* epi = reinterpret_cast<float*>(lds) + wave * (16 * kEpiStride);  // 4352 B per wave
+  float* epi = reinterpret_cast<float*>(lds_a0) + wave * (16 * kEpiStride);  // 4352 B per wave
   uint16_t* out = static_cast<uint16_t*>(p.out);
   const int ncol0 = nt0 * 16;
 #pragma unroll
@@ -257,9 +248,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
-      const int r = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
-      const float* src = epi + r * kEpiStride + cc;
-      const int row = m0 + 16 * mt + r, col = ncol0 + cc;
+      const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
+      const float* src = epi + rr * kEpiStride + cc;
+      const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
       float rs = 1.f;
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
       u32x4 packed;
@@ -304,7 +295,8 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   a.ntiles = (int)(n / kTileN);
   a.mblocks = (int)((m + kBM - 1) / kBM);
   a.nblocks = (a.ntiles + kBNT - 1) / kBNT;
-  const size_t total = ((size_t)a.mblocks * a.nblocks + 7) / 8 * 8;
+  a.super_n = (a.nblocks + 7) / 8;
+  const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
   KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
   dim3 grid((unsigned)total);
   const int gpt = (int)(kTileK / g);

@@ -1,0 +1,146 @@
+#!/usr/bin/env python3
+"""Writes the golden vectors of tests/golden/*.npz.
+
+Everything here is computed by an independent statement of the formats -- plain numpy integer arithmetic and
+float64 sums, no call into the oracle and none into the GPU library -- so the fixtures pin both.  The formats
+follow KsanaLLM's loader and FP8 helpers (KS = src/ksana_llm, LU = 3rdparty/LLM_kernels/csrc/utils/nvidia):
+
+  gptq_64x64      KS/models/quant/quant_weight.cpp:291-300   qweight int32 [K/8,N], element k=8r+j in bits 4j..4j+3
+  awq_128x64      KS/models/quant/quant_weight.cpp:262-287   qweight int32 [K,N/8], slot j = column 8c+[0,2,4,6,1,3,5,7][j]
+  rowmajor        KS/models/quant/quant_weight.cpp:304-328   int8 [K,N/2], low nibble = even column, signed u-8
+  e4m3_table      OCP FP8 E4M3 (bias 7, no infinities, 0x7f/0xff NaN, max 448), as __nv_fp8_e4m3 in LU/cuda_fp8_utils.h
+  w4a16_*         out = sum_k a[m,k] * s[k/g,n] * (u[k,n] - z[k/g,n]) in float64 from the exact fp16 / bf16 values,
+                  stored rounded once to float32
+  fp8_quant_*     LU/cuda_fp8_utils.cu:27-44, 85-127         scale = max(absmax/448, 1/(448*512)), q = e4m3(clamp(x/scale))
+  fp8_gemm_*      KS/kernels/nvidia/kernel_wrapper.cpp:1033-1041  out = (sum_k a*w) * w_scale[n] * a_scale[m] in float64
+
+Run from the repository root:  python tests/golden/make_fixtures.py
+"""
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+AWQ_ORDER = [0, 2, 4, 6, 1, 3, 5, 7]
+
+
+def f16_bits(x):
+    return np.asarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
+
+
+def f16_value(b):
+    return b.view(np.float16).astype(np.float64)
+
+
+def bf16_bits(x):
+    """float32 -> bfloat16 bit pattern, round to nearest even (finite inputs)."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+
+def bf16_value(b):
+    return (b.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+def gptq_pack(u):
+    K, N = u.shape
+    q = np.zeros((K // 8, N), dtype=np.uint32)
+    for r in range(K // 8):
+        for j in range(8):
+            q[r] |= u[8 * r + j].astype(np.uint32) << np.uint32(4 * j)
+    return q.view(np.int32)
+
+
+def awq_pack(u):
+    K, N = u.shape
+    q = np.zeros((K, N // 8), dtype=np.uint32)
+    for c in range(N // 8):
+        for j in range(8):
+            q[:, c] |= u[:, 8 * c + AWQ_ORDER[j]].astype(np.uint32) << np.uint32(4 * j)
+    return q.view(np.int32)
+
+
+def rowmajor_pack(u):
+    s = (u.astype(np.int16) - 8) & 0xF
+    return (s[:, 0::2] | (s[:, 1::2] << 4)).astype(np.uint8).view(np.int8)
+
+
+def e4m3_table():
+    t = np.zeros(256, dtype=np.float64)
+    for c in range(256):
+        sign = -1.0 if c & 0x80 else 1.0
+        e, m = (c >> 3) & 0xF, c & 7
+        if e == 15 and m == 7:
+            t[c] = np.nan
+        elif e == 0:
+            t[c] = sign * m * 2.0 ** -9
+        else:
+            t[c] = sign * (1 + m / 8.0) * 2.0 ** (e - 7)
+    return t
+
+
+def e4m3_encode(x, table):
+    """Nearest representable value, ties to the even code, saturating at 448; x is float64 and already clamped."""
+    pos = table[:127]  # 0 .. 448, increasing
+    ax = np.abs(x)
+    hi = np.searchsorted(pos, ax, side="left").clip(1, 126)
+    lo = hi - 1
+    dlo, dhi = ax - pos[lo], pos[hi] - ax
+    pick_hi = (dhi < dlo) | ((dhi == dlo) & (hi % 2 == 0))
+    code = np.where(pick_hi, hi, lo).astype(np.uint8)
+    return code | np.where(np.signbit(x), 0x80, 0).astype(np.uint8)
+
+
+def w4a16_case(seed, M, K, N, g, awq, bf16):
+    rng = np.random.default_rng(seed)
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8) if awq else np.full((K // g, N), 8, dtype=np.uint8)
+    s = np.abs(rng.standard_normal((K // g, N))).astype(np.float32) * 0.02 + 1e-3
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    to_bits, to_val = (bf16_bits, bf16_value) if bf16 else (f16_bits, f16_value)
+    sb, ab = to_bits(s), to_bits(a)
+    w = (u.astype(np.float64) - np.repeat(z, g, axis=0)) * np.repeat(to_val(sb), g, axis=0)
+    out = to_val(ab) @ w
+    d = dict(u=u, scales_bits=sb, act_bits=ab, out=out.astype(np.float32), group=np.int64(g), bf16=np.int64(bf16))
+    if awq:
+        d.update(qweight=awq_pack(u), qzeros=awq_pack(z), z=z)
+    else:
+        d.update(qweight=gptq_pack(u))
+    return d
+
+
+def main():
+    rng = np.random.default_rng(20240607)
+    table = e4m3_table()
+
+    u = rng.integers(0, 16, size=(64, 64), dtype=np.uint8)
+    np.savez_compressed(os.path.join(HERE, "gptq_64x64.npz"), u=u, qweight=gptq_pack(u), rowmajor=rowmajor_pack(u))
+    u = rng.integers(0, 16, size=(128, 64), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(1, 64), dtype=np.uint8)
+    np.savez_compressed(os.path.join(HERE, "awq_128x64.npz"), u=u, qweight=awq_pack(u), z=z, qzeros=awq_pack(z),
+                        rowmajor=rowmajor_pack(u))
+    np.savez_compressed(os.path.join(HERE, "e4m3_table.npz"), value=table)
+
+    np.savez_compressed(os.path.join(HERE, "w4a16_gptq_f16_16x256x128.npz"), **w4a16_case(1, 16, 256, 128, 128, False, False))
+    np.savez_compressed(os.path.join(HERE, "w4a16_awq_f16_5x256x64_g64.npz"), **w4a16_case(2, 5, 256, 64, 64, True, False))
+    np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_16x384x128.npz"), **w4a16_case(3, 16, 384, 128, 128, True, True))
+    np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_130x256x272.npz"), **w4a16_case(4, 130, 256, 272, 128, True, True))
+
+    # FP8 activation quantisation, per token, fp16 input 8 x 256
+    x = (rng.standard_normal((8, 256)) * 0.7).astype(np.float32)
+    xb = f16_bits(x)
+    xv = f16_value(xb).astype(np.float32)
+    scale = np.maximum(np.abs(xv).max(axis=1) / np.float32(448.0), np.float32(1.0 / (448.0 * 512.0))).astype(np.float32)
+    ratio = np.clip((xv / scale[:, None]).astype(np.float32), -448.0, 448.0)
+    aq = e4m3_encode(ratio.astype(np.float64), table)
+    # FP8 weight 64 x 256 with per-channel scales, and the GEMM 8 x 256 x 64
+    wq = rng.integers(0, 256, size=(64, 256), dtype=np.uint8)
+    wq[(wq & 0x7F) == 0x7F] = 0x30
+    w_scale = (rng.random(64).astype(np.float32) * 0.01 + 1e-3).astype(np.float32)
+    out = (table[aq] @ table[wq].T) * w_scale.astype(np.float64)[None, :] * scale.astype(np.float64)[:, None]
+    np.savez_compressed(os.path.join(HERE, "fp8_8x256x64.npz"), x_bits=xb, a_scale=scale, aq=aq, wq=wq, w_scale=w_scale,
+                        out=out.astype(np.float32))
+
+
+if __name__ == "__main__":
+    main()
