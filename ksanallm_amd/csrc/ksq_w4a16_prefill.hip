@@ -172,20 +172,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   };
   BTile b0, b1;
 
-  auto load_a = [&](u32x4* buf, int kt) {  // k tile kt of the activations -> buf; past K the data is never used
+  // The loads of the next k tile are issued a few at a time between the matrix instructions of the current one
+  // (a burst of 16 memory instructions would hold the wave in the issue queue of the memory pipeline, and the
+  // matrix cores with it).  Part q = 0..3 of a tile's loads: two activation fragments (global -> LDS, no registers)
+  // and the weight fragment + scale/zero word of column tile q (past the last k tile the resources return zero).
+  auto load_part = [&](u32x4* buf, BTile& b, int kt, int q) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 2 * q; i < 2 * q + 2; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (8 * wave + i) * 64), 16, a_off[i >> 2],
                                                kt * 256 + (i & 3) * 64, 0, 0);
-  };
-  auto load_b = [&](BTile& b, int kt) {  // past the last k tile the resource returns zero
+    b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
 #pragma unroll
-    for (int t = 0; t < kNT; ++t) {
-      b.w[t] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[t], w_voff + kt * 1024u, 0, 0));
-#pragma unroll
-      for (int gi = 0; gi < GPT; ++gi)
-        b.sz[t][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[t], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
-    }
+    for (int gi = 0; gi < GPT; ++gi)
+      b.sz[q][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[q], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
   };
 
   uint32_t m_lo = Ops<_Float16>::kMaskLo, m_hi = Ops<_Float16>::kMaskHi, g_lo = Ops<_Float16>::kMagicLo,
@@ -195,7 +194,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   asm volatile("" : "+v"(g_hi));
   asm volatile("" : "+v"(m_hi));
 
-  auto compute = [&](const u32x4* buf, const BTile& bt) {
+  // Activation fragments are read from LDS four at a time (half of the row tiles of one 32-k step), one half ahead
+  // of the matrix instructions that use them, so that the LDS latency hides behind 16 MFMAs.
+  auto read_half = [&](u32x4 (&a)[4], const u32x4* buf, int ks, int h) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] = buf[((4 * h + i) * 4 + ks) * 64 + lane];
+  };
+  auto mfma_half = [&](const u32x4 (&a)[4], const u32x4 (&b)[kNT], int h) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int t = 0; t < kNT; ++t) acc[4 * h + i][t] = O::mfma(a[i], b[t], acc[4 * h + i][t]);
+  };
+  // One k tile.  On entry everything in flight (this tile's activations and weights) has landed and is visible to
+  // the whole workgroup, and every wave is done with the other buffer.
+  auto step = [&](const u32x4* cur, u32x4* nxt, const BTile& bt, BTile& bn, int kt) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 a0[4], a1[4];
+    read_half(a0, cur, 0, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       u32x4 b[kNT];
@@ -204,28 +222,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
         const typename DQ::Consts k = DQ::prepare(bt.sz[t][GPT == 2 ? (ks >> 1) : 0]);
         b[t] = DQ::run(bt.w[t][ks], k, m_lo, m_hi, g_lo, g_hi);
       }
-#pragma unroll
-      for (int mt = 0; mt < kMT; ++mt) {
-        const u32x4 af = buf[(mt * 4 + ks) * 64 + lane];
-#pragma unroll
-        for (int t = 0; t < kNT; ++t) acc[mt][t] = O::mfma(af, b[t], acc[mt][t]);
-      }
+      read_half(a1, cur, ks, 1);
+      if (ks < 2) load_part(nxt, bn, kt + 1, 2 * ks);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_half(a0, b, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks < 3) read_half(a0, cur, ks + 1, 0);
+      if (ks < 2) load_part(nxt, bn, kt + 1, 2 * ks + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_half(a1, b, 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // One k tile: everything in flight (this tile's activations and weights) has landed and is visible to the whole
-  // workgroup, and every wave is done with the other buffer; then the next tile's loads go out before the math.
-  auto step = [&](u32x4* cur, u32x4* nxt, const BTile& bc, BTile& bn, int kt) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    load_a(nxt, kt + 1);
-    load_b(bn, kt + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(cur, bc);
-  };
 
-  load_a(lds_a0, 0);
-  load_b(b0, 0);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) load_part(lds_a0, b0, 0, q);
   int kt = 0;
   for (; kt + 2 <= p.KT; kt += 2) {
     step(lds_a0, lds_a1, b0, b1, kt);
