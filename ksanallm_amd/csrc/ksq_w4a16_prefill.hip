@@ -176,15 +176,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   // (a burst of 16 memory instructions would hold the wave in the issue queue of the memory pipeline, and the
   // matrix cores with it).  Part q = 0..3 of a tile's loads: two activation fragments (global -> LDS, no registers)
   // and the weight fragment + scale/zero word of column tile q (past the last k tile the resources return zero).
-  auto load_part = [&](u32x4* buf, BTile& b, int kt, int q) {
-#pragma unroll
-    for (int i = 2 * q; i < 2 * q + 2; ++i)
+  auto load_item = [&](u32x4* buf, BTile& b, int kt, int q, int item) {
+    if (item < 2) {
+      const int i = 2 * q + item;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (8 * wave + i) * 64), 16, a_off[i >> 2],
                                                kt * 256 + (i & 3) * 64, 0, 0);
-    b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
+    } else if (item == 2) {
+      b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
+    } else {
 #pragma unroll
-    for (int gi = 0; gi < GPT; ++gi)
-      b.sz[q][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[q], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
+      for (int gi = 0; gi < GPT; ++gi)
+        b.sz[q][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[q], sz_voff + (kt * GPT + gi) * 64u, 0, 0);
+    }
+  };
+  auto load_part = [&](u32x4* buf, BTile& b, int kt, int q) {
+#pragma unroll
+    for (int item = 0; item < 4; ++item) load_item(buf, b, kt, q, item);
   };
 
   uint32_t m_lo = Ops<_Float16>::kMaskLo, m_hi = Ops<_Float16>::kMaskHi, g_lo = Ops<_Float16>::kMagicLo,
@@ -200,11 +207,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
     for (int i = 0; i < 4; ++i) a[i] = buf[((4 * h + i) * 4 + ks) * 64 + lane];
   };
-  auto mfma_half = [&](const u32x4 (&a)[4], const u32x4 (&b)[kNT], int h) {
+  auto mfma_row = [&](const u32x4& a, const u32x4 (&b)[kNT], int mt) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int t = 0; t < kNT; ++t) acc[4 * h + i][t] = O::mfma(a[i], b[t], acc[4 * h + i][t]);
+    for (int t = 0; t < kNT; ++t) acc[mt][t] = O::mfma(a, b[t], acc[mt][t]);
   };
   // One k tile.  On entry everything in flight (this tile's activations and weights) has landed and is visible to
   // the whole workgroup, and every wave is done with the other buffer.
@@ -223,15 +228,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
         b[t] = DQ::run(bt.w[t][ks], k, m_lo, m_hi, g_lo, g_hi);
       }
       read_half(a1, cur, ks, 1);
-      if (ks < 2) load_part(nxt, bn, kt + 1, 2 * ks);
       __builtin_amdgcn_sched_barrier(0);
-      mfma_half(a0, b, 0);
-      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mfma_row(a0[i], b, i);
+        if (ks < 2) load_item(nxt, bn, kt + 1, 2 * ks, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if (ks < 3) read_half(a0, cur, ks + 1, 0);
-      if (ks < 2) load_part(nxt, bn, kt + 1, 2 * ks + 1);
       __builtin_amdgcn_sched_barrier(0);
-      mfma_half(a1, b, 1);
-      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mfma_row(a1[i], b, 4 + i);
+        if (ks < 2) load_item(nxt, bn, kt + 1, 2 * ks + 1, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
 
