@@ -15,6 +15,8 @@
 // magnitude); the row factor 2^e is applied to the fp32 accumulators in the epilogue, and the bf16 group scales
 // are converted to fp16.
 // Workgroups are numbered so that those sharing a row block of the activations run on the same XCD (own L2).
+#include <cstdlib>
+
 #include "ksq_internal.h"
 #include "ksq_w4a16_ops.h"
 
@@ -35,7 +37,7 @@ struct PrefillArgs {
   int M, N, K, KT, G, ntiles, mblocks, nblocks, super_n;
 };
 
-constexpr int kBM = 128, kBNT = 16;  // rows and column tiles (of 16) per workgroup
+constexpr int kBM = 128;             // rows per workgroup
 constexpr int kMT = 8, kNT = 4;      // MFMA tiles per wave: 8 x 4
 
 template <typename T>
@@ -108,8 +110,11 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_kernel(const uint16_t* _
   }
 }
 
-template <typename T, int GPT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
+template <typename T, int GPT, int NW>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
+  static_assert(NW == 4 || NW == 8, "four or eight waves side by side");
+  constexpr int kFPW = 32 / NW;  // activation fragments of a stage that one wave brings in
+  constexpr int kSN = 32 / NW;   // column blocks per super-tile
   using O = Ops<_Float16>;  // the matrix cores run in fp16 for both element types
   using DQ = Dequant<T>;
   constexpr bool kBF16 = sizeof(T) == 2 && !__is_same(T, _Float16);
@@ -124,16 +129,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   const int c = lane & 15, j = lane >> 4;
 
   // Workgroup numbering.  Hardware hands consecutive workgroup ids to the 8 XCDs in turn; every XCD (own L2) gets a
-  // contiguous run of logical ids, and logical ids walk 8 x 8 super-tiles of (row block, column block) pairs, so the
-  // 64 workgroups resident on an XCD share 8 activation row blocks and 8 weight column blocks.
+  // contiguous run of logical ids, and logical ids walk super-tiles of 8 row blocks x kSN column blocks, so the
+  // workgroups resident on an XCD at one time (two per CU with four waves, one with eight) share 8 activation row
+  // blocks and 2048 weight columns.
   const int per_xcd = gridDim.x >> 3;
   const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int st = lid >> 6, r = lid & 63;
+  const int st = lid / (8 * kSN), r = lid - st * (8 * kSN);
   const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
-  const int mb = st_m * 8 + (r & 7), nb = st_n * 8 + (r >> 3);
+  const int mb = st_m * 8 + (r & 7), nb = st_n * kSN + (r >> 3);
   if (mb >= p.mblocks || nb >= p.nblocks) return;  // padding of partial super-tiles
   const int m0 = mb * kBM;
-  const int nt0 = nb * kBNT + wave * kNT;
+  const int nt0 = (nb * NW + wave) * kNT;
 
   __amdgpu_buffer_rsrc_t rs_w[kNT], rs_sz[kNT];
 #pragma unroll
@@ -148,13 +154,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   }
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
-  // Staging role of this wave: fragments f = 8 * wave + i of a stage, f = 4 * (row tile) + (32-k step); rows past M
-  // repeat row M - 1 (their results are never stored).  A fragment is 64 lanes x 16 bytes, lane (c, j) = row c,
-  // k = 8 j .. 8 j + 7 of the step, and goes from global memory straight into LDS at lane * 16.
-  unsigned a_off[2];
+  // Staging role of this wave: fragments f = kFPW * wave + i of a stage, f = 4 * (row tile) + (32-k step); rows
+  // past M repeat row M - 1 (their results are never stored).  A fragment is 64 lanes x 16 bytes, lane (c, j) =
+  // row c, k = 8 j .. 8 j + 7 of the step, and goes from global memory straight into LDS at lane * 16.
+  unsigned a_off[2] = {0u, 0u};  // kFPW / 4 of them in use
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    int row = m0 + 16 * (2 * wave + h) + c;
+  for (int h = 0; h < kFPW / 4; ++h) {
+    int row = m0 + 16 * (kFPW / 4 * wave + h) + c;
     row = row < p.M ? row : p.M - 1;
     a_off[h] = ((unsigned)row * p.K + 8 * j) * 2u;
   }
@@ -174,13 +180,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
 
   // The loads of the next k tile are issued a few at a time between the matrix instructions of the current one
   // (a burst of 16 memory instructions would hold the wave in the issue queue of the memory pipeline, and the
-  // matrix cores with it).  Part q = 0..3 of a tile's loads: two activation fragments (global -> LDS, no registers)
-  // and the weight fragment + scale/zero word of column tile q (past the last k tile the resources return zero).
+  // matrix cores with it).  Part q = 0..3 of a tile's loads, in four items: activation fragments (global -> LDS,
+  // no registers; two with four waves, one with eight), the weight fragment of column tile q, its scale/zero
+  // words (past the last k tile the resources return zero).
   auto load_item = [&](u32x4* buf, BTile& b, int kt, int q, int item) {
     if (item < 2) {
-      const int i = 2 * q + item;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (8 * wave + i) * 64), 16, a_off[i >> 2],
-                                               kt * 256 + (i & 3) * 64, 0, 0);
+      if (item < kFPW / 4) {
+        const int i = kFPW / 4 * q + item;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i >> 2],
+                                                 kt * 256 + (i & 3) * 64, 0, 0);
+      }
     } else if (item == 2) {
       b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
     } else {
@@ -258,7 +267,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   // ---- epilogue: transpose each 16-row slab through LDS so that every lane stores 16 contiguous bytes
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
   __syncthreads();
-  float* epi = reinterpret_cast<float*>(lds_a0) + wave * (16 * kEpiStride);  // 4352 B per wave
+  float* epi = reinterpret_cast<float*>(wave < 4 ? lds_a0 : lds_a1) + (wave & 3) * (16 * kEpiStride);  // 4352 B
   uint16_t* out = static_cast<uint16_t*>(p.out);
   const int ncol0 = nt0 * 16;
 #pragma unroll
@@ -283,6 +292,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
+}
+
+template <typename T>
+void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, hipStream_t s) {
+  if (gpt == 1 && nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 4>), grid, block, 0, s, a);
+  else if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 8>), grid, block, 0, s, a);
+  else if (nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 4>), grid, block, 0, s, a);
+  else hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 8>), grid, block, 0, s, a);
 }
 
 }  // namespace
@@ -316,15 +333,24 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   a.G = (int)(k / g);
   a.ntiles = (int)(n / kTileN);
   a.mblocks = (int)((m + kBM - 1) / kBM);
-  a.nblocks = (a.ntiles + kBNT - 1) / kBNT;
-  a.super_n = (a.nblocks + 7) / 8;
-  const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
+  // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; they are
+  // used when that still leaves at least one workgroup for every CU, otherwise four waves (128 x 256, two per CU).
+  const DeviceInfo* di = device_info();
+  KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
+  int nw = (size_t)a.mblocks * ((a.ntiles + 31) / 32) >= (size_t)di->cus ? 8 : 4;
+  if (const char* e = getenv("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v == 4 || v == 8) nw = v;
+  }
+  const int bnt = nw * kNT, sn = 32 / nw;
+  a.nblocks = (a.ntiles + bnt - 1) / bnt;
+  a.super_n = (a.nblocks + sn - 1) / sn;
+  const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * (8 * sn);  // whole super-tiles
   KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
-  dim3 grid((unsigned)total);
+  dim3 grid((unsigned)total), block(64 * nw);
   const int gpt = (int)(kTileK / g);
   if (dtype == KSQ_F16) {
-    if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<_Float16, 1>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((w4a16_prefill_kernel<_Float16, 2>), grid, dim3(256), 0, s, a);
+    launch_typed<_Float16>(a, gpt, nw, grid, block, s);
   } else {
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "bf16 prefill needs its workspace");
     uint16_t* a16 = static_cast<uint16_t*>(workspace);
@@ -333,8 +359,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
                        a16, row_scale, (int)k);
     a.act = a16;
     a.row_scale = row_scale;
-    if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<__bf16, 1>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((w4a16_prefill_kernel<__bf16, 2>), grid, dim3(256), 0, s, a);
+    launch_typed<__bf16>(a, gpt, nw, grid, block, s);
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;

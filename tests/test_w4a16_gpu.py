@@ -110,6 +110,24 @@ def test_forced_split_k_and_tile_widths(gpu, dtype, M, ksplit, nt, slices):
     assert np.array_equal(got1, got2), "split-K result must be deterministic and repeatable"
 
 
+@pytest.mark.parametrize("waves", [4, 8])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 128, 384, 528),    # odd number of k tiles, 33 column tiles: ragged in N for both widths
+    ("bf16", "awq", 128, 333, 512, 1040),  # ragged rows, three column blocks of 512
+    ("f16", "gptq", 64, 257, 256, 272),    # two groups per k tile
+    ("bf16", "gptq", 64, 130, 640, 512),
+])
+def test_prefill_kernel_widths(gpu, waves, dtype, kind, g, M, K, N):
+    """The large-M kernel in both workgroup widths (128 x 256 and 128 x 512), whichever the planner would pick."""
+    case = W4Case(1250 + waves + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    with _env(KSQ_W4_PREFILL_WAVES=waves):
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"prefill waves={waves} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+
+
 def test_no_workspace_still_correct(gpu):
     case = W4Case(1300, 16, 4096, 512, kind="gptq", dtype="f16")
     dev = W4Device(case, gpu)
