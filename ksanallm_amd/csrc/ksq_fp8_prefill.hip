@@ -2,11 +2,15 @@
 //
 // Workgroup tile 128 rows x 256 columns, four waves side by side, every wave 8 x 4 MFMA tiles of 16 x 16 with fp32
 // accumulators, K = 128 per instruction (v_mfma_f32_16x16x128_f8f6f4, both operands OCP e4m3, no block scaling).
-// Activations go through LDS in fragment order (one 128-row x 128-k stage = 16 KiB, double-buffered, one barrier per
-// stage); weights are read by each wave for its own 64 columns straight from the [N][K] tensor, one stage ahead.
+// Activations go from global memory straight into LDS in fragment order (one 128-row x 128-k stage = 16 KiB, four
+// stages in flight as four separate objects, loaded two stages ahead, one barrier per stage); weights are read by
+// each wave for its own 64 columns straight from the [N][K] tensor into registers, one stage ahead.  The loads of
+// the coming stages are issued one at a time between the matrix instructions.
 // Inside one instruction lane (r, j) holds bytes [16j, 16j+16) and [64+16j, 64+16j+16) of row r's 128-byte k
 // slice -- the same assignment on both operands, so the products pair up, and every 128-bit load of a 16-lane
-// group covers 64 contiguous bytes of a row.
+// group covers 64 contiguous bytes of a row.  K must be a multiple of 128 (other K take the streaming kernel).
+#include <cstdlib>
+
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -15,6 +19,7 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
 
 struct Fp8PrefillArgs {
   const uint8_t* aq;  // [M][K]
@@ -22,7 +27,7 @@ struct Fp8PrefillArgs {
   const float* a_scale;
   const float* w_scale;
   void* out;
-  int M, N, K, KS /* 128-byte k stages, rounded up */, mblocks, nblocks;
+  int M, N, K, KS /* 128-byte k stages */, mblocks, nblocks, super_n;
   int a_scale_per_row, w_scale_per_col;
 };
 
@@ -48,39 +53,47 @@ __device__ inline i32x8 join(u32x4 lo, u32x4 hi) {
 
 template <typename T>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void fp8_prefill_kernel(Fp8PrefillArgs p) {
-  constexpr int kStage = kMT * 2 * 64;  // 16-byte elements per activation stage
+  constexpr int kStage = kMT * 2 * 64;  // 16-byte elements per activation stage (16 KiB)
   constexpr int kEpiStride = 68;
-  __shared__ u32x4 lds[2 * kStage];
+  // four stages as four separate objects: loads into one are then known not to alias reads of another
+  __shared__ u32x4 lds0[kStage];
+  __shared__ u32x4 lds1[kStage];
+  __shared__ u32x4 lds2[kStage];
+  __shared__ u32x4 lds3[kStage];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, j = lane >> 4;
 
-  const int total = gridDim.x, per_xcd = total >> 3;
+  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn; every XCD (own L2) gets a contiguous run of
+  // logical ids, which walk 8 x 8 super-tiles of (row block, column block) pairs.
+  const int per_xcd = gridDim.x >> 3;
   const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int mb = lid / p.nblocks, nb = lid - mb * p.nblocks;
-  if (mb >= p.mblocks) return;
+  const int st = lid >> 6, rr0 = lid & 63;
+  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
+  const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 8 + (rr0 >> 3);
+  if (mb >= p.mblocks || nb >= p.nblocks) return;
   const int m0 = mb * kBM, n0 = nb * kBN + wave * (kNT * 16);
 
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_w =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.wq), 0, (int)((size_t)p.N * p.K), 0x00020000);
-  // activation staging role: fragments f = 4 * wave + i (row tile f >> 1, half f & 1), this lane's 16 bytes
-  unsigned a_off[4];
+  // Staging role of this wave: fragments f = 4 * wave + i (row tile f >> 1, half f & 1) of a stage, this lane's 16
+  // bytes; rows past M repeat row M - 1 (their results are never stored).
+  unsigned a_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int f = 4 * wave + i, mt = f >> 1, h = f & 1;
-    const int row = m0 + 16 * mt + r;
-    a_off[i] = row < p.M ? (unsigned)row * p.K + 64 * h + 16 * j : 0x80000000u;
+  for (int h = 0; h < 2; ++h) {
+    int row = m0 + 16 * (2 * wave + h) + r;
+    row = row < p.M ? row : p.M - 1;
+    a_off[h] = (unsigned)row * p.K + 16 * j;
   }
-  unsigned w_off[kNT];
+  unsigned w_off[kNT];  // rows past N read as zero
 #pragma unroll
   for (int t = 0; t < kNT; ++t) {
     const int row = n0 + 16 * t + r;
     w_off[t] = row < p.N ? (unsigned)row * p.K + 16 * j : 0x80000000u;
   }
-  // a 16-byte piece at k offset ko inside a row is valid iff ko + 16 <= K (K % 16 == 0); otherwise it reads zero
 
   f32x4 acc[kMT][kNT];
 #pragma unroll
@@ -88,66 +101,78 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
     for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  u32x4 a_reg[4];
-  u32x4 b_cur[kNT][2], b_nxt[kNT][2];
-  auto load_a = [&](int s) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const unsigned ko = (unsigned)s * 128u + 64u * ((4 * wave + i) & 1) + 16u * j;
-      a_reg[i] = __builtin_bit_cast(
-          u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                     rs_a, (ko + 16u <= (unsigned)p.K && a_off[i] != 0x80000000u) ? a_off[i] + s * 128u : 0x80000000u, 0,
-                     0));
-    }
+  struct BStage {
+    u32x4 w[kNT][2];
   };
-  auto write_a = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) lds[buf * kStage + (4 * wave + i) * 64 + lane] = a_reg[i];
+  BStage b0, b1;
+
+  // item i < 4: activation fragment 4 * wave + i of stage s -> buf (past K: inside the buffer or out of range, never
+  // used either way)
+  auto load_a_item = [&](u32x4* buf, int s, int i) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (4 * wave + i) * 64), 16, a_off[i >> 1],
+                                             s * 128 + (i & 1) * 64, 0, 0);
   };
-  auto load_b = [&](int s) {
-#pragma unroll
-    for (int t = 0; t < kNT; ++t)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const unsigned ko = (unsigned)s * 128u + 64u * h + 16u * j;
-        b_nxt[t][h] = __builtin_bit_cast(
-            u32x4,
-            __builtin_amdgcn_raw_buffer_load_b128(
-                rs_w, (ko + 16u <= (unsigned)p.K && w_off[t] != 0x80000000u) ? w_off[t] + s * 128u + 64u * h : 0x80000000u,
-                0, 0));
-      }
+  // item i < 8: weight piece (column tile i >> 1, half i & 1) of stage s; a stage past K is never used
+  auto load_b_item = [&](BStage& b, int s, int i) {
+    const int t = i >> 1, h = i & 1;
+    b.w[t][h] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_off[t] + s * 128u + 64u * h, 0, 0));
   };
-  auto compute = [&](int buf) {
-#pragma unroll
-    for (int mt = 0; mt < kMT; ++mt) {
-      const i32x8 af = join(lds[buf * kStage + (mt * 2 + 0) * 64 + lane], lds[buf * kStage + (mt * 2 + 1) * 64 + lane]);
-#pragma unroll
-      for (int t = 0; t < kNT; ++t)
-        acc[mt][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, join(b_cur[t][0], b_cur[t][1]), acc[mt][t], 0,
-                                                                      0, 0, 0, 0, 0);
-    }
+  auto read_a = [&](const u32x4* buf, int mt) {
+    return join(buf[(mt * 2 + 0) * 64 + lane], buf[(mt * 2 + 1) * 64 + lane]);
   };
 
-  load_b(0);
-  load_a(0);
-  write_a(0);
-  load_a(1);
-  for (int s = 0; s < p.KS; ++s) {
+  // One stage.  On entry all loads but the four newest (the activations of stage s + 1) have landed; after the
+  // barrier stage s is visible to every wave and every wave is done with the buffer that stage s + 2 goes into.
+  auto step = [&](const u32x4* cur, u32x4* dst, const BStage& bc, BStage& bn, int s) {
+    __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    i32x8 bf[kNT];
 #pragma unroll
-    for (int t = 0; t < kNT; ++t) {
-      b_cur[t][0] = b_nxt[t][0];
-      b_cur[t][1] = b_nxt[t][1];
+    for (int t = 0; t < kNT; ++t) bf[t] = join(bc.w[t][0], bc.w[t][1]);
+    i32x8 a_cur = read_a(cur, 0), a_nxt = read_a(cur, 1);
+#pragma unroll
+    for (int mt = 0; mt < kMT; ++mt) {
+      const i32x8 af = a_cur;
+      a_cur = a_nxt;
+      if (mt + 2 < kMT) a_nxt = read_a(cur, mt + 2);
+      load_b_item(bn, s + 1, mt);  // weights of the next stage first ...
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < kNT; ++t)
+        acc[mt][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf[t], acc[mt][t], 0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();        // stage s is visible; everyone has finished reading the other buffer
-    write_a((s + 1) & 1);   // stage s + 1
-    load_a(s + 2);
-    load_b(s + 1);
-    compute(s & 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_a_item(dst, s + 2, i);  // ... then the activations two stages ahead
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load_a_item(lds0, 0, i);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_b_item(b0, 0, i);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load_a_item(lds1, 1, i);
+  int s = 0;
+  for (; s + 4 <= p.KS; s += 4) {
+    step(lds0, lds2, b0, b1, s);
+    step(lds1, lds3, b1, b0, s + 1);
+    step(lds2, lds0, b0, b1, s + 2);
+    step(lds3, lds1, b1, b0, s + 3);
+  }
+  if (s < p.KS) {
+    step(lds0, lds2, b0, b1, s);
+    if (s + 1 < p.KS) {
+      step(lds1, lds3, b1, b0, s + 1);
+      if (s + 2 < p.KS) step(lds2, lds0, b0, b1, s + 2);
+    }
   }
 
   // ---- epilogue: scales, then a transpose through LDS so that every lane stores 16 contiguous bytes
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetches must not land on top of the transposes
   __syncthreads();
-  float* epi = reinterpret_cast<float*>(lds) + wave * (16 * kEpiStride);
+  float* epi = reinterpret_cast<float*>(wave == 0 ? lds0 : wave == 1 ? lds1 : wave == 2 ? lds2 : lds3);
   uint16_t* out = static_cast<uint16_t*>(p.out);
   float ws[kNT];
 #pragma unroll
@@ -176,10 +201,144 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
   }
 }
 
+
+// The same GEMM with a 256 x 256 workgroup tile: eight waves as 2 x 4, every wave 128 rows x 64 columns.  Both
+// operands go from global memory straight into LDS (one stage = 256 rows x 128 k of each = 64 KiB, two stages), so
+// each byte crosses the CU's vector memory path once per workgroup: 128 x 256 tiles need 46 B/clk per CU at the
+// matrix cores' FP8 rate, this one 32.  One workgroup per CU.
+template <typename T>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void fp8_prefill256_kernel(Fp8PrefillArgs p) {
+  constexpr int kHalf = 16 * 2 * 64;  // 16-byte elements of one operand of one stage (32 KiB)
+  constexpr int kEpiStride = 68;
+  __shared__ u32x4 lds_a0[kHalf];
+  __shared__ u32x4 lds_b0[kHalf];
+  __shared__ u32x4 lds_a1[kHalf];
+  __shared__ u32x4 lds_b1[kHalf];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int r = lane & 15, j = lane >> 4;
+
+  // super-tiles of 8 row blocks x 4 column blocks = the 32 workgroups resident on one XCD
+  const int per_xcd = gridDim.x >> 3;
+  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int st = lid >> 5, rr0 = lid & 31;
+  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
+  const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 4 + (rr0 >> 3);
+  if (mb >= p.mblocks || nb >= p.nblocks) return;
+  const int m0 = mb * 256, n0 = nb * 256;
+
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_w =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.wq), 0, (int)((size_t)p.N * p.K), 0x00020000);
+  // Staging role of this wave: fragments 4 * wave + i, i < 4, of each operand (16-row tile (4 wave + i) >> 1, half
+  // i & 1); rows past M / N repeat the last row (their results are never stored).
+  unsigned a_off[2], w_off[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    int row = m0 + 16 * (2 * wave + h) + r;
+    row = row < p.M ? row : p.M - 1;
+    a_off[h] = (unsigned)row * p.K + 16 * j;
+    int col = n0 + 16 * (2 * wave + h) + r;
+    col = col < p.N ? col : p.N - 1;
+    w_off[h] = (unsigned)col * p.K + 16 * j;
+  }
+
+  f32x4 acc[kMT][kNT];
+#pragma unroll
+  for (int mt = 0; mt < kMT; ++mt)
+#pragma unroll
+    for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // item i < 8 of a stage's loads: i < 4 activations, else weights
+  auto load_item = [&](u32x4* abuf, u32x4* bbuf, int s, int i) {
+    const int f = i & 3;
+    if (i < 4)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f >> 1],
+                                               s * 128 + (f & 1) * 64, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f >> 1],
+                                               s * 128 + (f & 1) * 64, 0, 0);
+  };
+  auto read_frag = [&](const u32x4* buf, int tile) {
+    return join(buf[(tile * 2 + 0) * 64 + lane], buf[(tile * 2 + 1) * 64 + lane]);
+  };
+
+  auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt, int s) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of stage s has landed
+    __builtin_amdgcn_s_barrier();        // ... everyone's has, and everyone is done with the other stage
+    __builtin_amdgcn_sched_barrier(0);
+    i32x8 bf[kNT];
+#pragma unroll
+    for (int t = 0; t < kNT; ++t) bf[t] = read_frag(bcur, 4 * wn + t);
+    i32x8 a_cur = read_frag(acur, 8 * wm + 0), a_nxt = read_frag(acur, 8 * wm + 1);
+#pragma unroll
+    for (int mt = 0; mt < kMT; ++mt) {
+      const i32x8 af = a_cur;
+      a_cur = a_nxt;
+      if (mt + 2 < kMT) a_nxt = read_frag(acur, 8 * wm + mt + 2);
+      if (mt < 4) {  // the next stage's loads go out in the first half, to have the second half to land
+        load_item(anxt, bnxt, s + 1, 2 * mt);
+        load_item(anxt, bnxt, s + 1, 2 * mt + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < kNT; ++t)
+        acc[mt][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af, bf[t], acc[mt][t], 0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_item(lds_a0, lds_b0, 0, i);
+  int s = 0;
+  for (; s + 2 <= p.KS; s += 2) {
+    step(lds_a0, lds_b0, lds_a1, lds_b1, s);
+    step(lds_a1, lds_b1, lds_a0, lds_b0, s + 1);
+  }
+  if (s < p.KS) step(lds_a0, lds_b0, lds_a1, lds_b1, s);
+
+  // ---- epilogue: scales, then a transpose through LDS so that every lane stores 16 contiguous bytes
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
+  __syncthreads();
+  float* epi = reinterpret_cast<float*>(wm == 0 ? lds_a0 : lds_a1) + wn * (16 * kEpiStride);
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int mw = m0 + 128 * wm, nw = n0 + 64 * wn;
+  float ws[kNT];
+#pragma unroll
+  for (int t = 0; t < kNT; ++t) {
+    const int col = nw + 16 * t + r;
+    ws[t] = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
+  }
+#pragma unroll
+  for (int mt = 0; mt < kMT; ++mt) {
+#pragma unroll
+    for (int t = 0; t < kNT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) epi[(4 * j + i) * kEpiStride + 16 * t + r] = acc[mt][t][i] * ws[t];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
+      const float* src = epi + rr * kEpiStride + cc;
+      const int row = mw + 16 * mt + rr, col = nw + cc;
+      const float as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
+      u32x4 packed;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        packed[q] = (uint32_t)out_bits<T>(src[2 * q] * as) | ((uint32_t)out_bits<T>(src[2 * q + 1] * as) << 16);
+      if (row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+}
+
 }  // namespace
 
 bool fp8_prefill_supported(size_t m, size_t n, size_t k) {
-  return m >= 128 && n % 8 == 0 && k % 16 == 0 && m * k < 0x7FFFFF00ull && n * k < 0x7FFFFF00ull;
+  return m >= 128 && n % 8 == 0 && k % 128 == 0 && m * k < 0x7FFFFF00ull && n * k < 0x7FFFFF00ull;
 }
 
 int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
@@ -195,15 +354,38 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
   a.M = (int)m;
   a.N = (int)n;
   a.K = (int)k;
-  a.KS = (int)((k + 127) / 128);
-  a.mblocks = (int)((m + kBM - 1) / kBM);
-  a.nblocks = (int)((n + kBN - 1) / kBN);
+  a.KS = (int)(k / 128);
   a.a_scale_per_row = act_scale_count > 1;
   a.w_scale_per_col = w_scale_count > 1;
-  const size_t total = ((size_t)a.mblocks * a.nblocks + 7) / 8 * 8;
-  KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
-  if (out_dtype == KSQ_F16) hipLaunchKernelGGL(fp8_prefill_kernel<_Float16>, dim3((unsigned)total), dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(fp8_prefill_kernel<__bf16>, dim3((unsigned)total), dim3(256), 0, s, a);
+  // 256 x 256 tiles (one workgroup per CU) when they still cover every CU, else 128 x 256 (two per CU)
+  const DeviceInfo* di = device_info();
+  KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
+  int tile = ((m + 255) / 256) * ((n + 255) / 256) >= (size_t)di->cus ? 256 : 128;
+  if (const char* e = getenv("KSQ_FP8_PREFILL_TILE")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v == 128 || v == 256) tile = v;
+  }
+  if (tile == 256) {
+    a.mblocks = (int)((m + 255) / 256);
+    a.nblocks = (int)((n + 255) / 256);
+    a.super_n = (a.nblocks + 3) / 4;
+    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 32;  // whole 8 x 4 super-tiles
+    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    if (out_dtype == KSQ_F16)
+      hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, dim3((unsigned)total), dim3(512), 0, s, a);
+    else
+      hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, dim3((unsigned)total), dim3(512), 0, s, a);
+  } else {
+    a.mblocks = (int)((m + kBM - 1) / kBM);
+    a.nblocks = (int)((n + kBN - 1) / kBN);
+    a.super_n = (a.nblocks + 7) / 8;
+    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
+    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    if (out_dtype == KSQ_F16)
+      hipLaunchKernelGGL(fp8_prefill_kernel<_Float16>, dim3((unsigned)total), dim3(256), 0, s, a);
+    else
+      hipLaunchKernelGGL(fp8_prefill_kernel<__bf16>, dim3((unsigned)total), dim3(256), 0, s, a);
+  }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

@@ -185,12 +185,33 @@ def test_gemm_per_tensor_scales_and_ragged_shapes(gpu):
 
 @pytest.mark.parametrize("M,K,N", [(128, 1024, 256), (300, 1008, 264), (257, 2048, 520)])
 def test_gemm_large_m_ragged(gpu, M, K, N):
-    """M >= 128 takes the MFMA-tiled kernel: ragged M, K not a multiple of the 128-byte stage, N not of the tile."""
+    """M >= 128: ragged M and N through the MFMA-tiled kernel; K not a multiple of 128 through the streaming kernel."""
     xq, xs, wq, ws = _fp8_case(410 + M, M, K, N)
     got = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
     orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"fp8 large M={M} K={K} N={N}")
     got1 = _run_gemm(gpu, xq, xs[:1].copy(), wq, ws[:1].copy(), "f16")
     orc.assert_parity(got1, orc.fp8_gemm(xq, xs[:1].copy(), wq, ws[:1].copy()), f"fp8 large per-tensor M={M}")
+
+
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("M,K,N", [(300, 1024, 264), (257, 2048, 520), (512, 384, 768), (128, 128, 256)])
+def test_gemm_large_m_both_tiles(gpu, tile, M, K, N):
+    """The MFMA-tiled kernel in both workgroup tiles (128 x 256 and 256 x 256), whichever the planner would pick."""
+    import os
+
+    xq, xs, wq, ws = _fp8_case(430 + M, M, K, N)
+    old = os.environ.get("KSQ_FP8_PREFILL_TILE")
+    os.environ["KSQ_FP8_PREFILL_TILE"] = str(tile)
+    try:
+        got = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+        got2 = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+    finally:
+        if old is None:
+            os.environ.pop("KSQ_FP8_PREFILL_TILE", None)
+        else:
+            os.environ["KSQ_FP8_PREFILL_TILE"] = old
+    orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"fp8 tile={tile} M={M} K={K} N={N}")
+    assert np.array_equal(got, got2)
 
 
 def test_gemm_large_m_small_integers_exact(gpu):
