@@ -1,4 +1,6 @@
 // FP8 e4m3 (OCP) path: activation quantisation, rescale, on-the-fly weight conversion and the streaming GEMM.
+#include <cstdlib>
+
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -98,6 +100,129 @@ __global__ __launch_bounds__(256) void quantize_per_token_kernel(const uint16_t*
   const float s = fmaxf(mx / kE4m3Max, kMinScale);
   if (threadIdx.x == 0) scale[row] = s;
   for (size_t i = threadIdx.x; i < k; i += 256) qr[i] = quantize_one(load_as_float<T>(xr, i), s);
+}
+
+// ---- vector forms (k a multiple of 8, 16-byte aligned rows): eight elements per lane and access
+template <typename T>
+__device__ inline void unpack8(u32x4 v, float (&f)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (__is_same(T, _Float16)) {
+      f[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[i] & 0xFFFFu));
+      f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[i] >> 16));
+    } else {
+      f[2 * i] = __builtin_bit_cast(float, v[i] << 16);
+      f[2 * i + 1] = __builtin_bit_cast(float, v[i] & 0xFFFF0000u);
+    }
+  }
+}
+
+__device__ inline float absmax8(const float (&f)[8], float mx) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) mx = fmaxf(mx, fabsf(f[i]));
+  return mx;
+}
+
+__device__ inline u32x2 quantize8(const float (&f)[8], float scale) {
+  float c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c[i] = fminf(fmaxf(f[i] / scale, -kE4m3Max), kE4m3Max);
+  int lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], lo, true);
+  int hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[4], c[5], 0, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[6], c[7], hi, true);
+  return u32x2{(uint32_t)lo, (uint32_t)hi};
+}
+
+template <int THREADS>
+__device__ inline float block_max(float v, float* smem) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float m = smem[0];
+#pragma unroll
+  for (int w = 1; w < THREADS / 64; ++w) m = fmaxf(m, smem[w]);
+  return m;
+}
+
+// One workgroup per row; the row stays in registers between the abs-max pass and the quantisation (R chunks of
+// eight elements per lane), so it is read once.  Serves per-token rows and, with a single row, small whole tensors.
+template <typename T, int THREADS, int R>
+__global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const uint16_t* x, size_t k, uint8_t* q,
+                                                                    float* scale) {
+  __shared__ float smem[THREADS / 64];
+  const size_t row = blockIdx.x;
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * k);
+  u32x2* qr = reinterpret_cast<u32x2*>(q + row * k);
+  const unsigned nchunks = (unsigned)(k / 8);
+  u32x4 v[R];
+  float mx = 0.0f;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const unsigned c = threadIdx.x + i * THREADS;
+    v[i] = c < nchunks ? xr[c] : u32x4{0u, 0u, 0u, 0u};
+    float f[8];
+    unpack8<T>(v[i], f);
+    mx = absmax8(f, mx);
+  }
+  mx = block_max<THREADS>(mx, smem);
+  const float s = fmaxf(mx / kE4m3Max, kMinScale);
+  if (threadIdx.x == 0) scale[row] = s;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const unsigned c = threadIdx.x + i * THREADS;
+    float f[8];
+    unpack8<T>(v[i], f);
+    if (c < nchunks) qr[c] = quantize8(f, s);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void absmax_scale_vec_kernel(const u32x4* x, size_t nchunks, float* scale) {
+  __shared__ float smem[4];
+  float mx = 0.0f;
+  for (size_t c = (size_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * 256) {
+    float f[8];
+    unpack8<T>(x[c], f);
+    mx = absmax8(f, mx);
+  }
+  mx = block_max<256>(mx, smem);
+  if (threadIdx.x == 0) {
+    float s = fmaxf(mx / kE4m3Max, kMinScale);
+    atomicMax(reinterpret_cast<unsigned int*>(scale), __builtin_bit_cast(unsigned int, s));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_vec_kernel(const u32x4* x, const float* scale, size_t nchunks,
+                                                           u32x2* q) {
+  const float s = scale[0];
+  for (size_t c = (size_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (size_t)gridDim.x * 256) {
+    float f[8];
+    unpack8<T>(x[c], f);
+    q[c] = quantize8(f, s);
+  }
+}
+
+template <typename T>
+bool launch_rows_vec(const uint16_t* x, size_t rows, size_t k, uint8_t* q, float* scale, hipStream_t s) {
+  if (k % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(q) & 7) != 0) return false;
+  const size_t nchunks = k / 8;
+  dim3 grid((unsigned)rows);
+  // few rows: spread a row over 1024 lanes; many rows: 256 lanes per row keep more rows in flight
+  if (rows > 64 && nchunks <= 256 * 4) {
+    if (nchunks <= 256) hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 256, 1>), grid, dim3(256), 0, s, x, k, q, scale);
+    else if (nchunks <= 512) hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 256, 2>), grid, dim3(256), 0, s, x, k, q, scale);
+    else hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 256, 4>), grid, dim3(256), 0, s, x, k, q, scale);
+    return true;
+  }
+  if (nchunks > 1024 * 8) return false;
+  if (nchunks <= 1024) hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 1024, 1>), grid, dim3(1024), 0, s, x, k, q, scale);
+  else if (nchunks <= 2048) hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 1024, 2>), grid, dim3(1024), 0, s, x, k, q, scale);
+  else if (nchunks <= 4096) hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 1024, 4>), grid, dim3(1024), 0, s, x, k, q, scale);
+  else hipLaunchKernelGGL((quantize_rows_vec_kernel<T, 1024, 8>), grid, dim3(1024), 0, s, x, k, q, scale);
+  return true;
 }
 
 __device__ inline float e4m3_to_float(uint8_t c) {
@@ -294,20 +419,45 @@ int ksq_fp8_quantize(int dtype, const void* act, size_t m, size_t k, int mode, v
   const bool f16 = dtype == KSQ_F16;
   if (mode == KSQ_FP8_PER_TOKEN_DYNAMIC) {
     KSQ_REQUIRE(m < (1ull << 31), KSQ_ERR_UNSUPPORTED, "m too large");
-    if (f16) hipLaunchKernelGGL(quantize_per_token_kernel<_Float16>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
-    else hipLaunchKernelGGL(quantize_per_token_kernel<__bf16>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
+    const bool done = f16 ? launch_rows_vec<_Float16>(x, m, k, q, act_scale, s) : launch_rows_vec<__bf16>(x, m, k, q, act_scale, s);
+    if (!done) {
+      if (f16) hipLaunchKernelGGL(quantize_per_token_kernel<_Float16>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
+      else hipLaunchKernelGGL(quantize_per_token_kernel<__bf16>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
+    }
   } else {
     const size_t count = m * k;
+    const bool vec = count % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(q) & 7) == 0;
+    // a small tensor is one row of one workgroup: abs-max and quantisation in a single launch
+    if (mode == KSQ_FP8_PER_TENSOR_DYNAMIC && vec && count <= 65536 &&
+        (f16 ? launch_rows_vec<_Float16>(x, 1, count, q, act_scale, s) : launch_rows_vec<__bf16>(x, 1, count, q, act_scale, s))) {
+      KSQ_HIP_TRY(hipGetLastError());
+      return KSQ_OK;
+    }
     if (mode == KSQ_FP8_PER_TENSOR_DYNAMIC) {
       // a fill kernel rather than a memset node keeps the call safe to record into a HIP graph
       hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, act_scale, 1);
-      const unsigned nb = blocks_for(count, 2048);
-      if (f16) hipLaunchKernelGGL(absmax_scale_kernel<_Float16>, dim3(nb), dim3(256), 0, s, x, count, act_scale);
-      else hipLaunchKernelGGL(absmax_scale_kernel<__bf16>, dim3(nb), dim3(256), 0, s, x, count, act_scale);
+      if (vec) {
+        const unsigned nb = blocks_for(count / 8, 1024);
+        const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+        if (f16) hipLaunchKernelGGL(absmax_scale_vec_kernel<_Float16>, dim3(nb), dim3(256), 0, s, xv, count / 8, act_scale);
+        else hipLaunchKernelGGL(absmax_scale_vec_kernel<__bf16>, dim3(nb), dim3(256), 0, s, xv, count / 8, act_scale);
+      } else {
+        const unsigned nb = blocks_for(count, 2048);
+        if (f16) hipLaunchKernelGGL(absmax_scale_kernel<_Float16>, dim3(nb), dim3(256), 0, s, x, count, act_scale);
+        else hipLaunchKernelGGL(absmax_scale_kernel<__bf16>, dim3(nb), dim3(256), 0, s, x, count, act_scale);
+      }
     }
-    const unsigned nb = blocks_for(count, 4096);
-    if (f16) hipLaunchKernelGGL(quantize_kernel<_Float16>, dim3(nb, 1), dim3(256), 0, s, x, act_scale, (size_t)1, count, q);
-    else hipLaunchKernelGGL(quantize_kernel<__bf16>, dim3(nb, 1), dim3(256), 0, s, x, act_scale, (size_t)1, count, q);
+    if (vec) {
+      const unsigned nb = blocks_for(count / 8, 1024);
+      const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+      u32x2* qv = reinterpret_cast<u32x2*>(q);
+      if (f16) hipLaunchKernelGGL(quantize_vec_kernel<_Float16>, dim3(nb), dim3(256), 0, s, xv, act_scale, count / 8, qv);
+      else hipLaunchKernelGGL(quantize_vec_kernel<__bf16>, dim3(nb), dim3(256), 0, s, xv, act_scale, count / 8, qv);
+    } else {
+      const unsigned nb = blocks_for(count, 4096);
+      if (f16) hipLaunchKernelGGL(quantize_kernel<_Float16>, dim3(nb, 1), dim3(256), 0, s, x, act_scale, (size_t)1, count, q);
+      else hipLaunchKernelGGL(quantize_kernel<__bf16>, dim3(nb, 1), dim3(256), 0, s, x, act_scale, (size_t)1, count, q);
+    }
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
@@ -367,6 +517,8 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     if (mm - 15 > max_m) break;
     Fp8Plan p = fp8_plan(mm, n, k, cus, (size_t)-1);
     if (p.partial_bytes > best) best = p.partial_bytes;
+    const Fp8KstatPlan kp = fp8_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
+    if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   }
   *bytes = best;
   return KSQ_OK;
@@ -395,6 +547,15 @@ int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_s
     return fp8_launch_prefill(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
                               static_cast<hipStream_t>(stream));
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
+  if (m <= 64) {
+    const char* e = getenv("KSQ_FP8_KSTAT");  // tuning / test switch: 0 sends small m to the streaming kernel
+    if (!(e && atoi(e) == 0)) {
+      const Fp8KstatPlan kp = fp8_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
+      if (kp.ok)
+        return fp8_launch_kstat(out_dtype, kp, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m,
+                                n, k, workspace, static_cast<hipStream_t>(stream));
+    }
+  }
   Fp8Plan plan = fp8_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
   Fp8Args a{};
   a.aq = static_cast<const uint8_t*>(act_q);

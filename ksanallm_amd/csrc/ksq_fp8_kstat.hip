@@ -1,0 +1,298 @@
+// FP8 e4m3 GEMM for M <= 64 (HBM-bound): k-stationary.
+//
+// A workgroup is 16 waves (8 for more than two row tiles: twice the registers each).  Wave w keeps the activation fragments of its own TPW k stages (128 bytes of k each)
+// for all MT row tiles in registers for the whole kernel and streams the weight rows of the workgroup's column
+// range, for its own stages only, straight from HBM into a register ring, one batch of NB column tiles ahead.
+// Nothing is re-read.  After every batch the 16 partial tiles of a (column tile, row tile) -- one per wave = per k
+// slice -- are summed through LDS in a fixed order.  K beyond waves x TPW stages is split over grid.y and finished by
+// the last-arriving workgroup through the workspace (partials in split order: deterministic).
+//
+// v_mfma_f32_16x16x128_f8f6f4 with both operands OCP e4m3 and no block scaling: lane (r, j) holds bytes
+// [16j, 16j+16) and [64+16j, 64+16j+16) of row r's 128-byte stage, on both operands.  Pieces past K read as zero on
+// both sides (K is a multiple of 16).  out = T(acc * w_scale[n] * a_scale[m]).
+#include <cstdlib>
+
+#include "ksq_internal.h"
+
+namespace ksq {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+struct Fp8KstatArgs {
+  const uint8_t* aq;  // [M][K]
+  const uint8_t* wq;  // [N][K]
+  const float* a_scale;
+  const float* w_scale;
+  void* out;           // [M][N] T
+  f32x4* partial;      // [ksplit][ntiles][MT][64]
+  unsigned* counters;  // [ntiles][MT]
+  int M, N, K, KS /* stages, rounded up */, ntiles, ksplit, nt_per_wg;
+  int a_scale_per_row, w_scale_per_col;
+};
+
+template <typename T>
+__device__ inline uint16_t out_bits(float v);
+template <>
+__device__ inline uint16_t out_bits<_Float16>(float v) {
+  return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+template <>
+__device__ inline uint16_t out_bits<__bf16>(float v) {
+  return __builtin_bit_cast(uint16_t, (__bf16)v);
+}
+
+__device__ inline i32x8 join(u32x4 lo, u32x4 hi) {
+  i32x8 v;
+  v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+  v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+  return v;
+}
+
+template <typename T, int MT, int TPW, int NB, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4))) void fp8_kstat_kernel(Fp8KstatArgs p) {
+  constexpr int D = NB * TPW;  // ring depth = one batch
+  static_assert(NB * MT * NW <= 64 && NB * MT <= NW, "two reduction buffers of at most 64 KiB, one tile per wave");
+  __shared__ f32x4 red[2 * NB * MT * NW * 64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, j = lane >> 4;
+  const int split = blockIdx.y;
+  const int wg_begin = (int)(((long)p.KS * split) / p.ksplit);
+  const int wg_end = (int)(((long)p.KS * (split + 1)) / p.ksplit);
+  const int s0 = wg_begin + wave * TPW;  // first stage of this wave
+  const int nt_begin = blockIdx.x * p.nt_per_wg;
+  int count = p.ntiles - nt_begin;
+  count = count < p.nt_per_wg ? count : p.nt_per_wg;
+  const int nbatches = (p.nt_per_wg + NB - 1) / NB;  // same for every workgroup
+
+  // The weight resource covers exactly the rows of this workgroup's column tiles (clipped to N): column tiles
+  // past the range and rows past N read as zero without touching memory.
+  int rows = count * 16;
+  if (nt_begin * 16 + rows > p.N) rows = p.N - nt_begin * 16;
+  if (rows < 0) rows = 0;
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(p.wq) + (size_t)nt_begin * 16 * p.K, 0, (int)((size_t)rows * p.K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
+  // per stage and half: offset of this lane's 16 bytes inside its row, or out of range (stage past the split's end,
+  // piece past K)
+  unsigned k_off[TPW][2];
+#pragma unroll
+  for (int t = 0; t < TPW; ++t)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const unsigned kb = (unsigned)(s0 + t) * 128u + 64u * h + 16u * j;
+      k_off[t][h] = (s0 + t < wg_end && kb + 16u <= (unsigned)p.K) ? kb : 0x80000000u;
+    }
+  // offset of this lane's piece of (stage t, half h) inside column tile 0; a parked offset stays out of range for
+  // every column tile (the range of one workgroup is below 2^30 bytes)
+  unsigned w_off[TPW][2];
+#pragma unroll
+  for (int t = 0; t < TPW; ++t)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) w_off[t][h] = k_off[t][h] + (unsigned)r * p.K;
+  const unsigned w_stride = 16u * (unsigned)p.K;
+
+  // activation fragments of this wave's stages: registers for the whole kernel
+  i32x8 af[MT][TPW];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+      const int row = 16 * mt + r;
+      u32x4 piece[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const unsigned ao = (row < p.M && k_off[t][h] != 0x80000000u) ? (unsigned)row * p.K + k_off[t][h] : 0x80000000u;
+        piece[h] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+      }
+      af[mt][t] = join(piece[0], piece[1]);
+    }
+
+  u32x4 wq[D][2];
+  auto fetch = [&](int slot, int i /* column tile inside the workgroup */, int t) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      wq[slot][h] = __builtin_bit_cast(
+          u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_off[t][h] + i * w_stride, 0, 2));
+  };
+
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int q = 0; q < D; ++q) {
+    fetch(q, q / TPW, q % TPW);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  for (int b = 0; b < nbatches; ++b) {
+    f32x4 accb[NB][MT];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) accb[i][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) {
+        const int slot = i * TPW + t;
+        const i32x8 bw = join(wq[slot][0], wq[slot][1]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          accb[i][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt][t], bw, accb[i][mt], 0, 0, 0, 0, 0, 0);
+        fetch(slot, (b + 1) * NB + i, t);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- sum the k slices of every tile of the batch (fixed order: deterministic).  The reduction buffer is
+    // double-buffered, so one barrier per batch is enough: whoever writes buffer b & 1 again (batch b + 2) has passed
+    // the barrier of batch b + 1, which the readers of batch b reach only after their reads.
+    f32x4* rb = red + (b & 1) * (NB * MT * NW * 64);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) rb[((i * MT + mt) * NW + wave) * 64 + lane] = accb[i][mt];
+    __syncthreads();
+    if (wave < NB * MT) {  // one (column tile, row tile) per wave
+      const int i = wave / MT, mt = wave - i * MT;
+      const int nt = nt_begin + b * NB + i;
+      const bool valid = b * NB + i < count && 16 * mt < p.M;
+      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w4 = 0; w4 < NW; w4 += 4) {  // four slices at a time: the weight ring is live in registers here
+#pragma unroll
+        for (int ww = w4; ww < w4 + 4; ++ww) sum += rb[(wave * NW + ww) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      bool store = valid;
+      if (p.ksplit > 1 && valid) {
+        // split across workgroups: park the fp32 tile, the last split to arrive adds them in split order
+        const size_t stride = (size_t)p.ntiles * MT * 64;
+        const size_t tile = ((size_t)nt * MT + mt) * 64 + lane;
+        store_agent(p.partial + (size_t)split * stride + tile, sum);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned* counter = p.counters + nt * MT + mt;
+        unsigned arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        store = arrived == (unsigned)(p.ksplit - 1);
+        if (store) {
+          asm volatile("" ::: "memory");
+          sum = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + (size_t)sp * stride + tile);
+          if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      if (store) {
+        const int col = nt * 16 + r;
+        if (col < p.N) {
+          const float ws = p.w_scale[p.w_scale_per_col ? col : 0];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int row = 16 * mt + 4 * j + e;
+            if (row < p.M) {
+              const float as = p.a_scale[p.a_scale_per_row ? row : 0];
+              out[(size_t)row * p.N + col] = out_bits<T>(sum[e] * ws * as);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+void launch(int mt, int tpw, int nb, const Fp8KstatArgs& a, dim3 grid, hipStream_t s) {
+  if (mt == 1) {
+    const dim3 block(1024);
+    if (tpw == 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 4, 2, 16>), grid, block, 0, s, a);
+    else if (tpw == 2 && nb >= 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 2, 4, 16>), grid, block, 0, s, a);
+    else if (tpw == 2) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 2, 2, 16>), grid, block, 0, s, a);
+    else if (nb >= 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 1, 4, 16>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 1, 2, 16>), grid, block, 0, s, a);
+  } else if (mt == 2) {
+    const dim3 block(1024);
+    if (tpw == 2) hipLaunchKernelGGL((fp8_kstat_kernel<T, 2, 2, 2, 16>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fp8_kstat_kernel<T, 2, 1, 2, 16>), grid, block, 0, s, a);
+  } else {
+    const dim3 block(512);
+    if (tpw == 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 4, 4, 2, 8>), grid, block, 0, s, a);
+    else if (tpw == 2) hipLaunchKernelGGL((fp8_kstat_kernel<T, 4, 2, 2, 8>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fp8_kstat_kernel<T, 4, 1, 2, 8>), grid, block, 0, s, a);
+  }
+}
+
+}  // namespace
+
+// Plan: row tiles (1, 2 or 4), waves per workgroup (8 with four row tiles, else 16), stages per wave (1, 2 or 4; at
+// most 2 with two row tiles: the activations of waves x TPW stages live in registers), split count, column tiles
+// per workgroup and per batch.
+Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  Fp8KstatPlan p{};
+  const size_t ntiles = (n + 15) / 16, stages = (k + 127) / 128;
+  p.ok = m >= 1 && m <= 64 && ntiles * 4 <= (size_t)kCountersPerSlot && m * k < 0x7FFFFF00ull;
+  if (!p.ok) return p;
+  p.mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
+  const size_t nw = p.mt == 4 ? 8 : 16;
+  const size_t cap = nw * (p.mt == 2 ? 2u : 4u);
+  size_t ksplit = (stages + cap - 1) / cap;
+  if (const char* e = getenv("KSQ_FP8_KSPLIT")) {  // tuning / test override; never below what the registers need
+    const size_t v = (size_t)atoi(e);
+    if (v > ksplit && v <= stages) ksplit = v;
+  }
+  auto need = [&](size_t ks) { return ks <= 1 ? (size_t)0 : ks * ntiles * p.mt * 64 * 16; };
+  if (need(ksplit) > workspace_bytes) {
+    p.ok = false;
+    return p;
+  }
+  const size_t per_split = (stages + ksplit - 1) / ksplit;
+  const size_t tpw = (per_split + nw - 1) / nw;
+  p.tpw = tpw <= 1 ? 1 : (tpw <= 2 ? 2 : 4);
+  p.ksplit = (int)ksplit;
+  size_t wgs = (size_t)cus / ksplit;
+  if (wgs < 1) wgs = 1;
+  if (wgs > ntiles) wgs = ntiles;
+  p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
+  p.grid_x = (int)((ntiles + p.nt_per_wg - 1) / p.nt_per_wg);
+  p.nb = (p.mt >= 2 || p.tpw == 4 || p.nt_per_wg < 3) ? 2 : 4;
+  p.partial_bytes = need(ksplit);
+  return p;
+}
+
+int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const void* act_q, const float* act_scale,
+                     size_t act_scale_count, const void* w_q, const float* w_scale, size_t w_scale_count, size_t m,
+                     size_t n, size_t k, void* workspace, hipStream_t s) {
+  KSQ_REQUIRE(((size_t)plan.nt_per_wg + 8) * 16 * k < 0x3FFFFF00ull, KSQ_ERR_UNSUPPORTED,
+              "column range of one workgroup larger than 1 GiB");
+  Fp8KstatArgs a{};
+  a.aq = static_cast<const uint8_t*>(act_q);
+  a.wq = static_cast<const uint8_t*>(w_q);
+  a.a_scale = act_scale;
+  a.w_scale = w_scale;
+  a.out = out;
+  a.partial = static_cast<f32x4*>(workspace);
+  a.M = (int)m;
+  a.N = (int)n;
+  a.K = (int)k;
+  a.KS = (int)((k + 127) / 128);
+  a.ntiles = (int)((n + 15) / 16);
+  a.ksplit = plan.ksplit;
+  a.nt_per_wg = plan.nt_per_wg;
+  a.a_scale_per_row = act_scale_count > 1;
+  a.w_scale_per_col = w_scale_count > 1;
+  a.counters = nullptr;
+  if (plan.ksplit > 1) {
+    KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
+    a.counters = counter_slot_device_ptr();
+    if (!a.counters) return KSQ_ERR_HIP;
+  }
+  dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
+  if (out_dtype == KSQ_F16) launch<_Float16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
+  else launch<__bf16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+}  // namespace ksq

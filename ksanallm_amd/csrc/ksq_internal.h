@@ -62,7 +62,7 @@ __host__ __device__ inline int frag_nibble_of(int e) { return (e & 1) ? 4 + (e >
 // kCounterSlots regions so that calls in flight on different streams do not share counters unless more than
 // kCounterSlots overlap.
 constexpr int kCounterSlots = 16;
-constexpr int kCountersPerSlot = 4096;
+constexpr int kCountersPerSlot = 16384;
 unsigned* counter_slot_device_ptr();  // next slot (device address), or nullptr on failure
 
 #if defined(__HIPCC__)
@@ -125,6 +125,21 @@ struct KstatPlan {
 KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
 int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+
+struct Fp8KstatPlan {
+  bool ok;        // the k-stationary kernel takes this shape (m <= 64)
+  int mt;         // 16-row tiles (1, 2 or 4)
+  int tpw;        // 128-byte k stages per wave (16 waves per workgroup)
+  int ksplit;     // grid.y
+  int nt_per_wg;  // column tiles per workgroup
+  int grid_x;
+  int nb;         // column tiles per batch
+  size_t partial_bytes;
+};
+Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const void* act_q, const float* act_scale,
+                     size_t act_scale_count, const void* w_q, const float* w_scale, size_t w_scale_count, size_t m,
+                     size_t n, size_t k, void* workspace, hipStream_t s);
 
 struct Fp8Plan {
   int MT;
