@@ -203,26 +203,43 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 }
 
+#define KSQ_GO(MT, TPW, NB, NW) hipLaunchKernelGGL((fp8_kstat_kernel<T, MT, TPW, NB, NW>), grid, dim3(64 * NW), 0, s, a)
 template <typename T>
 void launch(int mt, int tpw, int nb, const Fp8KstatArgs& a, dim3 grid, hipStream_t s) {
   if (mt == 1) {
-    const dim3 block(1024);
-    if (tpw == 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 4, 2, 16>), grid, block, 0, s, a);
-    else if (tpw == 2 && nb >= 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 2, 4, 16>), grid, block, 0, s, a);
-    else if (tpw == 2) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 2, 2, 16>), grid, block, 0, s, a);
-    else if (nb >= 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 1, 4, 16>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, 1, 2, 16>), grid, block, 0, s, a);
+    if (tpw == 4) {
+      if (nb == 1) KSQ_GO(1, 4, 1, 16);
+      else KSQ_GO(1, 4, 2, 16);
+    } else if (tpw == 2) {
+      if (nb == 1) KSQ_GO(1, 2, 1, 16);
+      else if (nb == 2) KSQ_GO(1, 2, 2, 16);
+      else KSQ_GO(1, 2, 4, 16);
+    } else {
+      if (nb == 1) KSQ_GO(1, 1, 1, 16);
+      else if (nb == 2) KSQ_GO(1, 1, 2, 16);
+      else KSQ_GO(1, 1, 4, 16);
+    }
   } else if (mt == 2) {
-    const dim3 block(1024);
-    if (tpw == 2) hipLaunchKernelGGL((fp8_kstat_kernel<T, 2, 2, 2, 16>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fp8_kstat_kernel<T, 2, 1, 2, 16>), grid, block, 0, s, a);
+    if (tpw == 2) {
+      if (nb == 1) KSQ_GO(2, 2, 1, 16);
+      else KSQ_GO(2, 2, 2, 16);
+    } else {
+      if (nb == 1) KSQ_GO(2, 1, 1, 16);
+      else KSQ_GO(2, 1, 2, 16);
+    }
   } else {
-    const dim3 block(512);
-    if (tpw == 4) hipLaunchKernelGGL((fp8_kstat_kernel<T, 4, 4, 2, 8>), grid, block, 0, s, a);
-    else if (tpw == 2) hipLaunchKernelGGL((fp8_kstat_kernel<T, 4, 2, 2, 8>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fp8_kstat_kernel<T, 4, 1, 2, 8>), grid, block, 0, s, a);
+    if (tpw == 4) {
+      if (nb == 1) KSQ_GO(4, 4, 1, 8);
+      else KSQ_GO(4, 4, 2, 8);
+    } else if (tpw == 2) {
+      if (nb == 1) KSQ_GO(4, 2, 1, 8);
+      else KSQ_GO(4, 2, 2, 8);
+    } else {
+      KSQ_GO(4, 1, 2, 8);
+    }
   }
 }
+#undef KSQ_GO
 
 }  // namespace
 
@@ -256,7 +273,14 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
   if (wgs > ntiles) wgs = ntiles;
   p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
   p.grid_x = (int)((ntiles + p.nt_per_wg - 1) / p.nt_per_wg);
-  p.nb = (p.mt >= 2 || p.tpw == 4 || p.nt_per_wg < 3) ? 2 : 4;
+  // a single row tile reduces after every column tile when the ring is deep enough without batching (measured:
+  // finer batches overlap the reduction of one tile with the stream of the next); more row tiles batch by two
+  p.nb = p.mt >= 2 ? 2 : (p.tpw == 4 ? 1 : (p.tpw == 2 ? 2 : 4));
+  if (p.nb > p.nt_per_wg) p.nb = p.nt_per_wg >= 2 ? 2 : 1;
+  if (const char* e = getenv("KSQ_FP8_NB")) {  // tuning override
+    const int v = atoi(e);
+    if (v == 1 || v == 2 || (v == 4 && p.mt == 1 && p.tpw < 4)) p.nb = v;
+  }
   p.partial_bytes = need(ksplit);
   return p;
 }

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
   using O = Ops<T>;
   constexpr int DPG = 4 / GPT;
   constexpr int D = NB * TPW;  // ring depth = one batch
-  __shared__ f32x4 red[NB * 16 * 64];
+  __shared__ f32x4 red[2 * NB * 16 * 64];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -134,16 +134,22 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- sum the 16 k slices of every column tile of the batch (fixed order: deterministic)
+    // ---- sum the 16 k slices of every column tile of the batch (fixed order: deterministic).  Two reduction
+    // buffers used in turn and one barrier per batch: whoever writes a buffer again (two batches later) has passed the
+    // barrier of the batch in between, which the readers of this batch reach only after their reads.  The reading
+    // waves rotate, so the trips to memory of one batch's epilogue overlap with the next batches.
+    f32x4* rb = red + (b & 1) * (NB * 16 * 64);
 #pragma unroll
-    for (int i = 0; i < NB; ++i) red[(i * 16 + wave) * 64 + lane] = accb[i];
+    for (int i = 0; i < NB; ++i) rb[(i * 16 + wave) * 64 + lane] = accb[i];
     __syncthreads();
-    if (wave < NB) {
-      const int nt = nt_begin + b * NB + wave;
-      const bool valid = b * NB + wave < count;
+    const int first = (b * NB) & 15;            // NB divides 16: the batch's readers are waves first .. first + NB - 1
+    if (wave >= first && wave < first + NB) {
+      const int i = wave - first;
+      const int nt = nt_begin + b * NB + i;
+      const bool valid = b * NB + i < count;
       f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ww = 0; ww < 16; ++ww) sum += red[(wave * 16 + ww) * 64 + lane];
+      for (int ww = 0; ww < 16; ++ww) sum += rb[(i * 16 + ww) * 64 + lane];
       bool store = valid;
       if (p.ksplit > 1 && valid) {
         // split across workgroups: park the fp32 tile, the last split to arrive adds them in split order
@@ -171,7 +177,6 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
         }
       }
     }
-    __syncthreads();  // the reduction buffer is reused by the next batch
   }
 }
 
