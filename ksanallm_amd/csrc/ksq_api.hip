@@ -206,9 +206,9 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     if (mm - 15 > max_m) break;
     W4Plan p = w4a16_plan(mm, n, k, cus, (size_t)-1);
     if (p.partial_bytes > best) best = p.partial_bytes;
+    KstatPlan kp = w4a16_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
+    if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   }
-  KstatPlan kp = w4a16_kstat_plan(1, n, k, cus, (size_t)-1);
-  if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   if (max_m >= 128) {  // the element type is not known here: size for the bf16 route of the prefill kernel
     const size_t pf = w4a16_prefill_workspace_bytes(KSQ_BF16, max_m, k);
     if (pf > best) best = pf;
@@ -235,7 +235,7 @@ int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, co
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g) &&
       (workspace ? workspace_bytes : 0) >= w4a16_prefill_workspace_bytes(dtype, m, k))
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, s);
-  if (m <= 16 && env_int("KSQ_W4_KSTAT", 1) != 0) {
+  if (m <= (size_t)env_int("KSQ_W4_KSTAT_MAX_M", 64) && env_int("KSQ_W4_KSTAT", 1) != 0) {
     KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
     if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s);
   }

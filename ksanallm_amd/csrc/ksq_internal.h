@@ -114,8 +114,10 @@ bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g);
 int w4a16_stream_max_slices(int mt, int nt);
 
 struct KstatPlan {
-  bool ok;       // the k-stationary decode kernel takes this shape
-  int tpw;       // k tiles per wave (16 waves per workgroup)
+  bool ok;       // the k-stationary decode kernel takes this shape (m <= 64)
+  int mt;        // 16-row tiles (1, 2 or 4)
+  int nw;        // waves per workgroup (16 or 8)
+  int tpw;       // k tiles per wave
   int ksplit;    // grid.y
   int nt_per_wg; // column tiles per workgroup
   int grid_x;

@@ -1,12 +1,13 @@
-// W4A16 decode kernel for M <= 16: k-stationary.
+// W4A16 decode kernel for M <= 64: k-stationary.
 //
-// A workgroup is 16 waves.  Wave w keeps the activation fragments of its own TPW k tiles in registers for the
-// whole kernel (the activations of a decode step are tiny: 16 x K) and streams the weight tiles (n tile, its k
-// tiles) of the workgroup's column range straight from HBM into a register ring, one batch of NB column tiles
-// ahead.  Nothing is re-read: no activation traffic per weight tile, no LDS on the streaming path.  After every
-// batch the 16 partial tiles of a column tile (one per wave = per k slice) are summed through LDS in a fixed
-// order.  Because k is covered inside the workgroup, narrow N needs no split across workgroups; only K > 48
-// tiles x 16 waves is split over grid.y and finished by the last-arriving workgroup through the workspace.
+// A workgroup is 16 waves (one 16-row tile of activations) or 8 waves with twice the registers each (two or four row
+// tiles).  Wave w keeps the activation fragments of its own TPW k tiles, for all MT row tiles, in registers for the
+// whole kernel (the activations of a decode step are small) and streams the weight tiles (n tile, its k tiles) of
+// the workgroup's column range straight from HBM into a register ring, one batch of NB column tiles ahead.  Nothing
+// is re-read: no activation traffic per weight tile, no LDS on the streaming path.  After every batch the partial
+// tiles of a (column tile, row tile) -- one per wave = per k slice -- are summed through LDS in a fixed order, one
+// tile per wave.  Because k is covered inside the workgroup, narrow N needs no split across workgroups; only K
+// beyond waves x TPW tiles is split over grid.y and finished by the last-arriving workgroup through the workspace.
 //
 // Arithmetic as in the streaming kernel: biased nibbles by bit operations, a correction MFMA with -(bias + z),
 // fp32 group sums scaled by s[g,n].
@@ -25,17 +26,18 @@ struct KstatArgs {
   const void* sz;      // [ntiles][G][16] x 4 B
   const void* act;     // [M][K] T
   void* out;           // [M][N] T
-  f32x4* partial;      // [ksplit][ntiles][64]
-  unsigned* counters;  // [ntiles]
+  f32x4* partial;      // [ksplit][ntiles][MT][64]
+  unsigned* counters;  // [ntiles][MT]
   int M, N, K, KT, G, ntiles, ksplit, nt_per_wg;
 };
 
-template <typename T, int GPT, int TPW, int NB>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void w4a16_kstat_kernel(KstatArgs p) {
+template <typename T, int GPT, int MT, int TPW, int NB, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4))) void w4a16_kstat_kernel(KstatArgs p) {
   using O = Ops<T>;
   constexpr int DPG = 4 / GPT;
   constexpr int D = NB * TPW;  // ring depth = one batch
-  __shared__ f32x4 red[2 * NB * 16 * 64];
+  static_assert(NB * MT * NW <= 64 && NB * MT <= NW && NW % (NB * MT) == 0, "reduction: two buffers of <= 64 KiB");
+  __shared__ f32x4 red[2 * NB * MT * NW * 64];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -72,15 +74,18 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
   const unsigned w_stride = (unsigned)p.KT * 1024u, sz_stride = (unsigned)p.G * 64u;
 
   // activation fragments of this wave's k tiles: registers for the whole kernel
-  u32x4 af[TPW][4];
+  u32x4 af[MT][TPW][4];
 #pragma unroll
-  for (int t = 0; t < TPW; ++t)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const bool ok = c < p.M && kt0 + t < wg_end;
-      const unsigned ao = ok ? ((unsigned)c * p.K + (kt0 + t) * kTileK + 32 * d + 8 * j) * 2u : 0x80000000u;
-      af[t][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
-    }
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const int row = 16 * mt + c;
+        const bool ok = row < p.M && kt0 + t < wg_end;
+        const unsigned ao = ok ? ((unsigned)row * p.K + (kt0 + t) * kTileK + 32 * d + 8 * j) * 2u : 0x80000000u;
+        af[mt][t][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+      }
 
   u32x4 wq[D];
   uint32_t szq[D][GPT];
@@ -106,10 +111,11 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
 
   uint16_t* out = static_cast<uint16_t*>(p.out);
   for (int b = 0; b < nbatches; ++b) {
-    f32x4 accb[NB];
+    f32x4 accb[NB][MT];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-      accb[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) accb[i][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int t = 0; t < TPW; ++t) {
         const int slot = i * TPW + t;
@@ -119,60 +125,75 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
           const uint32_t z = szw >> 16;
           const u32x4 corr = O::correction(z | (z << 16));
           const float s = O::scale_to_float(szw);
-          f32x4 P = {0.f, 0.f, 0.f, 0.f};
+          f32x4 P[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int dd = 0; dd < DPG; ++dd) {
             const int d = gi * DPG + dd;
             const u32x4 bw = O::unpack(wq[slot][d], m_lo, m_hi, c_lo, c_hi);
-            P = O::mfma(af[t][d], corr, P);
-            P = O::mfma(af[t][d], bw, P);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              P[mt] = O::mfma(af[mt][t][d], corr, P[mt]);
+              P[mt] = O::mfma(af[mt][t][d], bw, P[mt]);
+            }
           }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) accb[i][e] += s * P[e];
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) accb[i][mt][e] += s * P[mt][e];
         }
         fetch(slot, (b + 1) * NB + i, t);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- sum the 16 k slices of every column tile of the batch (fixed order: deterministic).  Two reduction
-    // buffers used in turn and one barrier per batch: whoever writes a buffer again (two batches later) has passed the
-    // barrier of the batch in between, which the readers of this batch reach only after their reads.  The reading
-    // waves rotate, so the trips to memory of one batch's epilogue overlap with the next batches.
-    f32x4* rb = red + (b & 1) * (NB * 16 * 64);
+    // ---- sum the k slices of every tile of the batch (fixed order: deterministic).  Two reduction buffers used in
+    // turn and one barrier per batch: whoever writes a buffer again (two batches later) has passed the barrier of
+    // the batch in between, which the readers of this batch reach only after their reads.  One (column tile, row
+    // tile) per wave, and the reading waves rotate, so the trips to memory of one batch's epilogue overlap with the
+    // next batches.
+    f32x4* rb = red + (b & 1) * (NB * MT * NW * 64);
 #pragma unroll
-    for (int i = 0; i < NB; ++i) rb[(i * 16 + wave) * 64 + lane] = accb[i];
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) rb[((i * MT + mt) * NW + wave) * 64 + lane] = accb[i][mt];
     __syncthreads();
-    const int first = (b * NB) & 15;            // NB divides 16: the batch's readers are waves first .. first + NB - 1
-    if (wave >= first && wave < first + NB) {
-      const int i = wave - first;
+    const int first = (b * NB * MT) & (NW - 1);  // NB * MT divides NW
+    if (wave >= first && wave < first + NB * MT) {
+      const int q = wave - first, i = q / MT, mt = q - i * MT;
       const int nt = nt_begin + b * NB + i;
-      const bool valid = b * NB + i < count;
+      const bool valid = b * NB + i < count && 16 * mt < p.M;
       f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ww = 0; ww < 16; ++ww) sum += rb[(i * 16 + ww) * 64 + lane];
+      for (int w4 = 0; w4 < NW; w4 += 4) {  // four slices at a time: the weight ring is live in registers here
+#pragma unroll
+        for (int ww = w4; ww < w4 + 4; ++ww) sum += rb[(q * NW + ww) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);
+      }
       bool store = valid;
       if (p.ksplit > 1 && valid) {
         // split across workgroups: park the fp32 tile, the last split to arrive adds them in split order
-        const size_t stride = (size_t)p.ntiles * 64;
-        store_agent(p.partial + (size_t)split * stride + (size_t)nt * 64 + lane, sum);
+        const size_t stride = (size_t)p.ntiles * MT * 64;
+        const size_t tile = ((size_t)nt * MT + mt) * 64 + lane;
+        store_agent(p.partial + (size_t)split * stride + tile, sum);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned* counter = p.counters + nt * MT + mt;
         unsigned arrived = 0;
-        if (lane == 0)
-          arrived = __hip_atomic_fetch_add(p.counters + nt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         arrived = __builtin_amdgcn_readfirstlane(arrived);
         store = arrived == (unsigned)(p.ksplit - 1);
         if (store) {
           asm volatile("" ::: "memory");
           sum = f32x4{0.f, 0.f, 0.f, 0.f};
-          for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + (size_t)sp * stride + (size_t)nt * 64 + lane);
-          if (lane == 0) __hip_atomic_store(p.counters + nt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + (size_t)sp * stride + tile);
+          if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
       if (store) {
         const int col = nt * 16 + c;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int row = 4 * j + e;
+          const int row = 16 * mt + 4 * j + e;
           if (row < p.M) out[(size_t)row * p.N + col] = O::to_bits(sum[e]);
         }
       }
@@ -180,54 +201,93 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
   }
 }
 
-template <typename T, int GPT, int TPW>
-void launch_nb(int nb, const KstatArgs& a, dim3 grid, hipStream_t s) {
-  if (nb >= 4) hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, TPW, 4>), grid, dim3(1024), 0, s, a);
-  else if (nb >= 2) hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, TPW, 2>), grid, dim3(1024), 0, s, a);
-  else hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, TPW, 1>), grid, dim3(1024), 0, s, a);
-}
-
+#define KSQ_GO(MT, TPW, NB, NW) \
+  hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, MT, TPW, NB, NW>), grid, dim3(64 * NW), 0, s, a)
 template <typename T, int GPT>
-void launch_tpw(int tpw, int nb, const KstatArgs& a, dim3 grid, hipStream_t s) {
-  if (tpw <= 1) launch_nb<T, GPT, 1>(nb, a, grid, s);
-  else if (tpw == 2) launch_nb<T, GPT, 2>(nb, a, grid, s);
-  else launch_nb<T, GPT, 3>(nb, a, grid, s);
+void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
+  const int tpw = pl.tpw, nb = pl.nb;
+  if (pl.mt == 1) {
+    if (tpw <= 1) {
+      if (nb >= 4) KSQ_GO(1, 1, 4, 16);
+      else if (nb >= 2) KSQ_GO(1, 1, 2, 16);
+      else KSQ_GO(1, 1, 1, 16);
+    } else if (tpw == 2) {
+      if (nb >= 4) KSQ_GO(1, 2, 4, 16);
+      else if (nb >= 2) KSQ_GO(1, 2, 2, 16);
+      else KSQ_GO(1, 2, 1, 16);
+    } else {
+      if (nb >= 2) KSQ_GO(1, 3, 2, 16);
+      else KSQ_GO(1, 3, 1, 16);
+    }
+  } else if (pl.mt == 2) {
+    if (tpw <= 2) {
+      if (nb >= 2) KSQ_GO(2, 2, 2, 8);
+      else KSQ_GO(2, 2, 1, 8);
+    } else {
+      if (nb >= 2) KSQ_GO(2, 4, 2, 8);
+      else KSQ_GO(2, 4, 1, 8);
+    }
+  } else {
+    if (tpw <= 1) {
+      if (nb >= 2) KSQ_GO(4, 1, 2, 8);
+      else KSQ_GO(4, 1, 1, 8);
+    } else {
+      if (nb >= 2) KSQ_GO(4, 2, 2, 8);
+      else KSQ_GO(4, 2, 1, 8);
+    }
+  }
 }
+#undef KSQ_GO
 
 }  // namespace
 
-// Plan of the k-stationary kernel: k tiles per wave (at most 3, i.e. 48 per workgroup), split count, column tiles
-// per workgroup and batch size.
+// Plan of the k-stationary kernel: row tiles (1, 2 or 4), waves per workgroup (16 for one row tile, else 8), k
+// tiles per wave (the activations of waves x tpw k tiles live in registers: at most 48, 32 or 16 k tiles per
+// workgroup for 1, 2 or 4 row tiles), split count, column tiles per workgroup and batch size.
 KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   KstatPlan p{};
   const size_t ntiles = n / kTileN, ktiles = k / kTileK;
-  p.ok = m >= 1 && m <= 16 && ntiles <= (size_t)kCountersPerSlot;
-  size_t ksplit = (ktiles + 47) / 48;
+  p.ok = m >= 1 && m <= 64 && ntiles * 4 <= (size_t)kCountersPerSlot;
+  if (!p.ok) return p;
+  p.mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
+  p.nw = p.mt == 1 ? 16 : 8;
+  const size_t tpw_max = p.mt == 1 ? 3 : (p.mt == 2 ? 4 : 2);
+  const size_t cap = (size_t)p.nw * tpw_max;
+  size_t ksplit = (ktiles + cap - 1) / cap;
   if (const char* e = getenv("KSQ_W4_KSPLIT")) {  // tuning / test override; never below what the registers need
     const size_t v = (size_t)atoi(e);
     if (v > ksplit && v <= ktiles) ksplit = v;
   }
-  if (ksplit > 1 && ksplit * ntiles * 64 * 16 > workspace_bytes) p.ok = false;
-  if (!p.ok) return p;
+  auto need = [&](size_t ks) { return ks <= 1 ? (size_t)0 : ks * ntiles * p.mt * 64 * 16; };
+  if (need(ksplit) > workspace_bytes) {
+    p.ok = false;
+    return p;
+  }
   const size_t per_split = (ktiles + ksplit - 1) / ksplit;
+  size_t tpw = (per_split + p.nw - 1) / p.nw;
+  if (p.mt == 2) tpw = tpw <= 2 ? 2 : 4;  // instantiated widths
   p.ksplit = (int)ksplit;
-  p.tpw = (int)((per_split + 15) / 16);
+  p.tpw = (int)tpw;
   size_t wgs = (size_t)cus / ksplit;
   if (wgs < 1) wgs = 1;
   if (wgs > ntiles) wgs = ntiles;
   p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
   p.grid_x = (int)((ntiles + p.nt_per_wg - 1) / p.nt_per_wg);
-  p.nb = p.nt_per_wg >= 3 ? 4 : (p.nt_per_wg >= 2 ? 2 : 1);  // ring depth = nb * tpw tiles in flight per wave
-  if (p.tpw >= 3 && p.nb > 2) p.nb = 2;  // register budget of 16 waves per workgroup
-  p.partial_bytes = ksplit > 1 ? ksplit * ntiles * 64 * 16 : 0;
+  if (p.mt == 1) {
+    p.nb = p.nt_per_wg >= 3 ? 4 : (p.nt_per_wg >= 2 ? 2 : 1);  // ring depth = nb * tpw tiles in flight per wave
+    if (p.tpw >= 3 && p.nb > 2) p.nb = 2;                       // register budget of 16 waves per workgroup
+  } else {
+    p.nb = p.nt_per_wg >= 2 ? 2 : 1;
+  }
+  p.partial_bytes = need(ksplit);
   return p;
 }
 
 int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
   KSQ_REQUIRE(m * k * 2 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED, "activation tensor larger than 2 GiB");
-  KSQ_REQUIRE((size_t)plan.nt_per_wg * (k / kTileK) * 1024 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED,
-              "column range of one workgroup larger than 2 GiB");
+  KSQ_REQUIRE(((size_t)plan.nt_per_wg + 8) * (k / kTileK) * 1024 < 0x3FFFFF00ull, KSQ_ERR_UNSUPPORTED,
+              "column range of one workgroup larger than 1 GiB");
   KstatArgs a{};
   a.weight = weight;
   a.sz = sz;
@@ -251,11 +311,11 @@ int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* 
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
   const int gpt = (int)(kTileK / g);
   if (dtype == KSQ_F16) {
-    if (gpt == 1) launch_tpw<_Float16, 1>(plan.tpw, plan.nb, a, grid, s);
-    else launch_tpw<_Float16, 2>(plan.tpw, plan.nb, a, grid, s);
+    if (gpt == 1) launch<_Float16, 1>(plan, a, grid, s);
+    else launch<_Float16, 2>(plan, a, grid, s);
   } else {
-    if (gpt == 1) launch_tpw<__bf16, 1>(plan.tpw, plan.nb, a, grid, s);
-    else launch_tpw<__bf16, 2>(plan.tpw, plan.nb, a, grid, s);
+    if (gpt == 1) launch<__bf16, 1>(plan, a, grid, s);
+    else launch<__bf16, 2>(plan, a, grid, s);
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
