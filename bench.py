@@ -6,7 +6,8 @@ decoder layer (qkv 4096x12288, o 4096x4096, gate_up 4096x22016, down 11008x4096;
 fp16 activations N(0,1)) at M = 16 tokens.  Consecutive steps use different layers (8 distinct weight sets,
 ~830 MB) so that no launch re-reads weights that are still resident in the 256 MB last-level cache.  All inputs
 are resident in HBM before the timed region; the K timed steps are one HIP graph on one stream, bracketed by
-events on that stream.
+events on that stream.  `extra` carries the other regimes of the path: the same layer at M = 64, the prefill kernel
+at M = 4096 (bf16 and fp16), and the FP8 GEMM at the Qwen-72B shapes (M = 1, 64, 2048).
 
 Prints ONE JSON line: value = whole-job algorithmic GB/s, plus `roofline` for the dominant kernel (the W4A16
 k-stationary decode kernel) and `cpu_baseline` (the CPU oracle -- dequantize to fp32 + blocked OpenMP GEMM -- timed on the
@@ -24,6 +25,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+MFMA_FP8_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
+SHAPES_72B = [("qkv", 8192, 10240), ("o", 8192, 8192), ("gate_up", 8192, 59136), ("down", 29568, 8192)]
 METRIC = "W4A16 GEMM GB/s (M≤16) & TFLOP/s (M=4096), Llama-7B shapes, 1×MI355X"
 SHAPES_7B = [("qkv", 4096, 12288), ("o", 4096, 4096), ("gate_up", 4096, 22016), ("down", 11008, 4096)]
 GROUP = 128
@@ -173,14 +176,74 @@ def main():
     extra = {}
     if not args.no_extra:
         extra["per_shape"] = per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, dtype)
+        if M != 64:
+            extra["decode_m64"] = per_shape(torch, capi, layers, {k: torch.randn((64, k), device=dev, generator=gen).to(
+                torch.float16) for k in (4096, 11008)}, {n: torch.empty((64, n), dtype=torch.float16, device=dev)
+                                                        for n in (12288, 4096, 22016)},
+                                            *workspace_for(torch, capi, dev, 64), stream, 64, dtype)
         extra["prefill_m4096"] = prefill(torch, capi, layers[0], dev, stream)
         extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], dev, stream, "f16")
+        del layers[1:]
+        torch.cuda.empty_cache()
+        extra["fp8_cfg4"] = fp8_sweep(torch, capi, dev, stream)
     if not args.no_cpu:
         result["cpu_baseline"], extra["parity_vs_cpu"] = cpu_baseline(np, torch, capi, layers[0], acts, outs,
                                                                       workspace, ws_bytes, M, dtype, step_bytes)
     if extra:
         result["extra"] = extra
     print(json.dumps(result), flush=True)
+
+
+def workspace_for(torch, capi, dev, m):
+    ws_bytes = max(capi.w4a16_workspace_bytes(m, n, k) for _, k, n in SHAPES_7B)
+    return torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev), ws_bytes
+
+
+def fp8_sweep(torch, capi, dev, stream):
+    """configs[4]: FP8 e4m3 GEMM at the Qwen-72B shapes, per-channel weight scales x per-token activation scales,
+    bf16 in / out.  M = 1 and 64 against the HBM peak (algorithmic bytes K*N + 4N + M*K + 4M + 2*M*N), M = 2048 against
+    the dense FP8 MFMA peak; the activation quantisation is timed on its own."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    table = {}
+    for name, k, n in SHAPES_72B:
+        ncopies = max(1, min(8, (600 << 20) // (k * n)))
+        ws = [torch.randint(0, 120, (n, k), dtype=torch.uint8, device=dev, generator=gen) for _ in range(ncopies)]
+        wscale = torch.rand(n, device=dev, generator=gen) * 0.01 + 1e-3
+        row = {}
+        for M in (1, 64, 2048):
+            act = torch.randn((M, k), device=dev, generator=gen).to(torch.bfloat16)
+            aq = torch.empty((M, k), dtype=torch.uint8, device=dev)
+            ascale = torch.empty(M, dtype=torch.float32, device=dev)
+            out = torch.empty((M, n), dtype=torch.bfloat16, device=dev)
+            wsb = capi.fp8_workspace_bytes(M, n, k)
+            wk = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+
+            def launch_q(i):
+                capi.fp8_quantize(capi.BF16, act, M, k, capi.FP8_PER_TOKEN_DYNAMIC, aq, ascale, stream.cuda_stream)
+
+            def launch_g(i):
+                capi.fp8_gemm(capi.BF16, out, aq, ascale, M, ws[i % ncopies], wscale, n, M, n, k, wk, wsb,
+                              stream.cuda_stream)
+
+            launch_q(0)
+            torch.cuda.synchronize()
+            reps = 32 if M <= 64 else 4
+            uq = time_graph(torch, stream, launch_q, reps)
+            ug = time_graph(torch, stream, launch_g, reps)
+            if M <= 64:
+                b = k * n + 4 * n + M * k + 4 * M + 2 * M * n
+                row[f"m{M}"] = {"quant_us": round(uq, 1), "gemm_us": round(ug, 1), "GBps": round(b / ug / 1e3, 1),
+                                "frac": round(b / ug / 1e3 / HBM_PEAK_GBPS, 3)}
+            else:
+                tf = 2.0 * M * k * n / ug / 1e6
+                row[f"m{M}"] = {"quant_us": round(uq, 1), "gemm_us": round(ug, 1), "TFLOPs": round(tf, 1),
+                                "frac": round(tf / MFMA_FP8_PEAK_TFLOPS, 4)}
+            del act, aq, out, wk
+        table[name] = row
+        del ws
+        torch.cuda.empty_cache()
+    return table
 
 
 def time_graph(torch, stream, launch, count):
