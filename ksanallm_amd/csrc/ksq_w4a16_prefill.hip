@@ -82,17 +82,29 @@ struct Dequant<__bf16> : Dequant<_Float16> {
 };
 
 // bf16 [M][K] -> fp16 [M][K] * 2^-e[row] (exact: power-of-two shift of an 8-bit significand into 11 bits), with
-// e[row] chosen so that the row maximum lands at 2^14; row_scale[row] = 2^e.  One workgroup per row.
+// e[row] chosen so that the row maximum lands at 2^14; row_scale[row] = 2^e.  One workgroup per row; the row stays
+// in registers between the maximum and the conversion (R chunks of eight elements per lane), so it is read once.
+template <int R>
 __global__ __launch_bounds__(256) void bf16_rows_to_f16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
                                                                float* __restrict__ row_scale, int K) {
   __shared__ float smem[4];
   const size_t row = blockIdx.x;
-  const uint16_t* s = src + row * K;
-  uint16_t* d = dst + row * K;
+  const u32x4* s = reinterpret_cast<const u32x4*>(src + row * K);
+  u32x4* d = reinterpret_cast<u32x4*>(dst + row * K);
+  const int nchunks = K / 8;  // K is a multiple of 128
+  u32x4 v[R];
   float mx = 0.f;
-  for (int i = threadIdx.x; i < K; i += 256) {
-    const float v = __builtin_fabsf(__builtin_bit_cast(float, (uint32_t)s[i] << 16));
-    mx = (v == v && v < __builtin_inff()) ? __builtin_fmaxf(mx, v) : mx;  // NaN / Inf do not set the exponent
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int ch = threadIdx.x + i * 256;
+    v[i] = ch < nchunks ? s[ch] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float lo = __builtin_fabsf(__builtin_bit_cast(float, v[i][q] << 16));
+      const float hi = __builtin_fabsf(__builtin_bit_cast(float, v[i][q] & 0xFFFF0000u));
+      mx = (lo == lo && lo < __builtin_inff()) ? __builtin_fmaxf(mx, lo) : mx;  // NaN / Inf do not set the exponent
+      mx = (hi == hi && hi < __builtin_inff()) ? __builtin_fmaxf(mx, hi) : mx;
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off));
@@ -101,7 +113,47 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_kernel(const uint16_t* _
   mx = __builtin_fmaxf(__builtin_fmaxf(smem[0], smem[1]), __builtin_fmaxf(smem[2], smem[3]));
   int e = 0;
   if (mx > 0.f) e = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFF) - 127 - 14;
-  const float down = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);  // 2^-e, e in [-163, 113]: clamp below
+  e = e < -100 ? -100 : e;  // keeps 2^-e and 2^e normal floats; rows that small lose bits that no output can show
+  const float down = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);  // 2^-e, e in [-100, 113]
+  const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
+  if (threadIdx.x == 0) row_scale[row] = up;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int ch = threadIdx.x + i * 256;
+    u32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float lo = __builtin_bit_cast(float, v[i][q] << 16) * down;
+      const float hi = __builtin_bit_cast(float, v[i][q] & 0xFFFF0000u) * down;
+      o[q] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) |
+             ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+    }
+    if (ch < nchunks) d[ch] = o;
+  }
+}
+
+// the same for rows longer than 16384 elements: two passes over global memory
+__global__ __launch_bounds__(256) void bf16_rows_to_f16_long_kernel(const uint16_t* __restrict__ src,
+                                                                    uint16_t* __restrict__ dst,
+                                                                    float* __restrict__ row_scale, int K) {
+  __shared__ float smem[4];
+  const size_t row = blockIdx.x;
+  const uint16_t* s = src + row * K;
+  uint16_t* d = dst + row * K;
+  float mx = 0.f;
+  for (int i = threadIdx.x; i < K; i += 256) {
+    const float v = __builtin_fabsf(__builtin_bit_cast(float, (uint32_t)s[i] << 16));
+    mx = (v == v && v < __builtin_inff()) ? __builtin_fmaxf(mx, v) : mx;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off));
+  if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = __builtin_fmaxf(__builtin_fmaxf(smem[0], smem[1]), __builtin_fmaxf(smem[2], smem[3]));
+  int e = 0;
+  if (mx > 0.f) e = (int)((__builtin_bit_cast(uint32_t, mx) >> 23) & 0xFF) - 127 - 14;
+  e = e < -100 ? -100 : e;  // keeps 2^-e and 2^e normal floats; rows that small lose bits that no output can show
+  const float down = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
   const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
   if (threadIdx.x == 0) row_scale[row] = up;
   for (int i = threadIdx.x; i < K; i += 256) {
@@ -355,8 +407,13 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "bf16 prefill needs its workspace");
     uint16_t* a16 = static_cast<uint16_t*>(workspace);
     float* row_scale = reinterpret_cast<float*>(static_cast<char*>(workspace) + (m * k * 2 + 255) / 256 * 256);
-    hipLaunchKernelGGL(bf16_rows_to_f16_kernel, dim3((unsigned)m), dim3(256), 0, s, static_cast<const uint16_t*>(act),
-                       a16, row_scale, (int)k);
+    const uint16_t* a_in = static_cast<const uint16_t*>(act);
+    const dim3 rows((unsigned)m), lanes(256);
+    if (k <= 2048) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<1>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
+    else if (k <= 4096) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<2>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
+    else if (k <= 8192) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<4>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
+    else if (k <= 16384) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<8>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
+    else hipLaunchKernelGGL(bf16_rows_to_f16_long_kernel, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     a.act = a16;
     a.row_scale = row_scale;
     launch_typed<__bf16>(a, gpt, nw, grid, block, s);

@@ -128,6 +128,24 @@ def test_prefill_kernel_widths(gpu, waves, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+def test_prefill_bf16_row_magnitudes(gpu):
+    """bf16 activations go through a per-row power-of-two re-encoding on the large-M route: rows of very different
+    magnitude (up to 2^100, down to 2^-60, an all-zero row) must each keep full relative accuracy."""
+    M, K, N = 160, 512, 256
+    rng = np.random.default_rng(1270)
+    act = rng.standard_normal((M, K)).astype(np.float32)
+    exps = rng.integers(-60, 101, size=M)
+    act *= np.exp2(exps.astype(np.float64)).astype(np.float32)[:, None]
+    act[7, :] = 0.0
+    case = W4Case(1271, M, K, N, kind="awq", dtype="bf16", act=act)
+    got = W4Device(case, gpu).gemm_f32()
+    want = case.oracle()
+    assert np.all(got[7] == 0.0)
+    for row in range(M):  # every row against its own scale
+        if row != 7:
+            orc.assert_parity(got[row:row + 1], want[row:row + 1], f"row {row} (2^{exps[row]})")
+
+
 def test_no_workspace_still_correct(gpu):
     case = W4Case(1300, 16, 4096, 512, kind="gptq", dtype="f16")
     dev = W4Device(case, gpu)
