@@ -73,19 +73,25 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
   const unsigned w_stride = (unsigned)p.KT * 1024u, sz_stride = (unsigned)p.G * 64u;
 
-  // activation fragments of this wave's k tiles: registers for the whole kernel
+  // Activation fragments of this wave's k tiles: registers for the whole kernel.  They are loaded with lane l on
+  // row l / 4, 16-byte piece l % 4 of a 32-k step, so that every aligned group of four lanes reads 64 contiguous
+  // bytes (the memory pipeline then takes four lanes per clock instead of one), and moved to the MFMA operand layout
+  // (lane 16 j + c = row c, piece j) by a lane permutation further down.
   u32x4 af[MT][TPW][4];
+  {
+    const int lr = lane >> 2, lp = lane & 3;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < TPW; ++t)
+      for (int t = 0; t < TPW; ++t)
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const int row = 16 * mt + c;
-        const bool ok = row < p.M && kt0 + t < wg_end;
-        const unsigned ao = ok ? ((unsigned)row * p.K + (kt0 + t) * kTileK + 32 * d + 8 * j) * 2u : 0x80000000u;
-        af[mt][t][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
-      }
+        for (int d = 0; d < 4; ++d) {
+          const int row = 16 * mt + lr;
+          const bool ok = row < p.M && kt0 + t < wg_end;
+          const unsigned ao = ok ? ((unsigned)row * p.K + (kt0 + t) * kTileK + 32 * d + 8 * lp) * 2u : 0x80000000u;
+          af[mt][t][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+        }
+  }
 
   u32x4 wq[D];
   uint32_t szq[D][GPT];
@@ -107,6 +113,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   for (int q = 0; q < D; ++q) {
     fetch(q, q / TPW, q % TPW);
     __builtin_amdgcn_sched_barrier(0);
+  }
+
+  {  // lane 16 j + c takes what lane 4 c + j loaded
+    const int from = (4 * c + j) * 4;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            af[mt][t][d][q] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)af[mt][t][d][q]);
   }
 
   uint16_t* out = static_cast<uint16_t*>(p.out);
