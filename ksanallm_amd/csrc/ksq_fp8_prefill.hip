@@ -233,18 +233,31 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_w =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.wq), 0, (int)((size_t)p.N * p.K), 0x00020000);
-  // Staging role of this wave: fragments 4 * wave + i, i < 4, of each operand (16-row tile (4 wave + i) >> 1, half
-  // i & 1); rows past M / N repeat the last row (their results are never stored).
-  unsigned a_off[2], w_off[2];
+  // Operand stage in LDS: 32 blocks of 1 KiB per operand, block (tile, q) = rows 8q .. 8q+7 of a 16-row tile, all
+  // 128 bytes of the stage.  A block is one global -> LDS load instruction (lane l lands at l * 16) with lane l on
+  // row l/4 % 8, half l / 32 of the 128 bytes and 16-byte piece (l % 4) ^ x(row, q): every aligned group of four
+  // lanes reads 64 contiguous bytes of one row (the memory pipeline then takes four lanes per clock instead of one),
+  // and the xor makes the 16 rows that one group of 16 lanes reads back for an MFMA operand fall on 16 different
+  // bank groups.  Rows past M / N repeat the last row (their results are never stored).  This wave brings in
+  // blocks 4 * wave .. 4 * wave + 3 of each operand, i.e. tiles 2 * wave and 2 * wave + 1.
+  unsigned a_off[4], w_off[4];
+  {
+    const int rr = (lane >> 2) & 7, hh = lane >> 5;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    int row = m0 + 16 * (2 * wave + h) + r;
-    row = row < p.M ? row : p.M - 1;
-    a_off[h] = (unsigned)row * p.K + 16 * j;
-    int col = n0 + 16 * (2 * wave + h) + r;
-    col = col < p.N ? col : p.N - 1;
-    w_off[h] = (unsigned)col * p.K + 16 * j;
+    for (int i = 0; i < 4; ++i) {
+      const int q = i & 1, x = (rr >> 2) | (q << 1);
+      const unsigned kb = 64u * hh + 16u * ((lane & 3) ^ x);
+      int row = m0 + 16 * (2 * wave + (i >> 1)) + 8 * q + rr;
+      row = row < p.M ? row : p.M - 1;
+      a_off[i] = (unsigned)row * p.K + kb;
+      int col = n0 + 16 * (2 * wave + (i >> 1)) + 8 * q + rr;
+      col = col < p.N ? col : p.N - 1;
+      w_off[i] = (unsigned)col * p.K + kb;
+    }
   }
+  // where lane (r, j) finds piece j of half 0 of row r of a tile inside the stage, apart from tile * 128 and
+  // half * 32 (in 16-byte units)
+  const int f_lane = (r >> 3) * 64 + (r & 7) * 4 + (j ^ (((r & 7) >> 2) | ((r >> 3) << 1)));
 
   f32x4 acc[kMT][kNT];
 #pragma unroll
@@ -256,14 +269,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   auto load_item = [&](u32x4* abuf, u32x4* bbuf, int s, int i) {
     const int f = i & 3;
     if (i < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f >> 1],
-                                               s * 128 + (f & 1) * 64, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], s * 128, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f >> 1],
-                                               s * 128 + (f & 1) * 64, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], s * 128, 0, 0);
   };
   auto read_frag = [&](const u32x4* buf, int tile) {
-    return join(buf[(tile * 2 + 0) * 64 + lane], buf[(tile * 2 + 1) * 64 + lane]);
+    return join(buf[tile * 128 + f_lane], buf[tile * 128 + 32 + f_lane]);
   };
 
   auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt, int s) {

@@ -1,8 +1,10 @@
 // W4A16 prefill kernel (large M, MFMA-bound).
 //
-// Workgroup tile 128 rows x 256 columns, four waves side by side: every wave owns a 128 x 64 output tile
-// (8 x 4 MFMA tiles of 16 x 16, fp32 accumulators in registers).  Activations are staged through LDS in MFMA
-// fragment order, 64 k at a time, double-buffered, one barrier per stage.  Weights never touch LDS: each wave
+// Workgroup tile 128 rows x 256 or 512 columns, four or eight waves side by side: every wave owns a 128 x 64 output
+// tile (8 x 4 MFMA tiles of 16 x 16, fp32 accumulators in registers).  Activations go from global memory straight
+// into LDS (no staging registers), 128 k at a time, two stages, one barrier per stage, in a layout that keeps both
+// the global reads (four lanes per 64 contiguous bytes) and the LDS reads (no bank conflicts) at full rate.
+// Weights never touch LDS: each wave
 // reads its own column tiles straight from the fragment-order buffer (one 128-bit load per lane = the B operands of
 // four 16x16x32 MFMAs), one k tile ahead, and dequantises them in registers once per 128 rows:
 //   w = T((u - z) * s), rounded once -- the reference's dequantise-then-MMA semantics
@@ -206,16 +208,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   }
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
-  // Staging role of this wave: fragments f = kFPW * wave + i of a stage, f = 4 * (row tile) + (32-k step); rows
-  // past M repeat row M - 1 (their results are never stored).  A fragment is 64 lanes x 16 bytes, lane (c, j) =
-  // row c, k = 8 j .. 8 j + 7 of the step, and goes from global memory straight into LDS at lane * 16.
-  unsigned a_off[2] = {0u, 0u};  // kFPW / 4 of them in use
+  // Activation stage in LDS: 32 blocks of 1 KiB, block (mt, q) = rows 4q .. 4q+3 of row tile mt, all 256 bytes of
+  // the k tile.  A block is one global -> LDS load instruction (lane l lands at l * 16), with lane l on row l/4 % 4,
+  // 32-k step l / 16 and 16-byte piece (l % 4) ^ q: every aligned group of four lanes reads 64 contiguous bytes of
+  // one row (the memory pipeline then takes four lanes per clock instead of one), and the xor by q makes the 16
+  // rows that one group of 16 lanes reads back for an MFMA operand (piece j of rows 0..15) fall on 16 different
+  // bank groups.  Rows past M repeat row M - 1 (their results are never stored).  This wave brings in blocks
+  // kFPW * wave .. kFPW * wave + kFPW - 1.
+  unsigned a_off[8];  // kFPW of them in use: block i of this wave
 #pragma unroll
-  for (int h = 0; h < kFPW / 4; ++h) {
-    int row = m0 + 16 * (kFPW / 4 * wave + h) + c;
-    row = row < p.M ? row : p.M - 1;
-    a_off[h] = ((unsigned)row * p.K + 8 * j) * 2u;
+  for (int i = 0; i < 8; ++i) {
+    a_off[i] = 0u;
+    if (i < kFPW) {
+      const int blk = kFPW * wave + i, mt = blk >> 2, q = blk & 3;
+      int row = m0 + 16 * mt + 4 * q + ((lane >> 2) & 3);
+      row = row < p.M ? row : p.M - 1;
+      a_off[i] = (unsigned)row * p.K * 2u + 64u * (lane >> 4) + 16u * ((lane & 3) ^ q);
+    }
   }
+  // where lane (c, j) finds piece j of row c of a (row tile, 32-k step) inside the stage, apart from
+  // row tile * 256 + step * 16 (in 16-byte units)
+  const int a_lane = (c >> 2) * 64 + (c & 3) * 4 + (j ^ (c >> 2));
   const unsigned w_voff = lane * 16u, sz_voff = c * 4u;
 
   f32x4 acc[kMT][kNT];
@@ -232,15 +245,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 
   // The loads of the next k tile are issued a few at a time between the matrix instructions of the current one
   // (a burst of 16 memory instructions would hold the wave in the issue queue of the memory pipeline, and the
-  // matrix cores with it).  Part q = 0..3 of a tile's loads, in four items: activation fragments (global -> LDS,
-  // no registers; two with four waves, one with eight), the weight fragment of column tile q, its scale/zero
-  // words (past the last k tile the resources return zero).
+  // matrix cores with it).  Part q = 0..3 of a tile's loads, in four items: activation blocks (global -> LDS, no
+  // registers; two with four waves, one with eight), the weight fragment of column tile q, its scale/zero words
+  // (past the last k tile the resources return zero).
   auto load_item = [&](u32x4* buf, BTile& b, int kt, int q, int item) {
     if (item < 2) {
       if (item < kFPW / 4) {
         const int i = kFPW / 4 * q + item;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i >> 2],
-                                                 kt * 256 + (i & 3) * 64, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i], kt * 256,
+                                                 0, 0);
       }
     } else if (item == 2) {
       b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
@@ -266,7 +279,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   // of the matrix instructions that use them, so that the LDS latency hides behind 16 MFMAs.
   auto read_half = [&](u32x4 (&a)[4], const u32x4* buf, int ks, int h) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = buf[((4 * h + i) * 4 + ks) * 64 + lane];
+    for (int i = 0; i < 4; ++i) a[i] = buf[(4 * h + i) * 256 + ks * 16 + a_lane];
   };
   auto mfma_row = [&](const u32x4& a, const u32x4 (&b)[kNT], int mt) {
 #pragma unroll
@@ -389,7 +402,8 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   // used when that still leaves at least one workgroup for every CU, otherwise four waves (128 x 256, two per CU).
   const DeviceInfo* di = device_info();
   KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
-  int nw = (size_t)a.mblocks * ((a.ntiles + 31) / 32) >= (size_t)di->cus ? 8 : 4;
+  // measured at M = 4096: eight waves win up to N = 8192 (fewer, fatter workgroups), four waves beyond
+  int nw = ((size_t)a.mblocks * ((a.ntiles + 31) / 32) >= (size_t)di->cus && a.ntiles <= 512) ? 8 : 4;
   if (const char* e = getenv("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
     const int v = atoi(e);
     if (v == 4 || v == 8) nw = v;
