@@ -78,14 +78,18 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
       const_cast<uint8_t*>(p.wq) + (size_t)nt_begin * 16 * p.K, 0, (int)((size_t)rows * p.K), 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
-  // per stage and half: offset of this lane's 16 bytes inside its row, or out of range (stage past the split's end,
-  // piece past K)
+  // Loads are issued with lane l on row l / 4 and 16-byte piece l % 4 of a 64-byte half stage, so that every aligned
+  // group of four lanes reads 64 contiguous bytes (the memory pipeline then takes four lanes per clock instead of
+  // one); a lane permutation (lane 16 j + r takes what lane 4 r + j loaded) gives the MFMA operand layout.
+  // per stage and half: offset of the loading lane's 16 bytes inside its row, or out of range (stage past the
+  // split's end, piece past K)
+  const int lr = lane >> 2, lp = lane & 3;
   unsigned k_off[TPW][2];
 #pragma unroll
   for (int t = 0; t < TPW; ++t)
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const unsigned kb = (unsigned)(s0 + t) * 128u + 64u * h + 16u * j;
+      const unsigned kb = (unsigned)(s0 + t) * 128u + 64u * h + 16u * lp;
       k_off[t][h] = (s0 + t < wg_end && kb + 16u <= (unsigned)p.K) ? kb : 0x80000000u;
     }
   // offset of this lane's piece of (stage t, half h) inside column tile 0; a parked offset stays out of range for
@@ -94,8 +98,18 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
 #pragma unroll
   for (int t = 0; t < TPW; ++t)
 #pragma unroll
-    for (int h = 0; h < 2; ++h) w_off[t][h] = k_off[t][h] + (unsigned)r * p.K;
+    for (int h = 0; h < 2; ++h) w_off[t][h] = k_off[t][h] + (unsigned)lr * p.K;
   const unsigned w_stride = 16u * (unsigned)p.K;
+  const int from = (4 * r + j) * 4;
+  auto to_operand = [&](u32x4 lo, u32x4 hi) {
+    i32x8 v;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      v[q] = __builtin_amdgcn_ds_bpermute(from, (int)lo[q]);
+      v[4 + q] = __builtin_amdgcn_ds_bpermute(from, (int)hi[q]);
+    }
+    return v;
+  };
 
   // activation fragments of this wave's stages: registers for the whole kernel
   i32x8 af[MT][TPW];
@@ -103,7 +117,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-      const int row = 16 * mt + r;
+      const int row = 16 * mt + lr;
       u32x4 piece[2];
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
@@ -128,6 +142,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
     __builtin_amdgcn_sched_barrier(0);
   }
 
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+      u32x4 lo, hi;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        lo[q] = (uint32_t)af[mt][t][q];
+        hi[q] = (uint32_t)af[mt][t][4 + q];
+      }
+      af[mt][t] = to_operand(lo, hi);
+    }
+
   uint16_t* out = static_cast<uint16_t*>(p.out);
   for (int b = 0; b < nbatches; ++b) {
     f32x4 accb[NB][MT];
@@ -138,7 +165,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
 #pragma unroll
       for (int t = 0; t < TPW; ++t) {
         const int slot = i * TPW + t;
-        const i32x8 bw = join(wq[slot][0], wq[slot][1]);
+        const i32x8 bw = to_operand(wq[slot][0], wq[slot][1]);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           accb[i][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[mt][t], bw, accb[i][mt], 0, 0, 0, 0, 0, 0);
