@@ -209,7 +209,7 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     KstatPlan kp = w4a16_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
     if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   }
-  if (max_m >= 128) {  // the element type is not known here: size for the bf16 route of the prefill kernel
+  if (max_m >= 65) {  // the element type is not known here: size for the bf16 route of the prefill kernel
     const size_t pf = w4a16_prefill_workspace_bytes(KSQ_BF16, max_m, k);
     if (pf > best) best = pf;
   }

@@ -18,6 +18,7 @@
 // are converted to fp16.
 // Workgroups are numbered so that those sharing a row block of the activations run on the same XCD (own L2).
 #include <cstdlib>
+#include <type_traits>
 
 #include "ksq_internal.h"
 #include "ksq_w4a16_ops.h"
@@ -359,8 +360,205 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   }
 }
 
+// The same GEMM for medium M, where 128-row tiles leave most CUs without work: workgroup tile 64 rows x 256 columns
+// (four waves, every wave 4 x 4 MFMA tiles, two workgroups per CU) and, because such grids run one or two waves
+// per SIMD with nobody to hide a memory round trip behind, everything three k tiles ahead: activations global -> LDS
+// over four stages of 16 KiB (four separate objects), weights in a ring of four register tiles.
+template <typename T, int GPT, int KNT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_mid_kernel(PrefillArgs p) {
+  using O = Ops<_Float16>;
+  using DQ = Dequant<T>;
+  constexpr bool kBF16 = sizeof(T) == 2 && !__is_same(T, _Float16);
+  constexpr int kRows = 4;              // row tiles per workgroup
+  constexpr int kStage = kRows * 4 * 64;  // 16-byte elements per activation stage (64 rows x 128 k) = 16 KiB
+  constexpr int kEpiStride = 68;
+  constexpr int kLoads = 4 + KNT * (1 + GPT);  // memory instructions per k tile and wave
+  __shared__ u32x4 lds_a0[kStage];
+  __shared__ u32x4 lds_a1[kStage];
+  __shared__ u32x4 lds_a2[kStage];
+  __shared__ u32x4 lds_a3[kStage];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, j = lane >> 4;
+
+  const int per_xcd = gridDim.x >> 3;
+  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int st = lid >> 6, r = lid & 63;
+  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
+  const int mb = st_m * 8 + (r & 7), nb = st_n * 8 + (r >> 3);
+  if (mb >= p.mblocks || nb >= p.nblocks) return;
+  const int m0 = mb * (16 * kRows);
+  const int nt0 = (nb * 4 + wave) * KNT;
+
+  __amdgpu_buffer_rsrc_t rs_w[KNT], rs_sz[KNT];
+#pragma unroll
+  for (int t = 0; t < KNT; ++t) {
+    const int nt = nt0 + t;
+    const bool ok = nt < p.ntiles;
+    const size_t ntc = ok ? (size_t)nt : 0;
+    rs_w[t] = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(static_cast<const char*>(p.weight) + ntc * p.KT * 1024), 0, ok ? p.KT * 1024 : 0, 0x00020000);
+    rs_sz[t] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(static_cast<const char*>(p.sz) + ntc * p.G * 64), 0,
+                                                 ok ? p.G * 64 : 0, 0x00020000);
+  }
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
+  // activation blocks as in the 128-row kernel: block (mt, q) = rows 4q .. 4q+3 of row tile mt; this wave brings in
+  // the four blocks of row tile `wave`
+  unsigned a_off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    int row = m0 + 16 * wave + 4 * q + ((lane >> 2) & 3);
+    row = row < p.M ? row : p.M - 1;
+    a_off[q] = (unsigned)row * p.K * 2u + 64u * (lane >> 4) + 16u * ((lane & 3) ^ q);
+  }
+  const int a_lane = (c >> 2) * 64 + (c & 3) * 4 + (j ^ (c >> 2));
+  const unsigned w_voff = lane * 16u, sz_voff = c * 4u;
+
+  f32x4 acc[kRows][KNT];
+#pragma unroll
+  for (int mt = 0; mt < kRows; ++mt)
+#pragma unroll
+    for (int t = 0; t < KNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  struct BTile {
+    u32x4 w[KNT];
+    uint32_t sz[KNT][GPT];
+  };
+  BTile b0, b1, b2, b3;
+
+  // item 0..3 of part q: activation block q, weight fragment of column tile q, its scale/zero words (two items of
+  // which the second is empty when a k tile is one group)
+  auto load_item = [&](u32x4* buf, BTile& b, int kt, int q, int item) {
+    if (item == 0) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (4 * wave + q) * 64), 16, a_off[q], kt * 256, 0, 0);
+    } else if (q < KNT) {
+      if (item == 1)
+        b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
+      else if (item - 2 < GPT)
+        b.sz[q][item - 2] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz[q], sz_voff + (kt * GPT + item - 2) * 64u, 0, 0);
+    }
+  };
+  auto load_tile = [&](u32x4* buf, BTile& b, int kt) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+      for (int item = 0; item < 4; ++item) load_item(buf, b, kt, q, item);
+      __builtin_amdgcn_sched_barrier(0);  // keep the issue order: the waits below count on it
+    }
+  };
+
+  uint32_t m_lo = Ops<_Float16>::kMaskLo, m_hi = Ops<_Float16>::kMaskHi, g_lo = Ops<_Float16>::kMagicLo,
+           g_hi = Ops<_Float16>::kMagicHi;
+  asm volatile("" : "+s"(m_lo));
+  asm volatile("" : "+v"(g_lo));
+  asm volatile("" : "+v"(g_hi));
+  asm volatile("" : "+v"(m_hi));
+
+  auto read_step = [&](u32x4 (&a)[kRows], const u32x4* buf, int ks) {
+#pragma unroll
+    for (int mt = 0; mt < kRows; ++mt) a[mt] = buf[mt * 256 + ks * 16 + a_lane];
+  };
+  // One k tile.  On entry all loads but those of the two youngest tiles have landed; after the barrier tile kt is
+  // visible to every wave and every wave is done with the buffer that tile kt + 3 goes into.
+  // In the steady state (`steady`) the wait leaves the loads of the two youngest tiles in flight and the step issues
+  // those of tile kt + 3; the last steps of a workgroup issue nothing and wait for everything.
+  auto step = [&](const u32x4* cur, u32x4* dst, const BTile& bt, BTile& bn, int kt, auto steady_tag) {
+    constexpr bool kSteady = decltype(steady_tag)::value;
+    constexpr int kCount = kSteady ? 2 * kLoads : 0;  // vmcnt: low four bits, high two bits in 15:14
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kCount & 15) | ((kCount >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 a0[kRows], a1[kRows];
+    read_step(a0, cur, 0);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      u32x4 b[KNT];
+#pragma unroll
+      for (int t = 0; t < KNT; ++t) {
+        const typename DQ::Consts k = DQ::prepare(bt.sz[t][GPT == 2 ? (ks >> 1) : 0]);
+        b[t] = DQ::run(bt.w[t][ks], k, m_lo, m_hi, g_lo, g_hi);
+      }
+      if (ks < 3) read_step((ks & 1) ? a0 : a1, cur, ks + 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < kRows; ++mt) {
+        const u32x4 af = (ks & 1) ? a1[mt] : a0[mt];
+#pragma unroll
+        for (int t = 0; t < KNT; ++t) acc[mt][t] = O::mfma(af, b[t], acc[mt][t]);
+        if constexpr (kSteady) load_item(dst, bn, kt + 3, ks, mt);  // tile kt + 3, one load per four MFMAs
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+
+  load_tile(lds_a0, b0, 0);
+  load_tile(lds_a1, b1, 1);
+  load_tile(lds_a2, b2, 2);
+  // Whole groups of four tiles run in the steady state: every step issues the loads of the tile three ahead, also
+  // past K (weights then read as zero without touching memory, activations as bytes that nobody uses), so that the
+  // number of loads in flight at a step's wait is always the same.  The remaining one to three tiles issue nothing.
+  int kt = 0;
+  for (; kt + 4 <= p.KT; kt += 4) {
+    step(lds_a0, lds_a3, b0, b3, kt, std::true_type{});
+    step(lds_a1, lds_a0, b1, b0, kt + 1, std::true_type{});
+    step(lds_a2, lds_a1, b2, b1, kt + 2, std::true_type{});
+    step(lds_a3, lds_a2, b3, b2, kt + 3, std::true_type{});
+  }
+  if (kt < p.KT) {
+    step(lds_a0, lds_a3, b0, b3, kt, std::false_type{});
+    if (kt + 1 < p.KT) {
+      step(lds_a1, lds_a0, b1, b0, kt + 1, std::false_type{});
+      if (kt + 2 < p.KT) step(lds_a2, lds_a1, b2, b1, kt + 2, std::false_type{});
+    }
+  }
+
+  // ---- epilogue: transpose each 16-row slab through LDS so that every lane stores 16 contiguous bytes
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the unused prefetches must not land on top of the transposes
+  __syncthreads();
+  float* epi = reinterpret_cast<float*>(wave == 0 ? lds_a0 : wave == 1 ? lds_a1 : wave == 2 ? lds_a2 : lds_a3);
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int ncol0 = nt0 * 16;
+#pragma unroll
+  for (int mt = 0; mt < kRows; ++mt) {
+#pragma unroll
+    for (int t = 0; t < KNT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) epi[(4 * j + i) * kEpiStride + 16 * t + c] = acc[mt][t][i];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
+      const float* src = epi + rr * kEpiStride + cc;
+      const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
+      float rs = 1.f;
+      if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
+      u32x4 packed;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        packed[q] = (uint32_t)Ops<T>::to_bits(src[2 * q] * rs) | ((uint32_t)Ops<T>::to_bits(src[2 * q + 1] * rs) << 16);
+      if (cc < 16 * KNT && row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+}
+
 template <typename T>
 void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, hipStream_t s) {
+  if (nw <= 0) {  // 64-row tiles; -nw = 16-column tiles per wave
+    const int knt = -nw;
+    if (gpt == 1) {
+      if (knt == 4) hipLaunchKernelGGL((w4a16_mid_kernel<T, 1, 4>), grid, block, 0, s, a);
+      else if (knt == 2) hipLaunchKernelGGL((w4a16_mid_kernel<T, 1, 2>), grid, block, 0, s, a);
+      else hipLaunchKernelGGL((w4a16_mid_kernel<T, 1, 1>), grid, block, 0, s, a);
+    } else {
+      if (knt == 4) hipLaunchKernelGGL((w4a16_mid_kernel<T, 2, 4>), grid, block, 0, s, a);
+      else if (knt == 2) hipLaunchKernelGGL((w4a16_mid_kernel<T, 2, 2>), grid, block, 0, s, a);
+      else hipLaunchKernelGGL((w4a16_mid_kernel<T, 2, 1>), grid, block, 0, s, a);
+    }
+    return;
+  }
   if (gpt == 1 && nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 4>), grid, block, 0, s, a);
   else if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 8>), grid, block, 0, s, a);
   else if (nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 4>), grid, block, 0, s, a);
@@ -372,7 +570,7 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, 
 bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g) {
   (void)g;
   (void)dtype;
-  return m >= 128 && n % 16 == 0 && m * k * 2 < 0x7FFFFF00ull && (k / kTileK) * 1024 < 0x7FFFFF00ull;
+  return m >= 65 && n % 16 == 0 && m * k * 2 < 0x7FFFFF00ull && (k / kTileK) * 1024 < 0x7FFFFF00ull;
 }
 
 // bf16 route: fp16 copy of the activations + one float per row
@@ -397,23 +595,49 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   a.KT = (int)(k / kTileK);
   a.G = (int)(k / g);
   a.ntiles = (int)(n / kTileN);
-  a.mblocks = (int)((m + kBM - 1) / kBM);
-  // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; they are
-  // used when that still leaves at least one workgroup for every CU, otherwise four waves (128 x 256, two per CU).
   const DeviceInfo* di = device_info();
   KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
-  // measured at M = 4096: eight waves win up to N = 8192 (fewer, fatter workgroups), four waves beyond
-  int nw = ((size_t)a.mblocks * ((a.ntiles + 31) / 32) >= (size_t)di->cus && a.ntiles <= 512) ? 8 : 4;
-  if (const char* e = getenv("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
+  // Row tile of the workgroup: 128 rows when such tiles (128 x 256) give every CU at least two workgroups, else 64
+  // rows with deeper prefetch.
+  int rows = ((m + 127) / 128) * ((size_t)(a.ntiles + 15) / 16) >= 2 * (size_t)di->cus ? 128 : 64;
+  if (const char* e = getenv("KSQ_W4_PREFILL_ROWS")) {  // tuning / test override
     const int v = atoi(e);
-    if (v == 4 || v == 8) nw = v;
+    if (v == 64 || v == 128) rows = v;
   }
-  const int bnt = nw * kNT, sn = 32 / nw;
-  a.nblocks = (a.ntiles + bnt - 1) / bnt;
-  a.super_n = (a.nblocks + sn - 1) / sn;
-  const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * (8 * sn);  // whole super-tiles
-  KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
-  dim3 grid((unsigned)total), block(64 * nw);
+  int nw = 0;  // > 0: waves of the 128-row kernel; <= 0: minus the column tiles per wave of the 64-row kernel
+  dim3 grid, block(256);
+  if (rows == 64) {
+    a.mblocks = (int)((m + 63) / 64);
+    // column tiles per wave: as many (4, 2, 1) as still give every CU two workgroups
+    int knt = 4;
+    while (knt > 1 && (size_t)a.mblocks * ((a.ntiles + 4 * knt - 1) / (4 * knt)) < 2 * (size_t)di->cus) knt >>= 1;
+    if (const char* e = getenv("KSQ_W4_PREFILL_NT")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 1 || v == 2 || v == 4) knt = v;
+    }
+    nw = -knt;
+    a.nblocks = (a.ntiles + 4 * knt - 1) / (4 * knt);
+    a.super_n = (a.nblocks + 7) / 8;
+    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
+    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    grid = dim3((unsigned)total);
+  } else {
+    a.mblocks = (int)((m + kBM - 1) / kBM);
+    // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; measured at
+    // M = 4096 they win up to N = 8192 (fewer, fatter workgroups), four waves (128 x 256, two per CU) beyond.
+    nw = ((size_t)a.mblocks * ((a.ntiles + 31) / 32) >= (size_t)di->cus && a.ntiles <= 512) ? 8 : 4;
+    if (const char* e = getenv("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 4 || v == 8) nw = v;
+    }
+    const int bnt = nw * kNT, sn = 32 / nw;
+    a.nblocks = (a.ntiles + bnt - 1) / bnt;
+    a.super_n = (a.nblocks + sn - 1) / sn;
+    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * (8 * sn);  // whole super-tiles
+    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    grid = dim3((unsigned)total);
+    block = dim3(64 * nw);
+  }
   const int gpt = (int)(kTileK / g);
   if (dtype == KSQ_F16) {
     launch_typed<_Float16>(a, gpt, nw, grid, block, s);

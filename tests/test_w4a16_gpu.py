@@ -128,6 +128,25 @@ def test_prefill_kernel_widths(gpu, waves, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("rows,nt", [(64, 1), (64, 2), (64, 4), (128, 4)])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 65, 640, 528),     # five k tiles: the four-deep ring wraps with a remainder
+    ("bf16", "awq", 128, 200, 1024, 272),
+    ("f16", "gptq", 64, 130, 384, 512),
+    ("bf16", "gptq", 64, 96, 128, 256),    # a single k tile
+])
+def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
+    """The large-M path with 64-row (1, 2 or 4 column tiles per wave) and 128-row workgroup tiles, whichever the
+    planner would pick."""
+    case = W4Case(1260 + rows + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    with _env(KSQ_W4_PREFILL_ROWS=rows, KSQ_W4_PREFILL_NT=nt):
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"prefill rows={rows} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+
+
 def test_prefill_bf16_row_magnitudes(gpu):
     """bf16 activations go through a per-row power-of-two re-encoding on the large-M route: rows of very different
     magnitude (up to 2^100, down to 2^-60, an all-zero row) must each keep full relative accuracy."""
