@@ -56,6 +56,11 @@ typedef enum ksq_zero_kind {
                                  (KS/models/quant/quant_weight.cpp:530-536); z is recovered exactly */
 } ksq_zero_kind;
 
+typedef enum ksq_fp8_merge_mode {
+  KSQ_FP8_MERGE_MAX = 0,         /* one scale = max of the three; the three row ranges are requantised in place */
+  KSQ_FP8_MERGE_PER_CHANNEL = 1  /* one scale per row of the fused weight; the weight bytes are left alone (exact) */
+} ksq_fp8_merge_mode;
+
 typedef enum ksq_fp8_quant_mode {
   KSQ_FP8_PER_TENSOR_DYNAMIC = 0, /* one scale from the abs-max of the whole [m,k] tensor (is_static = false) */
   KSQ_FP8_PER_TENSOR_STATIC = 1,  /* caller-supplied scalar scale (checkpoint input_scale, is_static = true) */
@@ -128,6 +133,19 @@ int ksq_fp8_rescale(const void* in, void* out, size_t count, const float* scale_
  * (KS/models/quant/quant_weight.cpp:685-726): w is [k,n] T; w_q becomes [n,k] e4m3 (k contiguous) with a single
  * scale written to w_scale[0]. */
 int ksq_fp8_convert_weight(int dtype, const void* w, size_t k, size_t n, void* w_q, float* w_scale, void* stream);
+
+/* The same with one scale per output channel (the per-channel x per-token form of ksq_fp8_gemm):
+ * w_scale[c] = max(absmax(w[:,c]) / 448, 1/(448*512)), w_q[c,:] = e4m3(clamp(w[:,c] / w_scale[c], +-448)). */
+int ksq_fp8_convert_weight_per_channel(int dtype, const void* w, size_t k, size_t n, void* w_q, float* w_scale,
+                                       void* stream);
+
+/* Fused q/k/v weight [nq+nk+nv, k] e4m3 whose three row ranges were quantised with their own scalar scales.
+ * KSQ_FP8_MERGE_MAX replaces BindFp8E4m3ScaleOfQkvWeight + GetMaxScaleOfQkv
+ * (KS/models/quant/quant_weight.cpp:816-897): w_scale[0] = max of the three and every range is requantised in place,
+ * w_q = e4m3(float(w_q) * (part_scale / w_scale[0])).  KSQ_FP8_MERGE_PER_CHANNEL writes nq+nk+nv scales instead and
+ * leaves w_q untouched (may be NULL): the per-channel GEMM then reproduces the three separate GEMMs exactly. */
+int ksq_fp8_merge_qkv_scales(int mode, const float* q_scale, const float* k_scale, const float* v_scale, size_t nq,
+                             size_t nk, size_t nv, void* w_q, size_t k, float* w_scale, void* stream);
 
 /* Replaces Fp8QuantizedMatMul (KS/kernels/nvidia/kernel_wrapper.cpp:1033-1041, cuBLASLt FP8 matmul through
  * LK/gemm_wrapper/gemm_wrapper.cc:39-107), extended to the per-token x per-channel scales of

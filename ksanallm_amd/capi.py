@@ -15,6 +15,7 @@ F16, BF16 = 0, 1
 W4_GPTQ_INT32_KPACK, W4_AWQ_INT32_NPACK, W4_ROWMAJOR_INT4_SIGNED = 0, 1, 2
 ZERO_NONE, ZERO_AWQ_INT32, ZERO_UINT8, ZERO_ADDITIVE = 0, 1, 2, 3
 FP8_PER_TENSOR_DYNAMIC, FP8_PER_TENSOR_STATIC, FP8_PER_TOKEN_DYNAMIC = 0, 1, 2
+FP8_MERGE_MAX, FP8_MERGE_PER_CHANNEL = 0, 1
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, -1, -2, -3, -4
 
 EXPORTS = [
@@ -22,7 +23,7 @@ EXPORTS = [
     "ksq_w4a16_repack_sizes", "ksq_w4a16_repack", "ksq_w4a16_repack_host",
     "ksq_w4a16_workspace_bytes", "ksq_w4a16_gemm",
     "ksq_fp8_quantize", "ksq_fp8_rescale", "ksq_fp8_convert_weight",
-    "ksq_fp8_workspace_bytes", "ksq_fp8_gemm",
+    "ksq_fp8_convert_weight_per_channel", "ksq_fp8_merge_qkv_scales", "ksq_fp8_workspace_bytes", "ksq_fp8_gemm",
 ]
 
 
@@ -55,6 +56,8 @@ def lib():
         L.ksq_fp8_quantize.argtypes = [ci, vp, sz, sz, ci, vp, vp, vp]
         L.ksq_fp8_rescale.argtypes = [vp, vp, sz, vp, vp, vp]
         L.ksq_fp8_convert_weight.argtypes = [ci, vp, sz, sz, vp, vp, vp]
+        L.ksq_fp8_convert_weight_per_channel.argtypes = [ci, vp, sz, sz, vp, vp, vp]
+        L.ksq_fp8_merge_qkv_scales.argtypes = [ci, vp, vp, vp, sz, sz, sz, vp, sz, vp, vp]
         L.ksq_fp8_workspace_bytes.argtypes = [sz, sz, sz, psz]
         L.ksq_fp8_gemm.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, vp, sz, vp]
         for name in EXPORTS:
@@ -128,6 +131,15 @@ def fp8_rescale(src, dst, count, scale_in, scale_out, stream=None):
 
 def fp8_convert_weight(dtype, w, k, n, w_q, w_scale, stream=None):
     _check(lib().ksq_fp8_convert_weight(dtype, _addr(w), k, n, _addr(w_q), _addr(w_scale), stream))
+
+
+def fp8_convert_weight_per_channel(dtype, w, k, n, w_q, w_scale, stream=None):
+    _check(lib().ksq_fp8_convert_weight_per_channel(dtype, _addr(w), k, n, _addr(w_q), _addr(w_scale), stream))
+
+
+def fp8_merge_qkv_scales(mode, q_scale, k_scale, v_scale, nq, nk, nv, w_q, k, w_scale, stream=None):
+    _check(lib().ksq_fp8_merge_qkv_scales(mode, _addr(q_scale), _addr(k_scale), _addr(v_scale), nq, nk, nv, _addr(w_q), k,
+                                          _addr(w_scale), stream))
 
 
 def fp8_workspace_bytes(max_m, n, k):

@@ -258,6 +258,48 @@ __global__ __launch_bounds__(256) void transpose_quantize_kernel(const uint16_t*
   }
 }
 
+// per-column abs-max of a [k,n] tensor -> scale[n] (merged over row blocks with an atomic max on the float bits)
+template <typename T>
+__global__ __launch_bounds__(256) void colmax_scale_kernel(const uint16_t* w, size_t k, size_t n, float* scale) {
+  const size_t col = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= n) return;
+  const size_t rows = (k + gridDim.y - 1) / gridDim.y, k0 = (size_t)blockIdx.y * rows;
+  const size_t k1 = k0 + rows < k ? k0 + rows : k;
+  float mx = 0.0f;
+  for (size_t r = k0; r < k1; ++r) mx = fmaxf(mx, fabsf(load_as_float<T>(w, r * n + col)));
+  const float s = fmaxf(mx / kE4m3Max, kMinScale);
+  atomicMax(reinterpret_cast<unsigned int*>(scale + col), __builtin_bit_cast(unsigned int, s));
+}
+
+// [k,n] T -> [n,k] e4m3 through a 64x64 LDS tile, one scale per column of the source (= row of the result)
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_quantize_per_channel_kernel(const uint16_t* w, size_t k, size_t n,
+                                                                             const float* scale, uint8_t* wq) {
+  __shared__ uint8_t tile[64][65];
+  const size_t k0 = (size_t)blockIdx.y * 64, n0 = (size_t)blockIdx.x * 64;
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    int kk = i >> 6, nn = i & 63;
+    uint8_t v = 0;
+    if (k0 + kk < k && n0 + nn < n) v = quantize_one(load_as_float<T>(w, (k0 + kk) * n + n0 + nn), scale[n0 + nn]);
+    tile[kk][nn] = v;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    int nn = i >> 6, kk = i & 63;
+    if (k0 + kk < k && n0 + nn < n) wq[(n0 + nn) * k + k0 + kk] = tile[kk][nn];
+  }
+}
+
+__global__ void max3_kernel(const float* a, const float* b, const float* c, float* out) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) out[0] = fmaxf(fmaxf(a[0], b[0]), c[0]);
+}
+
+__global__ __launch_bounds__(256) void expand3_kernel(const float* a, const float* b, const float* c, size_t na,
+                                                      size_t nb, size_t nc, float* out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < na + nb + nc) out[i] = i < na ? a[0] : (i < na + nb ? b[0] : c[0]);
+}
+
 // ---- streaming GEMM ------------------------------------------------------------------------------------------
 struct Fp8Args {
   const uint8_t* aq;  // [M][K]
@@ -492,6 +534,62 @@ int ksq_fp8_convert_weight(int dtype, const void* w, size_t k, size_t n, void* w
     hipLaunchKernelGGL(absmax_scale_kernel<__bf16>, dim3(nb), dim3(256), 0, s, x, count, w_scale);
     hipLaunchKernelGGL(transpose_quantize_kernel<__bf16>, grid, dim3(256), 0, s, x, k, n, w_scale,
                        static_cast<uint8_t*>(w_q));
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+int ksq_fp8_convert_weight_per_channel(int dtype, const void* w, size_t k, size_t n, void* w_q, float* w_scale,
+                                       void* stream) {
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(w && w_q && w_scale, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  KSQ_REQUIRE(k > 0 && n > 0, KSQ_ERR_INVALID_ARGUMENT, "k and n must be positive");
+  KSQ_REQUIRE((k + 63) / 64 <= 65535 && n < (1ull << 31), KSQ_ERR_UNSUPPORTED, "k or n too large");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint16_t* x = static_cast<const uint16_t*>(w);
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, w_scale, (int)n);
+  size_t kblocks = (k + 511) / 512;
+  if (kblocks > 64) kblocks = 64;
+  dim3 cgrid((unsigned)((n + 255) / 256), (unsigned)kblocks);
+  dim3 grid((unsigned)((n + 63) / 64), (unsigned)((k + 63) / 64));
+  if (dtype == KSQ_F16) {
+    hipLaunchKernelGGL(colmax_scale_kernel<_Float16>, cgrid, dim3(256), 0, s, x, k, n, w_scale);
+    hipLaunchKernelGGL(transpose_quantize_per_channel_kernel<_Float16>, grid, dim3(256), 0, s, x, k, n, w_scale,
+                       static_cast<uint8_t*>(w_q));
+  } else {
+    hipLaunchKernelGGL(colmax_scale_kernel<__bf16>, cgrid, dim3(256), 0, s, x, k, n, w_scale);
+    hipLaunchKernelGGL(transpose_quantize_per_channel_kernel<__bf16>, grid, dim3(256), 0, s, x, k, n, w_scale,
+                       static_cast<uint8_t*>(w_q));
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+int ksq_fp8_merge_qkv_scales(int mode, const float* q_scale, const float* k_scale, const float* v_scale, size_t nq,
+                             size_t nk, size_t nv, void* w_q, size_t k, float* w_scale, void* stream) {
+  KSQ_REQUIRE(mode == KSQ_FP8_MERGE_MAX || mode == KSQ_FP8_MERGE_PER_CHANNEL, KSQ_ERR_INVALID_ARGUMENT,
+              "bad merge mode %d", mode);
+  KSQ_REQUIRE(q_scale && k_scale && v_scale && w_scale, KSQ_ERR_INVALID_ARGUMENT, "null scale pointer");
+  KSQ_REQUIRE(nq > 0 && nk > 0 && nv > 0 && k > 0, KSQ_ERR_INVALID_ARGUMENT, "row counts and k must be positive");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (mode == KSQ_FP8_MERGE_PER_CHANNEL) {
+    const size_t n = nq + nk + nv;
+    KSQ_REQUIRE(n < (1ull << 31), KSQ_ERR_UNSUPPORTED, "too many rows");
+    hipLaunchKernelGGL(expand3_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, q_scale, k_scale, v_scale, nq,
+                       nk, nv, w_scale);
+  } else {
+    KSQ_REQUIRE(w_q != nullptr, KSQ_ERR_INVALID_ARGUMENT, "the max merge rescales the weight: w_q is null");
+    hipLaunchKernelGGL(max3_kernel, dim3(1), dim3(64), 0, s, q_scale, k_scale, v_scale, w_scale);
+    uint8_t* base = static_cast<uint8_t*>(w_q);
+    const float* part_scale[3] = {q_scale, k_scale, v_scale};
+    const size_t part_rows[3] = {nq, nk, nv};
+    size_t row0 = 0;
+    for (int i = 0; i < 3; ++i) {
+      const size_t count = part_rows[i] * k;
+      hipLaunchKernelGGL(rescale_kernel, dim3(blocks_for(count, 4096)), dim3(256), 0, s, base + row0 * k, base + row0 * k,
+                         count, part_scale[i], w_scale);
+      row0 += part_rows[i];
+    }
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;

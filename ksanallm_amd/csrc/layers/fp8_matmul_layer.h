@@ -28,4 +28,19 @@ class Fp8MatMulLayer : public BaseLayer {
   size_t max_n_hint_ = 0;
 };
 
+// Load-time half (replaces the device work of QuantWeight::ConvertFp8E4m3Tensor and BindFp8E4m3ScaleOfQkvWeight,
+// KS/models/quant/quant_weight.cpp:685-726, 816-897).
+//
+// ConvertFp8Weight: weight [k, n] T on the device -> weight_fp8 [n, k] e4m3 + weight_scale (1 float, or n floats
+// with per_channel), both allocated here; weight_fp8.weight_scales is bound.
+Status ConvertFp8Weight(const Tensor& weight, bool per_channel, Tensor& weight_fp8, Tensor& weight_scale, int rank,
+                        Stream& stream);
+// MergeFp8QkvScales: qkv_weight [nq + nk + nv, k] e4m3 whose three row ranges carry the scalar scales q/k/v_scale.
+// per_channel = false is the reference: one scale = their maximum and the ranges are requantised in place;
+// per_channel = true writes one scale per row and leaves the bytes alone.  merged_scale is allocated here and bound
+// to qkv_weight.weight_scales.
+Status MergeFp8QkvScales(Tensor& qkv_weight, const Tensor& q_scale, const Tensor& k_scale, const Tensor& v_scale,
+                         size_t nq, size_t nk, size_t nv, bool per_channel, Tensor& merged_scale, int rank,
+                         Stream& stream);
+
 }  // namespace ksana_llm

@@ -233,6 +233,41 @@ Status Fp8MatMulLayer<T>::Forward(const std::vector<Tensor>& input_tensors, std:
   return Status();
 }
 
+Status ConvertFp8Weight(const Tensor& weight, bool per_channel, Tensor& weight_fp8, Tensor& weight_scale, int rank,
+                        Stream& stream) {
+  if (weight.shape.size() != 2) KLLM_THROW("ConvertFp8Weight: weight must be [k, n].");
+  if (weight.dtype != TYPE_FP16 && weight.dtype != TYPE_BF16) KLLM_THROW("ConvertFp8Weight: weight must be fp16 or bf16.");
+  const size_t k = weight.shape[0], n = weight.shape[1];
+  CreateTensor(weight_fp8, {n, k}, TYPE_FP8_E4M3, rank, MEMORY_DEVICE);
+  CreateTensor(weight_scale, {per_channel ? n : 1}, TYPE_FP32, rank, MEMORY_DEVICE);
+  const int dt = weight.dtype == TYPE_FP16 ? KSQ_F16 : KSQ_BF16;
+  if (per_channel)
+    ThrowOnKsqError(ksq_fp8_convert_weight_per_channel(dt, weight.GetPtr<void>(), k, n, weight_fp8.GetPtr<void>(),
+                                                       weight_scale.GetPtr<float>(), stream.Get()),
+                    "ksq_fp8_convert_weight_per_channel");
+  else
+    ThrowOnKsqError(ksq_fp8_convert_weight(dt, weight.GetPtr<void>(), k, n, weight_fp8.GetPtr<void>(),
+                                           weight_scale.GetPtr<float>(), stream.Get()),
+                    "ksq_fp8_convert_weight");
+  weight_fp8.weight_scales = &weight_scale;
+  return Status();
+}
+
+Status MergeFp8QkvScales(Tensor& qkv_weight, const Tensor& q_scale, const Tensor& k_scale, const Tensor& v_scale,
+                         size_t nq, size_t nk, size_t nv, bool per_channel, Tensor& merged_scale, int rank,
+                         Stream& stream) {
+  if (qkv_weight.shape.size() != 2 || qkv_weight.shape[0] != nq + nk + nv)
+    KLLM_THROW("MergeFp8QkvScales: weight must be [nq + nk + nv, k].");
+  CreateTensor(merged_scale, {per_channel ? nq + nk + nv : 1}, TYPE_FP32, rank, MEMORY_DEVICE);
+  ThrowOnKsqError(
+      ksq_fp8_merge_qkv_scales(per_channel ? KSQ_FP8_MERGE_PER_CHANNEL : KSQ_FP8_MERGE_MAX, q_scale.GetPtr<float>(),
+                               k_scale.GetPtr<float>(), v_scale.GetPtr<float>(), nq, nk, nv, qkv_weight.GetPtr<void>(),
+                               qkv_weight.shape[1], merged_scale.GetPtr<float>(), stream.Get()),
+      "ksq_fp8_merge_qkv_scales");
+  qkv_weight.weight_scales = &merged_scale;
+  return Status();
+}
+
 template class Fp8MatMulLayer<float16>;
 template class Fp8MatMulLayer<bfloat16>;
 

@@ -384,6 +384,18 @@ void orc_fp8_convert_weight(const void* w_kn, int dtype, size_t K, size_t N, uin
   free(t);
 }
 
+/* The same with one scale per output channel (column of the [K,N] source): the per-channel extension of
+ * KS/models/quant/quant_weight.cpp:685-726 that the row-wise FP8 GEMM
+ * (LK/asymmetric_gemm/fp8_rowwise_gemm/fp8_rowwise_gemm_kernel_template_sm90.h:119-131) consumes. */
+void orc_fp8_convert_weight_per_channel(const void* w_kn, int dtype, size_t K, size_t N, uint8_t* wq_nk, float* scale) {
+  float* t = (float*)malloc(sizeof(float) * K * N);
+  for (size_t k = 0; k < K; ++k)
+    for (size_t n = 0; n < N; ++n) t[n * K + k] = load_elem(w_kn, k * N + n, dtype);
+  orc_fp8_compute_scale(t, ORC_F32, N, K, scale);
+  orc_fp8_quantize(t, ORC_F32, scale, N, K, wq_nk);
+  free(t);
+}
+
 int orc_num_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

@@ -247,6 +247,28 @@ def fp8_convert_weight(w_kn_bits, dtype):
     return wq, s
 
 
+def fp8_convert_weight_per_channel(w_kn_bits, dtype):
+    w_kn_bits = _c(w_kn_bits)
+    K, N = w_kn_bits.shape
+    wq = np.empty((N, K), dtype=np.uint8)
+    s = np.empty((N,), dtype=np.float32)
+    lib().orc_fp8_convert_weight_per_channel(_p(w_kn_bits), dtype, _sz(K), _sz(N), _p(wq), _p(s))
+    return wq, s
+
+
+def fp8_merge_qkv_max(wq, q_scale, k_scale, v_scale, nq, nk, nv):
+    """KS/models/quant/quant_weight.cpp:816-897: one scale = max of the three, every row range requantised as
+    e4m3(float(w) * (part_scale / max_scale)).  Returns (merged weight, scale[1])."""
+    merged = np.array([max(float(q_scale), float(k_scale), float(v_scale))], dtype=np.float32)
+    out = np.array(wq, copy=True)
+    row = 0
+    for rows, s in ((nq, q_scale), (nk, k_scale), (nv, v_scale)):
+        part = out[row:row + rows].reshape(-1)
+        out[row:row + rows] = fp8_rescale(part, np.float32(s), merged[0]).reshape(rows, -1)
+        row += rows
+    return out, merged
+
+
 def num_threads():
     return int(lib().orc_num_threads())
 

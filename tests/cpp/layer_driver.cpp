@@ -4,6 +4,8 @@
 //   layer_driver w4a16 <dir> <f16|bf16> <m> <k> <n> <g> <gptq|awq> <gptq|awq|rowmajor> <none|awq|uint8|additive>
 //       reads <dir>/qweight.bin, qzeros.bin (unless none), scales.bin, act.bin; writes <dir>/out.bin
 //   layer_driver fp8 <dir> <f16|bf16> <m> <k> <n> <wscales: 1|n> <static: 0|1>
+//   layer_driver fp8load <dir> <f16|bf16> <m> <k> <nq> <nkv> <per_channel: 0|1>
+//     q/k/v weights [k, n*] T from wq_src.bin / wk_src.bin / wv_src.bin: converted per tensor, fused, scales merged
 //       reads <dir>/wq.bin, wscale.bin, act.bin, iscale.bin (static); writes <dir>/out.bin
 //   layer_driver errors
 //       exercises the error conventions; prints one line per check
@@ -151,6 +153,55 @@ static int RunFp8(int argc, char** argv) {
   return 0;
 }
 
+// The load-time path of an FP8 checkpoint that stores q, k and v separately: convert each [k, n] weight on the fly
+// (one scale per tensor), put the three [n, k] results one after another, merge the scales, run the layer.
+template <typename T>
+static int RunFp8Load(int argc, char** argv) {
+  const std::string dir = argv[2];
+  const size_t m = atol(argv[4]), k = atol(argv[5]), nq = atol(argv[6]), nkv = atol(argv[7]);
+  const bool per_channel = atoi(argv[8]) != 0;
+  const DataType dt = TypeTraits<T>::kDataType;
+  auto context = std::make_shared<Context>(1);
+  Stream& stream = context->GetComputeStreams()[0];
+  const size_t n = nq + 2 * nkv;
+  Tensor fused;
+  CreateTensor(fused, {n, k}, TYPE_FP8_E4M3, 0, MEMORY_DEVICE);
+  const char* names[3] = {"/wq_src.bin", "/wk_src.bin", "/wv_src.bin"};
+  const size_t rows[3] = {nq, nkv, nkv};
+  Tensor part_fp8[3], part_scale[3];
+  size_t row0 = 0;
+  for (int i = 0; i < 3; ++i) {
+    Tensor src = Upload(ReadFile(dir + names[i]), dt, {k, rows[i]});
+    ConvertFp8Weight(src, false, part_fp8[i], part_scale[i], 0, stream);
+    if (hipMemcpyAsync(fused.GetPtr<char>() + row0 * k, part_fp8[i].GetPtr<void>(), rows[i] * k, hipMemcpyDeviceToDevice,
+                       static_cast<hipStream_t>(stream.Get())) != hipSuccess)
+      throw std::runtime_error("hipMemcpyAsync failed");
+    row0 += rows[i];
+  }
+  Tensor merged;
+  MergeFp8QkvScales(fused, part_scale[0], part_scale[1], part_scale[2], nq, nkv, nkv, per_channel, merged, 0, stream);
+  if (hipStreamSynchronize(static_cast<hipStream_t>(stream.Get())) != hipSuccess) throw std::runtime_error("sync failed");
+  Download(fused, dir + "/fused.bin");
+  Download(merged, dir + "/merged_scale.bin");
+
+  ModelConfig cfg;
+  cfg.max_scheduler_token_num = m;
+  std::shared_ptr<Tensor> workspace;
+  MatMulLayerFactory<T> factory(workspace, cfg, 0, context);
+  auto holder = std::make_shared<OneWeight>();
+  holder->t = fused;
+  auto layer = factory.AutoCreateLayer(holder, "model.layers.0.self_attn.query_key_value.weight", TYPE_FP8_E4M3, dt, dt, {});
+  Tensor act = Upload(ReadFile(dir + "/act.bin"), dt, {m, k});
+  Tensor out;
+  CreateTensor(out, {m, n}, dt, 0, MEMORY_DEVICE);
+  std::vector<Tensor> outputs = {out};
+  Status st = layer->Forward({act, fused}, outputs);
+  if (!st.OK()) throw std::runtime_error("Forward returned " + st.GetMessage());
+  Download(outputs[0], dir + "/out.bin");
+  std::cout << "OK " << outputs[0].shape[0] << " " << outputs[0].shape[1] << " " << outputs[0].dtype << std::endl;
+  return 0;
+}
+
 template <typename F>
 static void Expect(const char* name, bool want_throw, F f) {
   bool threw = false;
@@ -263,6 +314,8 @@ int main(int argc, char** argv) {
       return std::string(argv[3]) == "f16" ? RunW4<float16>(argc, argv) : RunW4<bfloat16>(argc, argv);
     if (argc == 9 && std::string(argv[1]) == "fp8")
       return std::string(argv[3]) == "f16" ? RunFp8<float16>(argc, argv) : RunFp8<bfloat16>(argc, argv);
+    if (argc == 9 && std::string(argv[1]) == "fp8load")
+      return std::string(argv[3]) == "f16" ? RunFp8Load<float16>(argc, argv) : RunFp8Load<bfloat16>(argc, argv);
     std::cerr << "usage: see the header of layer_driver.cpp" << std::endl;
     return 2;
   } catch (const std::exception& e) {

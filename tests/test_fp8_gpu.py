@@ -243,3 +243,65 @@ def test_config4_qwen72b_shape(gpu, M):
     xq, xs, wq, ws = _fp8_case(403, M, 8192, 8192)
     got = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
     orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"cfg4 8192x8192 M={M}")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_convert_weight_per_channel(gpu, dtype):
+    import torch
+
+    from ksanallm_amd import capi
+
+    rng = np.random.default_rng(440)
+    K, N = 200, 136
+    wv = (rng.standard_normal((K, N)) * np.exp2(rng.integers(-8, 3, size=N))[None, :]).astype(np.float32)
+    wv[:, 5] = 0.0
+    w = orc.to_bits(wv, ORC_DT[dtype])
+    dw = _upload_bits(w, dtype, gpu)
+    wq = torch.zeros((N, K), dtype=torch.uint8, device=gpu)
+    ws = torch.full((N,), -1.0, dtype=torch.float32, device=gpu)
+    capi.fp8_convert_weight_per_channel(capi_dtype(dtype), dw, K, N, wq, ws)
+    torch.cuda.synchronize()
+    want_q, want_s = orc.fp8_convert_weight_per_channel(w, ORC_DT[dtype])
+    assert np.array_equal(ws.cpu().numpy(), want_s)
+    got = wq.cpu().numpy()
+    nz = (want_q & 0x7F) != 0
+    assert np.array_equal(got[nz], want_q[nz]) and np.all((got[~nz] & 0x7F) == 0)
+
+
+def test_merge_qkv_scales(gpu):
+    """Max merge bit-exact against the oracle; the per-channel merge leaves the bytes alone and the fused GEMM then
+    equals the three separate GEMMs exactly."""
+    import torch
+
+    from ksanallm_amd import capi
+
+    rng = np.random.default_rng(441)
+    nq, nk, nv, K, M = 64, 32, 32, 256, 5
+    wq = rng.integers(0, 256, size=(nq + nk + nv, K), dtype=np.uint8)
+    wq[(wq & 0x7F) == 0x7F] = 0x2a
+    scales = [np.array([v], dtype=np.float32) for v in (0.021, 0.0503, 0.0127)]
+    d_scales = [torch.from_numpy(x).to(gpu) for x in scales]
+    dw = torch.from_numpy(wq).to(gpu)
+    out_s = torch.zeros(1, dtype=torch.float32, device=gpu)
+    capi.fp8_merge_qkv_scales(capi.FP8_MERGE_MAX, *d_scales, nq, nk, nv, dw, K, out_s)
+    torch.cuda.synchronize()
+    want_w, want_s = orc.fp8_merge_qkv_max(wq, scales[0][0], scales[1][0], scales[2][0], nq, nk, nv)
+    assert np.array_equal(out_s.cpu().numpy(), want_s)
+    got = dw.cpu().numpy()
+    nz = (want_w & 0x7F) != 0
+    assert np.array_equal(got[nz], want_w[nz]) and np.all((got[~nz] & 0x7F) == 0)
+
+    dw2 = torch.from_numpy(wq).to(gpu)
+    chan = torch.zeros(nq + nk + nv, dtype=torch.float32, device=gpu)
+    capi.fp8_merge_qkv_scales(capi.FP8_MERGE_PER_CHANNEL, *d_scales, nq, nk, nv, None, K, chan)
+    torch.cuda.synchronize()
+    want_chan = np.concatenate([np.full(nq, scales[0][0]), np.full(nk, scales[1][0]), np.full(nv, scales[2][0])])
+    assert np.array_equal(chan.cpu().numpy(), want_chan.astype(np.float32))
+    xq = rng.integers(0, 120, size=(M, K), dtype=np.uint8)
+    xs = (rng.random(M).astype(np.float32) * 0.01 + 1e-3).astype(np.float32)
+    fused = _run_gemm(gpu, xq, xs, wq, want_chan.astype(np.float32), "f16")
+    row = 0
+    for rows, sc in ((nq, scales[0]), (nk, scales[1]), (nv, scales[2])):
+        part = _run_gemm(gpu, xq, xs, np.ascontiguousarray(wq[row:row + rows]), sc, "f16")
+        assert np.array_equal(fused[:, row:row + rows], part)
+        row += rows

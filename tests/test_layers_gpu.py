@@ -84,6 +84,44 @@ def test_fp8_matmul_layer_forward(gpu, tmp_path, dtype, wscales, static, M):
     orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"Fp8MatMulLayer wscales={wscales} static={static} {dtype}")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("per_channel", [0, 1])
+def test_fp8_load_time_pipeline(gpu, tmp_path, dtype, per_channel):
+    """A checkpoint with separate q/k/v weights in T: on-the-fly conversion, fusion, scale merge (the reference's max
+    merge or the exact per-channel one), then the layer; every stage against the oracle."""
+    M, K, nq, nkv = 9, 256, 96, 32
+    rng = np.random.default_rng(610 + per_channel)
+    d = str(tmp_path)
+    parts, scales = [], []
+    for name, rows, mag in (("wq_src", nq, 0.02), ("wk_src", nkv, 0.05), ("wv_src", nkv, 0.011)):
+        w = orc.to_bits((rng.standard_normal((K, rows)) * mag).astype(np.float32), ORC_DT[dtype])
+        w.tofile(f"{d}/{name}.bin")
+        q, s = orc.fp8_convert_weight(w, ORC_DT[dtype])
+        parts.append(q)
+        scales.append(s[0])
+    x = orc.to_bits(rng.standard_normal((M, K)).astype(np.float32), ORC_DT[dtype])
+    x.tofile(d + "/act.bin")
+    fused = np.concatenate(parts, axis=0)
+    if per_channel:
+        want_w = fused
+        want_s = np.concatenate([np.full(nq, scales[0]), np.full(nkv, scales[1]), np.full(nkv, scales[2])]).astype(np.float32)
+        xs = orc.fp8_compute_scale(x, ORC_DT[dtype], M, K)
+        xq = orc.fp8_quantize(x, ORC_DT[dtype], xs, M, K)
+    else:
+        want_w, want_s = orc.fp8_merge_qkv_max(fused, scales[0], scales[1], scales[2], nq, nkv, nkv)
+        xs = orc.fp8_compute_scale(x, ORC_DT[dtype], 1, M * K)
+        xq = orc.fp8_quantize(x, ORC_DT[dtype], xs, 1, M * K).reshape(M, K)
+    N = nq + 2 * nkv
+    rc, out = _run(["fp8load", d, dtype, M, K, nq, nkv, per_channel])
+    assert rc == 0 and out.splitlines()[-1] == f"OK {M} {N} {DTYPE_ENUM[dtype]}", out
+    got_w = np.fromfile(d + "/fused.bin", dtype=np.uint8).reshape(N, K)
+    nz = (want_w & 0x7F) != 0
+    assert np.array_equal(got_w[nz], want_w[nz]) and np.all((got_w[~nz] & 0x7F) == 0)
+    assert np.array_equal(np.fromfile(d + "/merged_scale.bin", dtype=np.float32), want_s)
+    got = orc.from_bits(np.fromfile(d + "/out.bin", dtype=np.uint16).reshape(M, N), ORC_DT[dtype])
+    orc.assert_parity(got, orc.fp8_gemm(xq, xs, want_w, want_s), f"fp8 load-time pipeline per_channel={per_channel}")
+
+
 def test_error_conventions(gpu):
     rc, out = _run(["errors"])
     lines = [ln for ln in out.splitlines() if ln.startswith(("PASS", "FAIL"))]

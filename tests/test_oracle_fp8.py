@@ -125,3 +125,46 @@ def test_fp8_convert_weight_transposes_and_uses_one_scale():
     assert np.isclose(s[0], np.abs(w.astype(np.float32)).max() / 448.0, rtol=1e-6)
     back = orc.e4m3_decode(wq) * s[0]
     assert np.max(np.abs(back - w.T.astype(np.float32))) <= np.abs(w.astype(np.float32)).max() / 448.0 * 16 + 1e-9
+
+
+def test_convert_weight_per_channel_closed_form():
+    """Per-channel conversion = the per-row closed form of LU/utils_test.cu:93-99 applied to the transposed tensor."""
+    rng = np.random.default_rng(77)
+    K, N = 48, 20
+    w = (rng.standard_normal((K, N)) * np.exp2(rng.integers(-6, 4, size=N))[None, :]).astype(np.float32)
+    w[:, 3] = 0.0  # an all-zero channel takes the minimum scale
+    bits = orc.to_bits(w, orc.F16)
+    wv = orc.from_bits(bits, orc.F16)
+    wq, s = orc.fp8_convert_weight_per_channel(bits, orc.F16)
+    want_s = np.maximum(np.abs(wv).max(axis=0) / np.float32(448.0), np.float32(1.0 / (448.0 * 512.0))).astype(np.float32)
+    assert np.array_equal(s, want_s)
+    ratio = np.clip((wv.T / want_s[:, None]).astype(np.float32), -448.0, 448.0)
+    want_q = orc.e4m3_encode(ratio.reshape(-1)).reshape(N, K)
+    assert np.array_equal(wq & 0x7F, want_q & 0x7F)
+    nz = (want_q & 0x7F) != 0
+    assert np.array_equal(wq[nz], want_q[nz])
+    # dequantised values are within half an e4m3 step (2^-4 relative) of the source
+    back = orc.e4m3_decode(wq.reshape(-1)).reshape(N, K) * s[:, None]
+    assert np.all(np.abs(back - wv.T) <= np.abs(wv.T) * 2.0**-4 + s[:, None] * 2.0**-10)
+
+
+def test_merge_qkv_max_matches_requantisation_of_the_parts():
+    """The max merge of KS/models/quant/quant_weight.cpp:816-897 on synthetic parts: the merged scale is the maximum,
+    the part that owns it is unchanged, the others are e4m3(value * ratio)."""
+    rng = np.random.default_rng(78)
+    nq, nk, nv, K = 8, 4, 4, 32
+    wq = rng.integers(0, 256, size=(nq + nk + nv, K), dtype=np.uint8)
+    wq[(wq & 0x7F) == 0x7F] = 0x11
+    sq, sk, sv = np.float32(0.02), np.float32(0.05), np.float32(0.0125)
+    merged, s = orc.fp8_merge_qkv_max(wq, sq, sk, sv, nq, nk, nv)
+    assert s.shape == (1,) and s[0] == sk
+    assert np.array_equal(merged[nq:nq + nk], wq[nq:nq + nk])
+    vals = orc.e4m3_decode(wq[:nq].reshape(-1)) * np.float32(sq / sk)
+    want = orc.e4m3_encode(vals.astype(np.float32)).reshape(nq, K)
+    nz = (want & 0x7F) != 0
+    assert np.array_equal(merged[:nq][nz], want[nz])
+    # v: ratio 0.25 is a power of two, so every normal value moves exactly
+    v_in = orc.e4m3_decode(wq[nq + nk:].reshape(-1))
+    v_out = orc.e4m3_decode(merged[nq + nk:].reshape(-1))
+    normal = np.abs(v_in) >= 2.0**-4
+    assert np.array_equal(v_out[normal], v_in[normal] * 0.25)
