@@ -472,22 +472,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
     __builtin_amdgcn_sched_barrier(0);
     u32x4 a0[kRows], a1[kRows];
     read_step(a0, cur, 0);
+    // The dequantisation of 32-k step ks + 1 is spread between the MFMAs of step ks (one column tile after each row
+    // of MFMAs): a wave that has a SIMD to itself then runs the vector ALU under the matrix pipeline instead of
+    // before it.
+    u32x4 b[2][KNT];
+#pragma unroll
+    for (int t = 0; t < KNT; ++t) {
+      const typename DQ::Consts k = DQ::prepare(bt.sz[t][0]);
+      b[0][t] = DQ::run(bt.w[t][0], k, m_lo, m_hi, g_lo, g_hi);
+    }
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      u32x4 b[KNT];
-#pragma unroll
-      for (int t = 0; t < KNT; ++t) {
-        const typename DQ::Consts k = DQ::prepare(bt.sz[t][GPT == 2 ? (ks >> 1) : 0]);
-        b[t] = DQ::run(bt.w[t][ks], k, m_lo, m_hi, g_lo, g_hi);
-      }
       if (ks < 3) read_step((ks & 1) ? a0 : a1, cur, ks + 1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mt = 0; mt < kRows; ++mt) {
         const u32x4 af = (ks & 1) ? a1[mt] : a0[mt];
 #pragma unroll
-        for (int t = 0; t < KNT; ++t) acc[mt][t] = O::mfma(af, b[t], acc[mt][t]);
+        for (int t = 0; t < KNT; ++t) acc[mt][t] = O::mfma(af, b[ks & 1][t], acc[mt][t]);
+        if (ks < 3 && mt < KNT) {
+          const typename DQ::Consts k = DQ::prepare(bt.sz[mt][GPT == 2 ? ((ks + 1) >> 1) : 0]);
+          b[(ks + 1) & 1][mt] = DQ::run(bt.w[mt][ks + 1], k, m_lo, m_hi, g_lo, g_hi);
+        }
         if constexpr (kSteady) load_item(dst, bn, kt + 3, ks, mt);  // tile kt + 3, one load per four MFMAs
+#pragma unroll
+        for (int t = 0; t < KNT; ++t) {  // one MFMA, then its share of the vector work
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, (20 + KNT - 1) / KNT, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
