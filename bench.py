@@ -7,7 +7,8 @@ fp16 activations N(0,1)) at M = 16 tokens.  Consecutive steps use different laye
 ~830 MB) so that no launch re-reads weights that are still resident in the 256 MB last-level cache.  All inputs
 are resident in HBM before the timed region; the K timed steps are one HIP graph on one stream, bracketed by
 events on that stream.  `extra` carries the other regimes of the path: the same layer at M = 64, the prefill kernel
-at M = 4096 (bf16 and fp16), and the FP8 GEMM at the Qwen-72B shapes (M = 1, 64, 2048).
+at M = 512, 2048 and 4096 (bf16; fp16 at 4096), the FP8 GEMM at the Qwen-72B shapes (M = 1, 64, 2048) and
+the GPTQ Llama-2-70B shapes (M = 1, 32, 256).
 
 Prints ONE JSON line: value = whole-job algorithmic GB/s, plus `roofline` for the dominant kernel (the W4A16
 k-stationary decode kernel) and `cpu_baseline` (the CPU oracle -- dequantize to fp32 + blocked OpenMP GEMM -- timed on the
@@ -183,9 +184,12 @@ def main():
                                             *workspace_for(torch, capi, dev, 64), stream, 64, dtype)
         extra["prefill_m4096"] = prefill(torch, capi, layers[0], dev, stream)
         extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], dev, stream, "f16")
+        extra["prefill_m2048"] = prefill(torch, capi, layers[0], dev, stream, M=2048)
+        extra["prefill_m512"] = prefill(torch, capi, layers[0], dev, stream, M=512)
         del layers[1:]
         torch.cuda.empty_cache()
         extra["fp8_cfg4"] = fp8_sweep(torch, capi, dev, stream)
+        extra["gptq_70b_cfg3"] = gptq_70b_sweep(torch, capi, dev, stream)
     if not args.no_cpu:
         result["cpu_baseline"], extra["parity_vs_cpu"] = cpu_baseline(np, torch, capi, layers[0], acts, outs,
                                                                       workspace, ws_bytes, M, dtype, step_bytes)
@@ -246,6 +250,52 @@ def fp8_sweep(torch, capi, dev, stream):
     return table
 
 
+def gptq_70b_sweep(torch, capi, dev, stream):
+    """configs[3]: symmetric GPTQ int4 g=128, fp16, the Llama-2-70B shapes at M = 1, 32 (HBM-bound: GB/s against the
+    HBM peak) and 256 (TFLOP/s against the dense MFMA peak)."""
+    shapes = [("qkv", 8192, 10240), ("o", 8192, 8192), ("gate_up", 8192, 57344), ("down", 28672, 8192)]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    table = {}
+    for name, k, n in shapes:
+        g = k // GROUP
+        ncopies = max(1, min(4, (600 << 20) // (k * n // 2)))
+        ws = []
+        for _ in range(ncopies):
+            qweight = torch.randint(-2**31, 2**31 - 1, (k // 8, n), dtype=torch.int32, device=dev, generator=gen)
+            scales = (torch.randn((g, n), device=dev, generator=gen).abs() * 0.02 + 1e-3).to(torch.float16)
+            wb, sb = capi.w4a16_repack_sizes(k, n, GROUP)
+            w = torch.empty(wb, dtype=torch.uint8, device=dev)
+            sz = torch.empty(sb // 4, dtype=torch.int32, device=dev)
+            capi.w4a16_repack(capi.W4_GPTQ_INT32_KPACK, qweight, capi.ZERO_NONE, None, scales, capi.F16, k, n, GROUP, w, sz)
+            ws.append((w, sz))
+            del qweight, scales
+        torch.cuda.synchronize()
+        row = {}
+        for M in (1, 32, 256):
+            act = torch.randn((M, k), device=dev, generator=gen).to(torch.float16)
+            out = torch.empty((M, n), dtype=torch.float16, device=dev)
+            wsb = capi.w4a16_workspace_bytes(M, n, k)
+            wk = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+
+            def launch(i):
+                w, sz = ws[i % ncopies]
+                capi.w4a16_gemm(capi.F16, out, act, w, sz, M, n, k, GROUP, wk, wsb, stream.cuda_stream)
+
+            us = time_graph(torch, stream, launch, 16)
+            if M <= 32:
+                b = w4a16_bytes(M, k, n, awq=False)
+                row[f"m{M}"] = {"us": round(us, 1), "GBps": round(b / us / 1e3, 1), "frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 3)}
+            else:
+                tf = 2.0 * M * k * n / us / 1e6
+                row[f"m{M}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1), "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+            del act, out, wk
+        table[name] = row
+        del ws
+        torch.cuda.empty_cache()
+    return table
+
+
 def time_graph(torch, stream, launch, count):
     """Average device time per launch (us) of `count` back-to-back launches replayed as one graph."""
     with torch.cuda.stream(stream):
@@ -279,10 +329,10 @@ def per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, d
     return table
 
 
-def prefill(torch, capi, layer, dev, stream, dtype_name="bf16"):
-    """configs[2] at M = 4096 (bf16 activations): TFLOP/s per shape against the dense MFMA peak.  The weights are
-    the fp16-scaled set of layer 0 re-used with bf16 activations only for timing (the arithmetic is the same)."""
-    M = 4096
+def prefill(torch, capi, layer, dev, stream, dtype_name="bf16", M=4096):
+    """configs[2] (bf16 activations, M = 512 / 2048 / 4096): TFLOP/s per shape against the dense MFMA peak.  The
+    weights are the fp16-scaled set of layer 0 re-used with bf16 activations only for timing (the arithmetic is the
+    same)."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(11)
     table = {}
