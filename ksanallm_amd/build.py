@@ -9,7 +9,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libksq.so")
 
-SOURCES = ["ksq_api.hip", "ksq_repack.hip", "ksq_w4a16_stream.hip", "ksq_w4a16_kstat.hip", "ksq_w4a16_prefill.hip", "ksq_fp8.hip", "ksq_fp8_kstat.hip", "ksq_fp8_prefill.hip"]
+SOURCES = ["ksq_api.hip", "ksq_repack.hip", "ksq_w4a16_stream.hip", "ksq_w4a16_kstat.hip", "ksq_w4a16_astream.hip", "ksq_w4a16_prefill.hip", "ksq_fp8.hip", "ksq_fp8_kstat.hip", "ksq_fp8_prefill.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -235,6 +235,15 @@ int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, co
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g) &&
       (workspace ? workspace_bytes : 0) >= w4a16_prefill_workspace_bytes(dtype, m, k))
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, s);
+  if (w4a16_astream_supported(m, n, k)) {
+    // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
+    // never slower than the k-stationary one; with two it wins only while every workgroup gets one to four
+    // column tiles.
+    const size_t ntiles = n / kTileN;
+    const bool dflt = m > 32 || (ntiles > (size_t)di->cus && ntiles <= 4 * (size_t)di->cus);
+    if (env_int("KSQ_W4_ASTREAM", dflt ? 1 : 0) != 0)
+      return w4a16_launch_astream(dtype, out, act, weight, sz, m, n, k, g, di->cus, s);
+  }
   if (m <= (size_t)env_int("KSQ_W4_KSTAT_MAX_M", 64) && env_int("KSQ_W4_KSTAT", 1) != 0) {
     KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
     if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s);

@@ -128,6 +128,11 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
 int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
 
+// accumulator-stationary decode kernel for 17 <= m <= 64 (no workspace, K never split across workgroups)
+bool w4a16_astream_supported(size_t m, size_t n, size_t k);
+int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
+                         size_t n, size_t k, size_t g, int cus, hipStream_t s);
+
 struct Fp8KstatPlan {
   bool ok;        // the k-stationary kernel takes this shape (m <= 64)
   int mt;         // 16-row tiles (1, 2 or 4)

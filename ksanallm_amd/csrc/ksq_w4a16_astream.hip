@@ -1,0 +1,263 @@
+// W4A16 decode kernel for 17 <= M <= 64: accumulator-stationary, both operands streamed.
+//
+// With two to four 16-row tiles the activations of a decode step no longer fit into the registers of one workgroup
+// for the whole of K, so here nothing but the accumulators stays: a workgroup (8 waves, two per SIMD) owns CNT
+// column tiles for all of K, wave w owns a contiguous slice of the k tiles, and for every k tile of its slice it
+// streams the activation fragments of all MT row tiles (from the L2: every workgroup reads all activations once) and
+// the CNT weight tiles (from HBM, once per device), one k tile ahead for the weights and half a k tile ahead for the
+// activations.  No barrier and no LDS until the end, where the 8 k slices of every (column tile, row tile) are
+// summed through LDS in a fixed order.  K is never split across workgroups: no workspace, no fix-up pass.
+//
+// Activation loads put lane l on row l / 4 and 16-byte piece l % 4 of a 32-k step, so that every aligned group of
+// four lanes reads 64 contiguous bytes (the memory pipeline then takes four lanes per clock instead of one); a lane
+// permutation gives the MFMA operand layout (lane 16 j + c = row c, piece j).
+//
+// Arithmetic as in the other decode kernels: biased nibbles by bit operations, a correction MFMA with -(bias + z),
+// fp32 sums over 64 k scaled by s[g,n].
+#include <cstdlib>
+
+#include "ksq_internal.h"
+#include "ksq_w4a16_ops.h"
+
+namespace ksq {
+namespace {
+
+using namespace w4;
+
+struct AstreamArgs {
+  const void* weight;  // [ntiles][KT][64] x 16 B
+  const void* sz;      // [ntiles][G][16] x 4 B
+  const void* act;     // [M][K] T
+  void* out;           // [M][N] T
+  int M, N, K, KT, G, ntiles;
+};
+
+template <typename T, int GPT, int MT, int CNT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_astream_kernel(AstreamArgs p) {
+  using O = Ops<T>;
+  constexpr int kWaves = 8;
+  constexpr int kTiles = CNT * MT;  // output tiles of the workgroup
+  __shared__ f32x4 red[kTiles * kWaves * 64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, j = lane >> 4;
+  const int nt_begin = blockIdx.x * CNT;
+  int count = p.ntiles - nt_begin;
+  count = count < CNT ? count : CNT;
+  // k slice of this wave, rounded up to an even number of tiles (the loop below runs in pairs; tiles past the end
+  // are parked out of range and read as zero)
+  const int slice = (p.KT + kWaves - 1) / kWaves;
+  const int kt_begin = wave * slice;
+  int kt_end = kt_begin + slice;
+  kt_end = kt_end < p.KT ? kt_end : p.KT;
+
+  // Resources cover exactly this workgroup's column tiles: tiles past `count` read as zero without traffic.
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(p.weight) + (size_t)nt_begin * p.KT * 1024), 0,
+      count > 0 ? count * p.KT * 1024 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_sz = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(p.sz) + (size_t)nt_begin * p.G * 64), 0, count > 0 ? count * p.G * 64 : 0,
+      0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
+  const unsigned w_stride = (unsigned)p.KT * 1024u, sz_stride = (unsigned)p.G * 64u;
+  const unsigned w_lane = lane * 16u, sz_lane = c * 4u;
+  // loading lane: row l / 4 of the row tile, piece l % 4 of the 32-k step
+  unsigned a_row[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int row = 16 * mt + (lane >> 2);
+    a_row[mt] = row < p.M ? ((unsigned)row * p.K + 8u * (lane & 3)) * 2u : 0x80000000u;
+  }
+  const int from = (4 * c + j) * 4;  // lane 16 j + c takes what lane 4 c + j loaded
+
+  struct WTile {
+    u32x4 w[CNT];
+    uint32_t sz[CNT][GPT];
+  };
+  auto load_w = [&](WTile& t, int kt) {
+    const bool ok = kt < kt_end;
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      t.w[i] = __builtin_bit_cast(
+          u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, ok ? w_lane + kt * 1024u + i * w_stride : 0x80000000u, 0, 2));
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi)
+        t.sz[i][gi] = __builtin_amdgcn_raw_buffer_load_b32(
+            rs_sz, ok ? sz_lane + (kt * GPT + gi) * 64u + i * sz_stride : 0x80000000u, 0, 0);
+    }
+  };
+  // half h of k tile kt: 32-k steps 2h and 2h + 1 of all row tiles, as loaded (before the lane permutation)
+  auto load_a = [&](u32x4 (&a)[MT][2], int kt, int h) {
+    const bool ok = kt < kt_end;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int dd = 0; dd < 2; ++dd)
+        a[mt][dd] = __builtin_bit_cast(
+            u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                       rs_a, (ok && a_row[mt] != 0x80000000u) ? a_row[mt] + (kt * kTileK + 32 * (2 * h + dd)) * 2u : 0x80000000u,
+                       0, 0));
+  };
+  auto permute = [&](u32x4 (&a)[MT][2]) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int dd = 0; dd < 2; ++dd)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) a[mt][dd][q] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)a[mt][dd][q]);
+  };
+
+  uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
+  asm volatile("" : "+s"(m_lo));
+  asm volatile("" : "+v"(c_lo));
+  asm volatile("" : "+v"(c_hi));
+  asm volatile("" : "+v"(m_hi));
+
+  f32x4 acc[CNT][MT];
+#pragma unroll
+  for (int i = 0; i < CNT; ++i)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[i][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // 64 k of all column tiles against all row tiles
+  auto compute_half = [&](const u32x4 (&a)[MT][2], const WTile& t, int h) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+      const uint32_t szw = t.sz[i][GPT == 2 ? h : 0];
+      const uint32_t z = szw >> 16;
+      const u32x4 corr = O::correction(z | (z << 16));
+      const float s = O::scale_to_float(szw);
+      f32x4 P[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dd = 0; dd < 2; ++dd) {
+        const u32x4 bw = O::unpack(t.w[i][2 * h + dd], m_lo, m_hi, c_lo, c_hi);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) P[mt] = O::mfma(a[mt][dd], corr, P[mt]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) P[mt] = O::mfma(a[mt][dd], bw, P[mt]);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][mt][e] += s * P[mt][e];
+    }
+  };
+
+  // One k tile: its weights (wc) and first activation half (a0) were requested a step earlier; request the second
+  // half, the next tile's weights and first half, and run the two halves.
+  u32x4 a0[MT][2], a1[MT][2];
+  WTile w0, w1;
+  auto tile = [&](WTile& wc, WTile& wn, int kt, int kt_next) {
+    load_a(a1, kt, 1);
+    load_w(wn, kt_next);
+    __builtin_amdgcn_sched_barrier(0);
+    permute(a0);
+    compute_half(a0, wc, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_a(a0, kt_next, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    permute(a1);
+    compute_half(a1, wc, 1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  load_w(w0, kt_begin);
+  load_a(a0, kt_begin, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int kt = kt_begin; kt < kt_end; kt += 2) {
+    tile(w0, w1, kt, kt + 1);
+    tile(w1, w0, kt + 1, kt + 2);
+  }
+
+  // ---- sum the 8 k slices of every output tile (fixed order: deterministic), one tile per wave and turn
+#pragma unroll
+  for (int i = 0; i < CNT; ++i)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[((i * MT + mt) * kWaves + wave) * 64 + lane] = acc[i][mt];
+  __syncthreads();
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  for (int q = wave; q < kTiles; q += kWaves) {
+    const int i = q / MT, mt = q - i * MT;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) sum += red[(q * kWaves + ww) * 64 + lane];
+    if (i < count) {
+      const int col = (nt_begin + i) * 16 + c;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int row = 16 * mt + 4 * j + e;
+        if (row < p.M) out[(size_t)row * p.N + col] = O::to_bits(sum[e]);
+      }
+    }
+  }
+}
+
+template <typename T, int GPT>
+void launch(int mt, int cnt, const AstreamArgs& a, dim3 grid, hipStream_t s) {
+  const dim3 block(512);
+#define KSQ_GO(MT, CNT) hipLaunchKernelGGL((w4a16_astream_kernel<T, GPT, MT, CNT>), grid, block, 0, s, a)
+  if (mt <= 2) {
+    if (cnt == 1) KSQ_GO(2, 1);
+    else if (cnt == 2) KSQ_GO(2, 2);
+    else if (cnt == 3) KSQ_GO(2, 3);
+    else KSQ_GO(2, 4);
+  } else {
+    if (cnt == 1) KSQ_GO(4, 1);
+    else if (cnt == 2 || GPT == 2) KSQ_GO(4, 2);
+    else KSQ_GO(4, 3);
+  }
+#undef KSQ_GO
+}
+
+}  // namespace
+
+bool w4a16_astream_supported(size_t m, size_t n, size_t k) {
+  return m >= 17 && m <= 64 && m * k * 2 < 0x7FFFFF00ull && 4 * (k / kTileK) * 1024 < 0x7FFFFF00ull && n / kTileN < (1u << 30);
+}
+
+int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
+                         size_t n, size_t k, size_t g, int cus, hipStream_t s) {
+  AstreamArgs a{};
+  a.weight = weight;
+  a.sz = sz;
+  a.act = act;
+  a.out = out;
+  a.M = (int)m;
+  a.N = (int)n;
+  a.K = (int)k;
+  a.KT = (int)(k / kTileK);
+  a.G = (int)(k / g);
+  a.ntiles = (int)(n / kTileN);
+  // column tiles per workgroup: one workgroup per CU if that needs at most four, else the split into whole rounds
+  // of workgroups that wastes least
+  const int mt = m <= 32 ? 2 : 4;
+  const int gpt = (int)(kTileK / g);
+  const int cnt_max = mt == 2 ? 4 : (gpt == 1 ? 3 : 2);  // what 256 registers per lane hold without spilling
+  int cnt = (a.ntiles + cus - 1) / cus;
+  if (cnt > cnt_max) {
+    const int rounds = (a.ntiles + cnt_max * cus - 1) / (cnt_max * cus);
+    cnt = (a.ntiles + rounds * cus - 1) / (rounds * cus);
+  }
+  if (const char* e = getenv("KSQ_W4_ASTREAM_CNT")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v > 0) cnt = v;
+  }
+  if (cnt < 1) cnt = 1;
+  if (cnt > cnt_max) cnt = cnt_max;
+  dim3 grid((unsigned)((a.ntiles + cnt - 1) / cnt));
+  if (dtype == KSQ_F16) {
+    if (gpt == 1) launch<_Float16, 1>(mt, cnt, a, grid, s);
+    else launch<_Float16, 2>(mt, cnt, a, grid, s);
+  } else {
+    if (gpt == 1) launch<__bf16, 1>(mt, cnt, a, grid, s);
+    else launch<__bf16, 2>(mt, cnt, a, grid, s);
+  }
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+}  // namespace ksq

@@ -582,7 +582,12 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, 
 bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g) {
   (void)g;
   (void)dtype;
-  return m >= 65 && n % 16 == 0 && m * k * 2 < 0x7FFFFF00ull && (k / kTileK) * 1024 < 0x7FFFFF00ull;
+  size_t min_m = 65;
+  if (const char* e = getenv("KSQ_W4_PREFILL_MIN_M")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v >= 1) min_m = (size_t)v;
+  }
+  return m >= min_m && n % 16 == 0 && m * k * 2 < 0x7FFFFF00ull && (k / kTileK) * 1024 < 0x7FFFFF00ull;
 }
 
 // bf16 route: fp16 copy of the activations + one float per row

@@ -86,6 +86,18 @@ def test_m_sweep_small_shape(gpu, dtype, M):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("route", [0, 1])
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 64])
+def test_m_sweep_both_decode_routes(gpu, dtype, route, M):
+    """17 <= M <= 64 is served by the k-stationary kernel (two or four row tiles) or by the accumulator-stationary
+    one, chosen per shape: force each."""
+    case = W4Case(1050 + M, M, 1024, 320, kind="awq", dtype=dtype)
+    with _env(KSQ_W4_ASTREAM=route):
+        got = W4Device(case, gpu).gemm_f32()
+    orc.assert_parity(got, case.oracle(), f"M={M} {dtype} route={route}")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("kind,g", [("gptq", 128), ("gptq", 64), ("awq", 64)])
 def test_group_sizes_and_kinds(gpu, dtype, kind, g):
     case = W4Case(1100, 9, 768, 208, g=g, kind=kind, dtype=dtype)
@@ -144,6 +156,29 @@ def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
         got1 = dev.gemm_f32()
         got2 = dev.gemm_f32()
     orc.assert_parity(got1, case.oracle(), f"prefill rows={rows} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+
+
+@pytest.mark.parametrize("cnt", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 17, 640, 528),      # five k tiles over eight waves: three waves idle, odd slices
+    ("bf16", "awq", 128, 32, 1152, 272),    # nine k tiles: slices of two with a remainder
+    ("f16", "gptq", 64, 33, 384, 512),
+    ("bf16", "gptq", 64, 64, 128, 4112),    # a single k tile, more column tiles than compute units
+    ("f16", "awq", 64, 48, 2048, 1040),
+])
+def test_accumulator_stationary_route(gpu, cnt, dtype, kind, g, M, K, N):
+    """The 17 <= M <= 64 kernel that keeps only accumulators and streams both operands, with every number of column
+    tiles per workgroup (0 = the launcher's own choice); twice, bit for bit."""
+    case = W4Case(1300 + cnt + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    env = dict(KSQ_W4_ASTREAM=1)
+    if cnt:
+        env["KSQ_W4_ASTREAM_CNT"] = cnt
+    with _env(**env):
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"astream cnt={cnt} {dtype} {kind} g={g} M={M}")
     assert np.array_equal(got1, got2)
 
 
