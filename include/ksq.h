@@ -44,8 +44,39 @@ typedef enum ksq_w4_layout {
   /* ksana's canonical form after CutlassAutoUnpack: int8 [K, N/2], low nibble = even column, signed q = u - 8
    * (KS/models/quant/quant_weight.cpp:249-251, :304-328) -- the input of the CUTLASS preprocessor that this
    * repack replaces (LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508). */
-  KSQ_W4_ROWMAJOR_INT4_SIGNED = 2
+  KSQ_W4_ROWMAJOR_INT4_SIGNED = 2,
+  /* What the loader's CUTLASS back end leaves in the weight tensor on sm80..sm89: the output of
+   * preprocess_weights_for_mixed_gemm for W4_A16 (LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508):
+   * rows permuted inside groups of 32 (:129-197), transposed to column major with eight k per 32-bit register
+   * (:203-323), four columns interleaved per 64 rows (:426-464; ColumnMajorTileInterleave<64, 4>,
+   * LK/cutlass_extensions/gemm/kernel/mixed_gemm_B_layout.h:106-120), nibbles biased to unsigned and
+   * re-ordered [e0 e2 e4 e6 e1 e3 e5 e7] inside every register (:352-401).  Same byte count as the row-major
+   * form; needs K % 64 == 0 and N % 4 == 0. */
+  KSQ_W4_CUTLASS_SM80_INTERLEAVED = 3,
+  /* The same preprocessor's output on sm90 (only the transpose runs: :487-490; the bias step is skipped,
+   * :497-499): int8 [N, K/2], low nibble = even k, signed q = u - 8. */
+  KSQ_W4_CUTLASS_SM90_COLMAJOR = 4
 } ksq_w4_layout;
+
+/* Order of the columns in the repacked weight (and in its scale / zero words). */
+typedef enum ksq_column_order {
+  KSQ_COLS_NATURAL = 0,
+  /* The source tensor is two halves side by side, [gate | up] along N (N/2 columns each); destination column
+   * 2i is gate column i and 2i + 1 is up column i, which puts each pair into neighbouring lanes of one MFMA tile
+   * for KSQ_EPILOGUE_SILU_MUL. */
+  KSQ_COLS_HALVES_INTERLEAVED = 1
+} ksq_column_order;
+
+/* What the GEMMs do with the fp32 result before it is stored. */
+typedef enum ksq_epilogue {
+  KSQ_EPILOGUE_NONE = 0,
+  /* out[m,n] = T(acc[m,n] + bias[n]), bias is T [n] (qkv bias: KS/models/common/common_model.cpp:456-459) */
+  KSQ_EPILOGUE_BIAS = 1,
+  /* weight columns interleaved as KSQ_COLS_HALVES_INTERLEAVED; out is [m, n/2]:
+   * out[m,i] = T(silu(acc[m,2i]) * acc[m,2i+1]), silu(x) = x / (1 + exp(-x)), in fp32.  One GEMM instead of the
+   * reference's two plus its SiLU-mul layer (common_model.cpp:540-547). */
+  KSQ_EPILOGUE_SILU_MUL = 2
+} ksq_epilogue;
 
 /* How zero points are handed to the repack step. */
 typedef enum ksq_zero_kind {
@@ -96,6 +127,29 @@ int ksq_w4a16_repack_host(int src_layout, const void* qweight_host, int zero_kin
                           const void* scales_host, int scale_dtype, size_t k, size_t n, size_t group_size,
                           void* dst_weight_host, void* dst_sz_host);
 
+/* The repack with a row permutation and a column order.  row_perm (int32 [k], device memory for the device
+ * call; NULL = identity) makes destination row i hold source row row_perm[i]: with the permutation of
+ * ksq_gptq_act_order_perm the rows of a desc_act GPTQ checkpoint end up grouped, so that scales[i / g] is the
+ * scale of row i and the ordinary kernels apply; the activations' columns are permuted to match at run time
+ * (the scheme of the reference's Marlin back end: LK/gptq_marlin/gptq_marlin.cu:380-392).  Scales and zeros are
+ * indexed by group and are not permuted. */
+int ksq_w4a16_repack_ex(int src_layout, const void* qweight, int zero_kind, const void* zeros, const void* scales,
+                        int scale_dtype, size_t k, size_t n, size_t group_size, const int32_t* row_perm,
+                        int column_order, void* dst_weight, void* dst_sz, void* stream);
+int ksq_w4a16_repack_ex_host(int src_layout, const void* qweight_host, int zero_kind, const void* zeros_host,
+                             const void* scales_host, int scale_dtype, size_t k, size_t n, size_t group_size,
+                             const int32_t* row_perm_host, int column_order, void* dst_weight_host,
+                             void* dst_sz_host);
+
+/* perm = stable argsort of g_idx (MarlinSortGIdx, KS/models/quant/quant_weight.cpp:455-460), on the host.
+ * Fails with KSQ_ERR_UNSUPPORTED unless every group 0 .. k/g - 1 has exactly g rows, which is what lets the
+ * permuted tensor run on the kernels for grouped rows (the reference's is_k_full case, gptq_marlin.cu:386-392). */
+int ksq_gptq_act_order_perm(const int32_t* g_idx_host, size_t k, size_t group_size, int32_t* perm_host);
+
+/* out[m, i] = in[m, perm[i]] for a row-major [m, k] tensor of 16-bit elements (permute_cols_kernel,
+ * LK/gptq_marlin/gptq_marlin.cu:380-384). */
+int ksq_permute_columns(void* out, const void* in, const int32_t* perm, size_t m, size_t k, void* stream);
+
 /* ------------------------------------------------------------------ W4A16: GEMM
  *
  * Replaces InvokeFpAIntBGroupCudaGemm / InvokeFpAIntBGroupCutlassGemm and
@@ -114,6 +168,17 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
 
 int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
                    size_t k, size_t group_size, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same GEMM with the steps either side of it fused in:
+ *   act_perm (int32 [k] or NULL): the activations' columns are gathered through it first (desc_act weights
+ *     repacked with the same permutation); needs a workspace from ksq_w4a16_workspace_bytes_ex(.., 1, ..),
+ *     whose first m*k*2 bytes (rounded up to 256) hold the permuted copy -- without one the call fails with
+ *     KSQ_ERR_WORKSPACE;
+ *   epilogue / bias: see ksq_epilogue.  n is the width of the weight; out has n/2 columns for SILU_MUL. */
+int ksq_w4a16_workspace_bytes_ex(size_t max_m, size_t n, size_t k, int act_order, size_t* bytes);
+int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
+                      size_t n, size_t k, size_t group_size, const int32_t* act_perm, int epilogue,
+                      const void* bias, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ FP8 e4m3 (OCP: bias 7, max 448, no inf)
  *
@@ -157,6 +222,18 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
 int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                  const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same GEMM with an epilogue (see ksq_epilogue).  For KSQ_EPILOGUE_SILU_MUL the rows of w_q (and, when there
+ * are n of them, its scales) are interleaved gate / up: row 2i = gate row i, row 2i + 1 = up row i
+ * (ksq_interleave_halves builds that from [gate ; up]); out is [m, n/2]. */
+int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                    const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                    int epilogue, const void* bias, void* workspace, size_t workspace_bytes, void* stream);
+
+/* out row 2i = in row i, out row 2i + 1 = in row rows/2 + i, for rows of row_bytes bytes (rows even, row_bytes a
+ * multiple of 4; in and out must not overlap).  Load-time helper for the interleaved gate / up weight and its
+ * per-channel scales (row_bytes = 4). */
+int ksq_interleave_halves(void* out, const void* in, size_t rows, size_t row_bytes, void* stream);
 
 #ifdef __cplusplus
 }

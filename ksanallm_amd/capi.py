@@ -13,6 +13,9 @@ LIB_PATH = os.path.join(_HERE, "libksq.so")
 # enums of include/ksq.h
 F16, BF16 = 0, 1
 W4_GPTQ_INT32_KPACK, W4_AWQ_INT32_NPACK, W4_ROWMAJOR_INT4_SIGNED = 0, 1, 2
+W4_CUTLASS_SM80_INTERLEAVED, W4_CUTLASS_SM90_COLMAJOR = 3, 4
+COLS_NATURAL, COLS_HALVES_INTERLEAVED = 0, 1
+EPILOGUE_NONE, EPILOGUE_BIAS, EPILOGUE_SILU_MUL = 0, 1, 2
 ZERO_NONE, ZERO_AWQ_INT32, ZERO_UINT8, ZERO_ADDITIVE = 0, 1, 2, 3
 FP8_PER_TENSOR_DYNAMIC, FP8_PER_TENSOR_STATIC, FP8_PER_TOKEN_DYNAMIC = 0, 1, 2
 FP8_MERGE_MAX, FP8_MERGE_PER_CHANNEL = 0, 1
@@ -24,6 +27,8 @@ EXPORTS = [
     "ksq_w4a16_workspace_bytes", "ksq_w4a16_gemm",
     "ksq_fp8_quantize", "ksq_fp8_rescale", "ksq_fp8_convert_weight",
     "ksq_fp8_convert_weight_per_channel", "ksq_fp8_merge_qkv_scales", "ksq_fp8_workspace_bytes", "ksq_fp8_gemm",
+    "ksq_w4a16_repack_ex", "ksq_w4a16_repack_ex_host", "ksq_gptq_act_order_perm", "ksq_permute_columns",
+    "ksq_w4a16_workspace_bytes_ex", "ksq_w4a16_gemm_ex", "ksq_fp8_gemm_ex", "ksq_interleave_halves",
 ]
 
 
@@ -60,6 +65,14 @@ def lib():
         L.ksq_fp8_merge_qkv_scales.argtypes = [ci, vp, vp, vp, sz, sz, sz, vp, sz, vp, vp]
         L.ksq_fp8_workspace_bytes.argtypes = [sz, sz, sz, psz]
         L.ksq_fp8_gemm.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, vp, sz, vp]
+        L.ksq_w4a16_repack_ex.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, ci, vp, vp, vp]
+        L.ksq_w4a16_repack_ex_host.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, ci, vp, vp]
+        L.ksq_gptq_act_order_perm.argtypes = [vp, sz, sz, vp]
+        L.ksq_permute_columns.argtypes = [vp, vp, vp, sz, sz, vp]
+        L.ksq_w4a16_workspace_bytes_ex.argtypes = [sz, sz, sz, ci, psz]
+        L.ksq_w4a16_gemm_ex.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, ci, vp, vp, sz, vp]
+        L.ksq_fp8_gemm_ex.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
+        L.ksq_interleave_halves.argtypes = [vp, vp, sz, sz, vp]
         for name in EXPORTS:
             if name not in ("ksq_last_error_string",):
                 getattr(L, name).restype = ci
@@ -110,6 +123,45 @@ def w4a16_repack_host(src_layout, qweight, zero_kind, zeros, scales, scale_dtype
                                        scale_dtype, k, n, group_size, _addr(dst_weight), _addr(dst_sz)))
 
 
+def w4a16_repack_ex(src_layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, group_size, row_perm,
+                    column_order, dst_weight, dst_sz, stream=None):
+    _check(lib().ksq_w4a16_repack_ex(src_layout, _addr(qweight), zero_kind, _addr(zeros), _addr(scales), scale_dtype,
+                                     k, n, group_size, _addr(row_perm), column_order, _addr(dst_weight),
+                                     _addr(dst_sz), stream))
+
+
+def w4a16_repack_ex_host(src_layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, group_size, row_perm,
+                         column_order, dst_weight, dst_sz):
+    _check(lib().ksq_w4a16_repack_ex_host(src_layout, _addr(qweight), zero_kind, _addr(zeros), _addr(scales),
+                                          scale_dtype, k, n, group_size, _addr(row_perm), column_order,
+                                          _addr(dst_weight), _addr(dst_sz)))
+
+
+def gptq_act_order_perm(g_idx, k, group_size, perm):
+    """Host arrays (numpy int32) in, host array out."""
+    _check(lib().ksq_gptq_act_order_perm(_addr(g_idx), k, group_size, _addr(perm)))
+
+
+def permute_columns(out, src, perm, m, k, stream=None):
+    _check(lib().ksq_permute_columns(_addr(out), _addr(src), _addr(perm), m, k, stream))
+
+
+def interleave_halves(out, src, rows, row_bytes, stream=None):
+    _check(lib().ksq_interleave_halves(_addr(out), _addr(src), rows, row_bytes, stream))
+
+
+def w4a16_workspace_bytes_ex(max_m, n, k, act_order):
+    b = ctypes.c_size_t(0)
+    _check(lib().ksq_w4a16_workspace_bytes_ex(max_m, n, k, int(bool(act_order)), ctypes.byref(b)))
+    return b.value
+
+
+def w4a16_gemm_ex(dtype, out, act, weight, sz, m, n, k, group_size, act_perm=None, epilogue=EPILOGUE_NONE, bias=None,
+                  workspace=None, workspace_bytes=0, stream=None):
+    _check(lib().ksq_w4a16_gemm_ex(dtype, _addr(out), _addr(act), _addr(weight), _addr(sz), m, n, k, group_size,
+                                   _addr(act_perm), epilogue, _addr(bias), _addr(workspace), workspace_bytes, stream))
+
+
 def w4a16_workspace_bytes(max_m, n, k):
     b = ctypes.c_size_t(0)
     _check(lib().ksq_w4a16_workspace_bytes(max_m, n, k, ctypes.byref(b)))
@@ -152,3 +204,10 @@ def fp8_gemm(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_
              workspace_bytes=0, stream=None):
     _check(lib().ksq_fp8_gemm(out_dtype, _addr(out), _addr(act_q), _addr(act_scale), act_scale_count, _addr(w_q),
                               _addr(w_scale), w_scale_count, m, n, k, _addr(workspace), workspace_bytes, stream))
+
+
+def fp8_gemm_ex(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
+                epilogue=EPILOGUE_NONE, bias=None, workspace=None, workspace_bytes=0, stream=None):
+    _check(lib().ksq_fp8_gemm_ex(out_dtype, _addr(out), _addr(act_q), _addr(act_scale), act_scale_count, _addr(w_q),
+                                 _addr(w_scale), w_scale_count, m, n, k, epilogue, _addr(bias), _addr(workspace),
+                                 workspace_bytes, stream))

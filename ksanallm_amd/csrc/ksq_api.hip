@@ -217,24 +217,52 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
   return KSQ_OK;
 }
 
-int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
-                   size_t k, size_t g, void* workspace, size_t workspace_bytes, void* stream) {
+int ksq_w4a16_workspace_bytes_ex(size_t max_m, size_t n, size_t k, int act_order, size_t* bytes) {
+  int rc = ksq_w4a16_workspace_bytes(max_m, n, k, bytes);
+  if (rc != KSQ_OK) return rc;
+  if (act_order) *bytes += (max_m * k * 2 + 255) / 256 * 256;  // the permuted copy of the activations, in front
+  return KSQ_OK;
+}
+
+int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                      size_t k, size_t g, const int32_t* act_perm, int epilogue, const void* bias, void* workspace,
+                      size_t workspace_bytes, void* stream) {
   KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
   KSQ_REQUIRE(out && act && weight && sz, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
+              "bad epilogue %d", epilogue);
+  KSQ_REQUIRE(epilogue != KSQ_EPILOGUE_BIAS || (bias && (reinterpret_cast<uintptr_t>(bias) & 15) == 0),
+              KSQ_ERR_INVALID_ARGUMENT, "the bias epilogue needs a 16-byte aligned bias");
   int rc = check_w4_shape(k, n, g);
   if (rc != KSQ_OK) return rc;
   if (m == 0) return KSQ_OK;
   KSQ_REQUIRE(m < (1u << 24), KSQ_ERR_UNSUPPORTED, "m=%zu too large", m);
   KSQ_REQUIRE((reinterpret_cast<uintptr_t>(act) & 15) == 0 && (reinterpret_cast<uintptr_t>(weight) & 15) == 0 &&
-                  (reinterpret_cast<uintptr_t>(sz) & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 1) == 0,
+                  (reinterpret_cast<uintptr_t>(sz) & 3) == 0 &&
+                  (reinterpret_cast<uintptr_t>(out) & (epilogue == KSQ_EPILOGUE_SILU_MUL ? 7 : 1)) == 0,
               KSQ_ERR_INVALID_ARGUMENT, "act and weight must be 16-byte aligned");
   const DeviceInfo* di = device_info();
   if (!di) return KSQ_ERR_HIP;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) workspace = nullptr;
+  if (!workspace) workspace_bytes = 0;
+  if (act_perm) {
+    const size_t need = (m * k * 2 + 255) / 256 * 256;
+    KSQ_REQUIRE(workspace_bytes >= need, KSQ_ERR_WORKSPACE,
+                "act_perm needs %zu bytes of 256-byte aligned workspace for the permuted activations", need);
+    rc = ksq_permute_columns(workspace, act, act_perm, m, k, stream);
+    if (rc != KSQ_OK) return rc;
+    act = workspace;
+    workspace = static_cast<char*>(workspace) + need;
+    workspace_bytes -= need;
+    if (workspace_bytes == 0) workspace = nullptr;
+  }
+  Epilogue epi;
+  epi.kind = epilogue;
+  epi.bias = bias;
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g) &&
-      (workspace ? workspace_bytes : 0) >= w4a16_prefill_workspace_bytes(dtype, m, k))
-    return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, s);
+      workspace_bytes >= w4a16_prefill_workspace_bytes(dtype, m, k))
+    return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, s, epi);
   if (w4a16_astream_supported(m, n, k)) {
     // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
     // never slower than the k-stationary one; with two it wins only while every workgroup gets one to four
@@ -242,14 +270,20 @@ int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, co
     const size_t ntiles = n / kTileN;
     const bool dflt = m > 32 || (ntiles > (size_t)di->cus && ntiles <= 4 * (size_t)di->cus);
     if (env_int("KSQ_W4_ASTREAM", dflt ? 1 : 0) != 0)
-      return w4a16_launch_astream(dtype, out, act, weight, sz, m, n, k, g, di->cus, s);
+      return w4a16_launch_astream(dtype, out, act, weight, sz, m, n, k, g, di->cus, s, epi);
   }
   if (m <= (size_t)env_int("KSQ_W4_KSTAT_MAX_M", 64) && env_int("KSQ_W4_KSTAT", 1) != 0) {
-    KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
-    if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s);
+    KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace_bytes);
+    if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s, epi);
   }
-  W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
-  return w4a16_launch_stream(dtype, plan, out, act, weight, sz, m, n, k, g, workspace, s);
+  W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace_bytes);
+  return w4a16_launch_stream(dtype, plan, out, act, weight, sz, m, n, k, g, workspace, s, epi);
+}
+
+int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                   size_t k, size_t g, void* workspace, size_t workspace_bytes, void* stream) {
+  return ksq_w4a16_gemm_ex(dtype, out, act, weight, sz, m, n, k, g, nullptr, KSQ_EPILOGUE_NONE, nullptr, workspace,
+                           workspace_bytes, stream);
 }
 
 }  // extern "C"

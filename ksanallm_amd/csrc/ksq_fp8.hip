@@ -1,6 +1,7 @@
 // FP8 e4m3 (OCP) path: activation quantisation, rescale, on-the-fly weight conversion and the streaming GEMM.
 #include <cstdlib>
 
+#include "ksq_epilogue.h"
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -311,6 +312,7 @@ struct Fp8Args {
   unsigned* counters;
   int M, N, K, KB /* 128-byte k blocks, rounded up */, ntiles, ksplit;
   int a_scale_per_row, w_scale_per_col;
+  Epilogue epi;
 };
 
 // Wave = one 16-column tile x a range of 128-k blocks.  Each lane reads 2 x 16 B of its weight row per block (the
@@ -387,14 +389,13 @@ __global__ __launch_bounds__(256) void fp8_stream_kernel(Fp8Args p) {
   const int col = nt * 16 + c;
   const float ws = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
   auto store_out = [&](int mt, f32x4 v) {
+    const int row0 = m0 + 16 * mt + 4 * j;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = m0 + 16 * mt + 4 * j + i;
-      if (row < p.M && col < p.N) {
-        const float as = p.a_scale[p.a_scale_per_row ? row : 0];
-        out[(size_t)row * p.N + col] = float_to_bits<T>((v[i] * ws) * as);
-      }
+      const int row = row0 + i;
+      v[i] = (v[i] * ws) * p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
     }
+    epi_store_acc<T>(p.epi, out, v, row0, col, p.M, p.N, col < p.N);
   };
 
   if (p.ksplit == 1) {
@@ -625,6 +626,22 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
 int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                  const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
                  void* workspace, size_t workspace_bytes, void* stream) {
+  return ksq_fp8_gemm_ex(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
+                         KSQ_EPILOGUE_NONE, nullptr, workspace, workspace_bytes, stream);
+}
+
+int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                    const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                    int epilogue, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+  KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
+              "bad epilogue %d", epilogue);
+  KSQ_REQUIRE(epilogue != KSQ_EPILOGUE_BIAS || (bias && (reinterpret_cast<uintptr_t>(bias) & 15) == 0),
+              KSQ_ERR_INVALID_ARGUMENT, "the bias epilogue needs a 16-byte aligned bias");
+  KSQ_REQUIRE(epilogue != KSQ_EPILOGUE_SILU_MUL || n % 16 == 0, KSQ_ERR_UNSUPPORTED,
+              "the SiLU-mul epilogue needs n %% 16 == 0 (got %zu)", n);
+  Epilogue epi;
+  epi.kind = epilogue;
+  epi.bias = bias;
   KSQ_REQUIRE(out_dtype == KSQ_F16 || out_dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", out_dtype);
   KSQ_REQUIRE(out && act_q && w_q, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
   // the reference layer refuses a missing weight scale (KS/layers/nvidia/fp8_matmul_layer.cpp:49-51)
@@ -643,7 +660,7 @@ int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_s
   if (!di) return KSQ_ERR_HIP;
   if (fp8_prefill_supported(m, n, k) && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
     return fp8_launch_prefill(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
-                              static_cast<hipStream_t>(stream));
+                              static_cast<hipStream_t>(stream), epi);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
   if (m <= 64) {
     const char* e = getenv("KSQ_FP8_KSTAT");  // tuning / test switch: 0 sends small m to the streaming kernel
@@ -651,11 +668,12 @@ int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_s
       const Fp8KstatPlan kp = fp8_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
       if (kp.ok)
         return fp8_launch_kstat(out_dtype, kp, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m,
-                                n, k, workspace, static_cast<hipStream_t>(stream));
+                                n, k, workspace, static_cast<hipStream_t>(stream), epi);
     }
   }
   Fp8Plan plan = fp8_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
   Fp8Args a{};
+  a.epi = epi;
   a.aq = static_cast<const uint8_t*>(act_q);
   a.wq = static_cast<const uint8_t*>(w_q);
   a.a_scale = act_scale;

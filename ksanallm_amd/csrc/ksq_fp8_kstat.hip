@@ -12,6 +12,7 @@
 // both sides (K is a multiple of 16).  out = T(acc * w_scale[n] * a_scale[m]).
 #include <cstdlib>
 
+#include "ksq_epilogue.h"
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -31,6 +32,7 @@ struct Fp8KstatArgs {
   unsigned* counters;  // [ntiles][MT]
   int M, N, K, KS /* stages, rounded up */, ntiles, ksplit, nt_per_wg;
   int a_scale_per_row, w_scale_per_col;
+  Epilogue epi;
 };
 
 template <typename T>
@@ -213,18 +215,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
         }
       }
       if (store) {
-        const int col = nt * 16 + r;
-        if (col < p.N) {
-          const float ws = p.w_scale[p.w_scale_per_col ? col : 0];
+        const int col = nt * 16 + r, row0 = 16 * mt + 4 * j;
+        const float ws = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int row = 16 * mt + 4 * j + e;
-            if (row < p.M) {
-              const float as = p.a_scale[p.a_scale_per_row ? row : 0];
-              out[(size_t)row * p.N + col] = out_bits<T>(sum[e] * ws * as);
-            }
-          }
+        for (int e = 0; e < 4; ++e) {
+          const int row = row0 + e;
+          sum[e] = sum[e] * ws * p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
         }
+        epi_store_acc<T>(p.epi, out, sum, row0, col, p.M, p.N, col < p.N);
       }
     }
   }
@@ -314,10 +312,11 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
 
 int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const void* act_q, const float* act_scale,
                      size_t act_scale_count, const void* w_q, const float* w_scale, size_t w_scale_count, size_t m,
-                     size_t n, size_t k, void* workspace, hipStream_t s) {
+                     size_t n, size_t k, void* workspace, hipStream_t s, const Epilogue& epi) {
   KSQ_REQUIRE(((size_t)plan.nt_per_wg + 8) * 16 * k < 0x3FFFFF00ull, KSQ_ERR_UNSUPPORTED,
               "column range of one workgroup larger than 1 GiB");
   Fp8KstatArgs a{};
+  a.epi = epi;
   a.aq = static_cast<const uint8_t*>(act_q);
   a.wq = static_cast<const uint8_t*>(w_q);
   a.a_scale = act_scale;

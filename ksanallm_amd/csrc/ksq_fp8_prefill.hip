@@ -11,6 +11,7 @@
 // group covers 64 contiguous bytes of a row.  K must be a multiple of 128 (other K take the streaming kernel).
 #include <cstdlib>
 
+#include "ksq_epilogue.h"
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -29,6 +30,7 @@ struct Fp8PrefillArgs {
   void* out;
   int M, N, K, KS /* 128-byte k stages */, mblocks, nblocks, super_n;
   int a_scale_per_row, w_scale_per_col;
+  Epilogue epi;
 };
 
 constexpr int kBM = 128, kBN = 256, kMT = 8, kNT = 4;
@@ -192,11 +194,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
       const float* src = epi + rr * kEpiStride + cc;
       const int row = m0 + 16 * mt + rr, col = n0 + cc;
       const float as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
-      u32x4 packed;
+      float vals[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        packed[q] = (uint32_t)out_bits<T>(src[2 * q] * as) | ((uint32_t)out_bits<T>(src[2 * q + 1] * as) << 16);
-      if (row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+      for (int q = 0; q < 8; ++q) vals[q] = src[q] * as;
+      if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
   }
 }
@@ -336,11 +337,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       const float* src = epi + rr * kEpiStride + cc;
       const int row = mw + 16 * mt + rr, col = nw + cc;
       const float as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
-      u32x4 packed;
+      float vals[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        packed[q] = (uint32_t)out_bits<T>(src[2 * q] * as) | ((uint32_t)out_bits<T>(src[2 * q + 1] * as) << 16);
-      if (row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+      for (int q = 0; q < 8; ++q) vals[q] = src[q] * as;
+      if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -354,9 +354,10 @@ bool fp8_prefill_supported(size_t m, size_t n, size_t k) {
 
 int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                        const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
-                       hipStream_t s) {
+                       hipStream_t s, const Epilogue& epi) {
   KSQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0, KSQ_ERR_INVALID_ARGUMENT, "output must be 16-byte aligned");
   Fp8PrefillArgs a{};
+  a.epi = epi;
   a.aq = static_cast<const uint8_t*>(act_q);
   a.wq = static_cast<const uint8_t*>(w_q);
   a.a_scale = act_scale;

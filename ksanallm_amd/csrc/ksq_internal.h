@@ -93,6 +93,12 @@ struct DeviceInfo {
 };
 const DeviceInfo* device_info();  // of the current device; nullptr on failure
 
+// What a GEMM does with its fp32 result on the way out (ksq_epilogue in include/ksq.h).
+struct Epilogue {
+  int kind = KSQ_EPILOGUE_NONE;
+  const void* bias = nullptr;  // T [n], 16-byte aligned
+};
+
 // ---- launch plans ------------------------------------------------------------------------------------------
 struct W4Plan {
   int MT;       // 16-row tiles per wave (1..4)
@@ -106,9 +112,11 @@ struct W4Plan {
 W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
 
 int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
-                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                        const Epilogue& epi = Epilogue());
 int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                        const Epilogue& epi = Epilogue());
 size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k);
 bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g);
 int w4a16_stream_max_slices(int mt, int nt);
@@ -126,12 +134,14 @@ struct KstatPlan {
 };
 KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
 int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
-                       const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s);
+                       const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                        const Epilogue& epi = Epilogue());
 
 // accumulator-stationary decode kernel for 17 <= m <= 64 (no workspace, K never split across workgroups)
 bool w4a16_astream_supported(size_t m, size_t n, size_t k);
 int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, int cus, hipStream_t s);
+                         size_t n, size_t k, size_t g, int cus, hipStream_t s,
+                         const Epilogue& epi = Epilogue());
 
 struct Fp8KstatPlan {
   bool ok;        // the k-stationary kernel takes this shape (m <= 64)
@@ -146,7 +156,7 @@ struct Fp8KstatPlan {
 Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
 int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const void* act_q, const float* act_scale,
                      size_t act_scale_count, const void* w_q, const float* w_scale, size_t w_scale_count, size_t m,
-                     size_t n, size_t k, void* workspace, hipStream_t s);
+                     size_t n, size_t k, void* workspace, hipStream_t s, const Epilogue& epi = Epilogue());
 
 struct Fp8Plan {
   int MT;
@@ -159,6 +169,6 @@ Fp8Plan fp8_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
 bool fp8_prefill_supported(size_t m, size_t n, size_t k);
 int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                        const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
-                       hipStream_t s);
+                       hipStream_t s, const Epilogue& epi = Epilogue());
 
 }  // namespace ksq

@@ -1,5 +1,7 @@
 // Load-time repack: checkpoint / canonical int4 layouts -> MFMA fragment order (see include/ksq.h).
 // Pure byte shuffling, bound by HBM bandwidth; one thread builds one 32-bit output word (eight nibbles).
+#include <vector>
+
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -13,7 +15,15 @@ struct RepackArgs {
   uint32_t* dst_sz;
   size_t K, N, g;
   int layout, zero_kind, scale_dtype;
+  const int32_t* row_perm;  // destination row i holds source row row_perm[i]; null = identity
+  int column_order;
 };
+
+// source column of destination column n
+__host__ __device__ inline size_t source_column(const RepackArgs& a, size_t n) {
+  if (a.column_order == KSQ_COLS_HALVES_INTERLEAVED) return (n & 1) * (a.N >> 1) + (n >> 1);
+  return n;
+}
 
 __host__ __device__ inline float bits16_to_float(uint16_t b, int dtype) {
   if (dtype == KSQ_BF16) {
@@ -59,6 +69,30 @@ __host__ __device__ inline uint32_t source_nibble(const RepackArgs& a, size_t k,
       int slot = (i >> 1) + 4 * (i & 1);
       return (w >> (4 * slot)) & 0xFu;
     }
+    case KSQ_W4_CUTLASS_SM80_INTERLEAVED: {
+      // Inverse of the four steps of preprocess_weights_for_mixed_gemm for W4_A16 on sm80
+      // (LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508), read backwards:
+      //  row permutation inside groups of 32 rows (:129-141, :143-197): position r' of a group holds row map[r'];
+      //  transpose to column major, eight consecutive rows per 32-bit register (:203-323);
+      //  four columns interleaved in tiles of 64 rows = 8 registers (:426-464, with the layout
+      //  ColumnMajorTileInterleave<64, 4> of LK/cutlass_extensions/gemm/kernel/mixed_gemm_B_layout.h);
+      //  + 8 and the register relayout [e0 e2 e4 e6 e1 e3 e5 e7] (:352-401).
+      const size_t r32 = k & 31;
+      // inverse of {0,1,8,9,16,17,24,25, 2,3,10,11,18,19,26,27, 4,5,12,13,20,21,28,29, 6,7,14,15,22,23,30,31}:
+      // row r32 = 8a + 2b + c (a, b < 4, c < 2) sits at position 8b + 2a + c
+      const size_t pos = 8 * ((r32 >> 1) & 3) + 2 * (r32 >> 3) + (r32 & 1);
+      const size_t rp = (k - r32) + pos;
+      const size_t v = rp >> 3, e = rp & 7;                    // register along k and element inside it
+      const size_t vw = 4 * (v & ~(size_t)7) + 8 * (n & 3) + (v & 7);
+      const uint32_t w = static_cast<const uint32_t*>(a.qweight)[(n >> 2) * (a.K >> 3) * 4 + vw];
+      const int slot = (e & 1) ? 4 + (int)(e >> 1) : (int)(e >> 1);
+      return (w >> (4 * slot)) & 0xFu;  // already unsigned
+    }
+    case KSQ_W4_CUTLASS_SM90_COLMAJOR: {  // transpose only: int8 [N, K/2], signed
+      uint8_t b = static_cast<const uint8_t*>(a.qweight)[n * (a.K >> 1) + (k >> 1)];
+      uint32_t nib = (k & 1) ? (b >> 4) : (b & 0xFu);
+      return nib ^ 8u;
+    }
     default: {  // KSQ_W4_ROWMAJOR_INT4_SIGNED: two's-complement q, u = q + 8 = nibble ^ 8
       uint8_t b = static_cast<const uint8_t*>(a.qweight)[k * (a.N >> 1) + (n >> 1)];
       uint32_t nib = (n & 1) ? (b >> 4) : (b & 0xFu);
@@ -70,7 +104,16 @@ __host__ __device__ inline uint32_t source_nibble(const RepackArgs& a, size_t k,
 __host__ __device__ inline uint32_t build_weight_word(const RepackArgs& a, size_t word) {
   size_t k0, n;
   frag_word_origin(word, a.K, &k0, &n);
+  n = source_column(a, n);
   uint32_t out = 0;
+  if (a.row_perm) {
+    for (int e = 0; e < 8; ++e) {
+      size_t kr = (size_t)(uint32_t)a.row_perm[k0 + e];
+      if (kr >= a.K) kr = 0;  // a bad entry must not turn into a wild read
+      out |= source_nibble(a, kr, n) << (4 * frag_nibble_of(e));
+    }
+    return out;
+  }
   if (a.layout == KSQ_W4_GPTQ_INT32_KPACK) {
     // the eight elements are the eight nibbles of one source word, in k order
     uint32_t w = static_cast<const uint32_t*>(a.qweight)[(k0 >> 3) * a.N + n];
@@ -86,7 +129,7 @@ __host__ __device__ inline uint32_t build_sz_word(const RepackArgs& a, size_t id
   const size_t G = a.K / a.g;
   size_t c = idx & 15, rest = idx >> 4;
   size_t gi = rest % G, nt = rest / G;
-  size_t n = nt * kTileN + c;
+  size_t n = source_column(a, nt * kTileN + c);
   uint16_t sbits = static_cast<const uint16_t*>(a.scales)[gi * a.N + n];
   uint32_t z = 8;
   switch (a.zero_kind) {
@@ -128,13 +171,15 @@ __global__ __launch_bounds__(256) void repack_sz_kernel(RepackArgs a, size_t cou
 }
 
 int validate(int layout, const void* qweight, int zero_kind, const void* zeros, const void* scales, int scale_dtype,
-             size_t k, size_t n, size_t g, const void* dw, const void* dsz) {
-  KSQ_REQUIRE(layout >= KSQ_W4_GPTQ_INT32_KPACK && layout <= KSQ_W4_ROWMAJOR_INT4_SIGNED, KSQ_ERR_INVALID_ARGUMENT,
+             size_t k, size_t n, size_t g, int column_order, const void* dw, const void* dsz) {
+  KSQ_REQUIRE(layout >= KSQ_W4_GPTQ_INT32_KPACK && layout <= KSQ_W4_CUTLASS_SM90_COLMAJOR, KSQ_ERR_INVALID_ARGUMENT,
               "bad source layout %d", layout);
   KSQ_REQUIRE(zero_kind >= KSQ_ZERO_NONE && zero_kind <= KSQ_ZERO_ADDITIVE, KSQ_ERR_INVALID_ARGUMENT,
               "bad zero kind %d", zero_kind);
   KSQ_REQUIRE(scale_dtype == KSQ_F16 || scale_dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad scale dtype %d",
               scale_dtype);
+  KSQ_REQUIRE(column_order == KSQ_COLS_NATURAL || column_order == KSQ_COLS_HALVES_INTERLEAVED,
+              KSQ_ERR_INVALID_ARGUMENT, "bad column order %d", column_order);
   KSQ_REQUIRE(qweight && scales && dw && dsz, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
   KSQ_REQUIRE(zero_kind == KSQ_ZERO_NONE || zeros, KSQ_ERR_INVALID_ARGUMENT, "zero points requested but null");
   size_t wb, sb;
@@ -144,19 +189,70 @@ int validate(int layout, const void* qweight, int zero_kind, const void* zeros, 
   return KSQ_OK;
 }
 
+RepackArgs make_args(int layout, const void* qweight, int zero_kind, const void* zeros, const void* scales,
+                     int scale_dtype, size_t k, size_t n, size_t g, const int32_t* row_perm, int column_order,
+                     void* dst_weight, void* dst_sz) {
+  RepackArgs a{};
+  a.qweight = qweight;
+  a.zeros = zeros;
+  a.scales = scales;
+  a.dst_weight = static_cast<uint32_t*>(dst_weight);
+  a.dst_sz = static_cast<uint32_t*>(dst_sz);
+  a.K = k;
+  a.N = n;
+  a.g = g;
+  a.layout = layout;
+  a.zero_kind = zero_kind;
+  a.scale_dtype = scale_dtype;
+  a.row_perm = row_perm;
+  a.column_order = column_order;
+  return a;
+}
+
+// out[m, i] = in[m, perm[i]]: one thread per eight destination elements (16 bytes stored)
+__global__ __launch_bounds__(256) void permute_columns_kernel(uint16_t* out, const uint16_t* in, const int32_t* perm,
+                                                              size_t m, size_t k) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // group of eight columns
+  const size_t per_row = k / 8;
+  if (i >= m * per_row) return;
+  const size_t row = i / per_row, c0 = (i - row * per_row) * 8;
+  const uint16_t* src = in + row * k;
+  uint32_t w[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    uint32_t p0 = (uint32_t)perm[c0 + 2 * q], p1 = (uint32_t)perm[c0 + 2 * q + 1];
+    p0 = p0 < k ? p0 : 0;  // a bad entry must not turn into a wild read
+    p1 = p1 < k ? p1 : 0;
+    const uint32_t lo = src[p0], hi = src[p1];
+    w[q] = lo | (hi << 16);
+  }
+  uint4 v{w[0], w[1], w[2], w[3]};
+  *reinterpret_cast<uint4*>(out + row * k + c0) = v;
+}
+
+// out row 2i = in row i, out row 2i + 1 = in row rows/2 + i; one thread per 32-bit word
+__global__ __launch_bounds__(256) void interleave_halves_kernel(uint32_t* out, const uint32_t* in, size_t rows,
+                                                                size_t row_words) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * row_words) return;
+  const size_t r = i / row_words, w = i - r * row_words;
+  const size_t src = (r & 1) * (rows / 2) + (r >> 1);
+  out[i] = in[src * row_words + w];
+}
+
 }  // namespace
 }  // namespace ksq
 
 using namespace ksq;
 
-extern "C" int ksq_w4a16_repack(int layout, const void* qweight, int zero_kind, const void* zeros,
-                                const void* scales, int scale_dtype, size_t k, size_t n, size_t g, void* dst_weight,
-                                void* dst_sz, void* stream) {
-  int rc = validate(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, dst_weight, dst_sz);
+extern "C" int ksq_w4a16_repack_ex(int layout, const void* qweight, int zero_kind, const void* zeros,
+                                   const void* scales, int scale_dtype, size_t k, size_t n, size_t g,
+                                   const int32_t* row_perm, int column_order, void* dst_weight, void* dst_sz,
+                                   void* stream) {
+  int rc = validate(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, column_order, dst_weight, dst_sz);
   if (rc != KSQ_OK) return rc;
-  RepackArgs a{qweight, zeros, scales, static_cast<uint32_t*>(dst_weight), static_cast<uint32_t*>(dst_sz),
-               k,       n,     g,      layout,                             zero_kind,
-               scale_dtype};
+  RepackArgs a = make_args(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, row_perm, column_order,
+                           dst_weight, dst_sz);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t words = k * n / 8, count = (k / g) * n;
   KSQ_REQUIRE((words + 255) / 256 < (1ull << 31), KSQ_ERR_UNSUPPORTED, "tensor too large for one launch");
@@ -166,16 +262,84 @@ extern "C" int ksq_w4a16_repack(int layout, const void* qweight, int zero_kind, 
   return KSQ_OK;
 }
 
-extern "C" int ksq_w4a16_repack_host(int layout, const void* qweight, int zero_kind, const void* zeros,
-                                     const void* scales, int scale_dtype, size_t k, size_t n, size_t g,
-                                     void* dst_weight, void* dst_sz) {
-  int rc = validate(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, dst_weight, dst_sz);
+extern "C" int ksq_w4a16_repack(int layout, const void* qweight, int zero_kind, const void* zeros,
+                                const void* scales, int scale_dtype, size_t k, size_t n, size_t g, void* dst_weight,
+                                void* dst_sz, void* stream) {
+  return ksq_w4a16_repack_ex(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, nullptr,
+                             KSQ_COLS_NATURAL, dst_weight, dst_sz, stream);
+}
+
+extern "C" int ksq_w4a16_repack_ex_host(int layout, const void* qweight, int zero_kind, const void* zeros,
+                                        const void* scales, int scale_dtype, size_t k, size_t n, size_t g,
+                                        const int32_t* row_perm, int column_order, void* dst_weight, void* dst_sz) {
+  int rc = validate(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, column_order, dst_weight, dst_sz);
   if (rc != KSQ_OK) return rc;
-  RepackArgs a{qweight, zeros, scales, static_cast<uint32_t*>(dst_weight), static_cast<uint32_t*>(dst_sz),
-               k,       n,     g,      layout,                             zero_kind,
-               scale_dtype};
+  if (row_perm)
+    for (size_t i = 0; i < k; ++i)
+      KSQ_REQUIRE(row_perm[i] >= 0 && (size_t)row_perm[i] < k, KSQ_ERR_INVALID_ARGUMENT,
+                  "row_perm[%zu] = %d is outside [0, %zu)", i, row_perm[i], k);
+  RepackArgs a = make_args(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, row_perm, column_order,
+                           dst_weight, dst_sz);
   const size_t words = k * n / 8, count = (k / g) * n;
   for (size_t i = 0; i < words; ++i) a.dst_weight[i] = build_weight_word(a, i);
   for (size_t i = 0; i < count; ++i) a.dst_sz[i] = build_sz_word(a, i);
+  return KSQ_OK;
+}
+
+extern "C" int ksq_w4a16_repack_host(int layout, const void* qweight, int zero_kind, const void* zeros,
+                                     const void* scales, int scale_dtype, size_t k, size_t n, size_t g,
+                                     void* dst_weight, void* dst_sz) {
+  return ksq_w4a16_repack_ex_host(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, nullptr,
+                                  KSQ_COLS_NATURAL, dst_weight, dst_sz);
+}
+
+extern "C" int ksq_gptq_act_order_perm(const int32_t* g_idx, size_t k, size_t g, int32_t* perm) {
+  KSQ_REQUIRE(g_idx && perm, KSQ_ERR_INVALID_ARGUMENT, "null pointer");
+  KSQ_REQUIRE(g > 0 && k > 0 && k % g == 0 && k < (1ull << 31), KSQ_ERR_INVALID_ARGUMENT,
+              "k=%zu must be a positive multiple of the group size %zu", k, g);
+  const size_t groups = k / g;
+  // counting sort = stable argsort for keys in [0, groups)
+  std::vector<size_t> fill(groups, 0);
+  for (size_t i = 0; i < k; ++i) {
+    KSQ_REQUIRE(g_idx[i] >= 0 && (size_t)g_idx[i] < groups, KSQ_ERR_INVALID_ARGUMENT,
+                "g_idx[%zu] = %d is outside [0, %zu)", i, g_idx[i], groups);
+    ++fill[(size_t)g_idx[i]];
+  }
+  for (size_t gi = 0; gi < groups; ++gi)
+    KSQ_REQUIRE(fill[gi] == g, KSQ_ERR_UNSUPPORTED,
+                "group %zu has %zu rows, not %zu: a partial group cannot run on kernels for grouped rows", gi,
+                fill[gi], g);
+  for (size_t gi = 0; gi < groups; ++gi) fill[gi] = gi * g;
+  for (size_t i = 0; i < k; ++i) perm[fill[(size_t)g_idx[i]]++] = (int32_t)i;
+  return KSQ_OK;
+}
+
+extern "C" int ksq_permute_columns(void* out, const void* in, const int32_t* perm, size_t m, size_t k,
+                                   void* stream) {
+  KSQ_REQUIRE(out && in && perm, KSQ_ERR_INVALID_ARGUMENT, "null pointer");
+  KSQ_REQUIRE(out != in, KSQ_ERR_INVALID_ARGUMENT, "in-place permutation is not supported");
+  KSQ_REQUIRE(k % 8 == 0, KSQ_ERR_UNSUPPORTED, "k=%zu must be a multiple of 8", k);
+  KSQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0, KSQ_ERR_INVALID_ARGUMENT, "out must be 16-byte aligned");
+  if (m == 0 || k == 0) return KSQ_OK;
+  const size_t items = m * (k / 8);
+  KSQ_REQUIRE((items + 255) / 256 < (1ull << 31), KSQ_ERR_UNSUPPORTED, "tensor too large for one launch");
+  hipLaunchKernelGGL(permute_columns_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<uint16_t*>(out), static_cast<const uint16_t*>(in),
+                     perm, m, k);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+extern "C" int ksq_interleave_halves(void* out, const void* in, size_t rows, size_t row_bytes, void* stream) {
+  KSQ_REQUIRE(out && in && out != in, KSQ_ERR_INVALID_ARGUMENT, "null or aliased pointers");
+  KSQ_REQUIRE(rows % 2 == 0 && row_bytes % 4 == 0, KSQ_ERR_UNSUPPORTED,
+              "rows=%zu must be even and row_bytes=%zu a multiple of 4", rows, row_bytes);
+  if (rows == 0 || row_bytes == 0) return KSQ_OK;
+  const size_t words = rows * (row_bytes / 4);
+  KSQ_REQUIRE((words + 255) / 256 < (1ull << 31), KSQ_ERR_UNSUPPORTED, "tensor too large for one launch");
+  hipLaunchKernelGGL(interleave_halves_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<uint32_t*>(out), static_cast<const uint32_t*>(in),
+                     rows, row_bytes / 4);
+  KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

@@ -16,6 +16,7 @@
 // fp32 sums over 64 k scaled by s[g,n].
 #include <cstdlib>
 
+#include "ksq_epilogue.h"
 #include "ksq_internal.h"
 #include "ksq_w4a16_ops.h"
 
@@ -30,6 +31,7 @@ struct AstreamArgs {
   const void* act;     // [M][K] T
   void* out;           // [M][N] T
   int M, N, K, KT, G, ntiles;
+  Epilogue epi;
 };
 
 template <typename T, int GPT, int MT, int CNT>
@@ -185,14 +187,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ww = 0; ww < kWaves; ++ww) sum += red[(q * kWaves + ww) * 64 + lane];
-    if (i < count) {
-      const int col = (nt_begin + i) * 16 + c;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int row = 16 * mt + 4 * j + e;
-        if (row < p.M) out[(size_t)row * p.N + col] = O::to_bits(sum[e]);
-      }
-    }
+    if (i < count) epi_store_acc<T>(p.epi, out, sum, 16 * mt + 4 * j, (nt_begin + i) * 16 + c, p.M, p.N, true);
   }
 }
 
@@ -220,8 +215,10 @@ bool w4a16_astream_supported(size_t m, size_t n, size_t k) {
 }
 
 int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, int cus, hipStream_t s) {
+                         size_t n, size_t k, size_t g, int cus, hipStream_t s,
+                         const Epilogue& epi) {
   AstreamArgs a{};
+  a.epi = epi;
   a.weight = weight;
   a.sz = sz;
   a.act = act;

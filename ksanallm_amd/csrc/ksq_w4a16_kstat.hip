@@ -14,6 +14,7 @@
 #include <cstdlib>
 
 #include "ksq_internal.h"
+#include "ksq_epilogue.h"
 #include "ksq_w4a16_ops.h"
 
 namespace ksq {
@@ -29,6 +30,7 @@ struct KstatArgs {
   f32x4* partial;      // [ksplit][ntiles][MT][64]
   unsigned* counters;  // [ntiles][MT]
   int M, N, K, KT, G, ntiles, ksplit, nt_per_wg;
+  Epilogue epi;
 };
 
 template <typename T, int GPT, int MT, int TPW, int NB, int NW>
@@ -208,14 +210,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
           if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
-      if (store) {
-        const int col = nt * 16 + c;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int row = 16 * mt + 4 * j + e;
-          if (row < p.M) out[(size_t)row * p.N + col] = O::to_bits(sum[e]);
-        }
-      }
+      if (store) epi_store_acc<T>(p.epi, out, sum, 16 * mt + 4 * j, nt * 16 + c, p.M, p.N, true);
     }
   }
 }
@@ -303,11 +298,13 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
 }
 
 int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
-                       const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
+                       const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                       const Epilogue& epi) {
   KSQ_REQUIRE(m * k * 2 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED, "activation tensor larger than 2 GiB");
   KSQ_REQUIRE(((size_t)plan.nt_per_wg + 8) * (k / kTileK) * 1024 < 0x3FFFFF00ull, KSQ_ERR_UNSUPPORTED,
               "column range of one workgroup larger than 1 GiB");
   KstatArgs a{};
+  a.epi = epi;
   a.weight = weight;
   a.sz = sz;
   a.act = act;

@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "ksq_internal.h"
+#include "ksq_epilogue.h"
 #include "ksq_w4a16_ops.h"
 
 namespace ksq {
@@ -38,6 +39,7 @@ struct PrefillArgs {
   void* out;
   const float* row_scale;  // bf16 route: 2^e per row of the re-encoded activations
   int M, N, K, KT, G, ntiles, mblocks, nblocks, super_n;
+  Epilogue epi;
 };
 
 constexpr int kBM = 128;             // rows per workgroup
@@ -350,11 +352,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
       float rs = 1.f;
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
-      u32x4 packed;
+      float vals[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        packed[q] = (uint32_t)Ops<T>::to_bits(src[2 * q] * rs) | ((uint32_t)Ops<T>::to_bits(src[2 * q + 1] * rs) << 16);
-      if (row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+      for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs;
+      if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -546,11 +547,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
       const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
       float rs = 1.f;
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
-      u32x4 packed;
+      float vals[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        packed[q] = (uint32_t)Ops<T>::to_bits(src[2 * q] * rs) | ((uint32_t)Ops<T>::to_bits(src[2 * q + 1] * rs) << 16);
-      if (cc < 16 * KNT && row < p.M && col + 8 <= p.N) *reinterpret_cast<u32x4*>(out + (size_t)row * p.N + col) = packed;
+      for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs;
+      if (cc < 16 * KNT && row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -597,10 +597,12 @@ size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k) {
 }
 
 int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
+                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                         const Epilogue& epi) {
   KSQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && n % 8 == 0, KSQ_ERR_INVALID_ARGUMENT,
               "prefill output must be 16-byte aligned");
   PrefillArgs a{};
+  a.epi = epi;
   a.weight = weight;
   a.sz = sz;
   a.act = act;

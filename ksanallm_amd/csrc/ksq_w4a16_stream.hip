@@ -20,6 +20,7 @@
 // keeps the pipeline free of branches (the hardware retires loads in order, and the compiler can only leave later
 // prefetches in flight across a wait when the number of loads issued after it is known statically).
 #include "ksq_internal.h"
+#include "ksq_epilogue.h"
 #include "ksq_w4a16_ops.h"
 
 namespace ksq {
@@ -35,6 +36,7 @@ struct StreamArgs {
   f32x4* partial;      // [ksplit][mblocks][ntiles][MT][64]
   unsigned* counters;  // [mblocks * ngroups]
   int M, N, K, KT, G, ntiles, ngroups, ksplit;
+  Epilogue epi;
 };
 
 template <typename T, int MT, int NT, int GPT, int D, int KCT, int KS>
@@ -277,13 +279,8 @@ w4a16_stream_kernel(StreamArgs p) {
   // ---- epilogue: lane (c, j) holds column 16*nt + c, rows m0 + 16*mt + 4*j + i
   uint16_t* out = static_cast<uint16_t*>(p.out);
   auto store_out = [&](int mt, int t, f32x4 v) {
-    if (!tile_ok[t]) return;
-    const int col = (nt0 + t) * 16 + c;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = m0 + 16 * mt + 4 * j + i;
-      if (row < p.M) out[(size_t)row * p.N + col] = O::to_bits(v[i]);
-    }
+    if (!tile_ok[t]) return;  // uniform over the wave
+    epi_store_acc<T>(p.epi, out, v, m0 + 16 * mt + 4 * j, (nt0 + t) * 16 + c, p.M, p.N, true);
   };
 
   if (p.ksplit == 1) {
@@ -377,12 +374,14 @@ int w4a16_stream_max_slices(int mt, int nt) {
 }
 
 int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
-                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s) {
+                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                        const Epilogue& epi) {
   // activations are addressed with 32-bit range-checked offsets
   KSQ_REQUIRE(m * k * 2 < 0x7FFFFF00ull, KSQ_ERR_UNSUPPORTED, "activation tensor larger than 2 GiB (m=%zu k=%zu)",
               m, k);
   KSQ_REQUIRE(plan.NT == 1 || plan.NT == 2 || plan.NT == 4, KSQ_ERR_INVALID_ARGUMENT, "bad plan");
   StreamArgs a{};
+  a.epi = epi;
   a.weight = weight;
   a.sz = sz;
   a.act = act;

@@ -396,6 +396,129 @@ void orc_fp8_convert_weight_per_channel(const void* w_kn, int dtype, size_t K, s
   free(t);
 }
 
+/* ---------------------------------------------------------------- CUTLASS weight preprocessor (F1 input layout)
+ *
+ * preprocess_weights_for_mixed_gemm for QuantType::W4_A16, shape {K, N}
+ * (LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508).  On sm80..sm89 the layout details are
+ * ColumnMajorTileInterleave<64, 4> with the LDSM row permutation
+ * (LK/cutlass_extensions/gemm/kernel/mixed_gemm_B_layout.h:106-120: ThreadblockK = 128*8/16 = 64,
+ * ColumnsInterleaved = (128*8/4)/64 = 4, OpMultiplyAddDequantizeInterleavedBToA), so all four steps run; on sm90
+ * (:130-136: ColumnMajor, OpMultiplyAdd) only the transpose runs and the bias step is skipped (:497-499).
+ * Each step below is a separate pass over a whole buffer, as in the reference, on nibble arrays for clarity:
+ * in[k][n] signed nibble as stored (two's complement), row-major bytes [K][N/2], low nibble = even n.
+ *
+ * Pinned by: every step being a bijection on nibble positions (the tests check that the multiset of values
+ * survives and that distinct inputs give distinct outputs), by the product's repack, which reads this layout
+ * through a closed-form inverse written independently of these loops, reproducing the repack of the
+ * row-major source bit for bit, and by bit-plane probes (a tensor with a single marked nibble lands where the
+ * closed form says).  The reference itself cannot be run here (CUTLASS headers and the CUDA runtime are absent).
+ */
+static inline uint8_t get_nib(const uint8_t* b, size_t i) { return (i & 1) ? (uint8_t)(b[i >> 1] >> 4) : (uint8_t)(b[i >> 1] & 0xF); }
+static inline void set_nib(uint8_t* b, size_t i, uint8_t v) {
+  if (i & 1) b[i >> 1] = (uint8_t)((b[i >> 1] & 0x0F) | (v << 4));
+  else b[i >> 1] = (uint8_t)((b[i >> 1] & 0xF0) | (v & 0xF));
+}
+
+/* :129-141 the map, :143-197 the pass: inside every group of 32 rows, row r of the output is row map[r] of the
+ * input (whole rows move; the reference moves them 32 bits at a time) */
+void orc_cutlass_permute_rows(const uint8_t* in, size_t K, size_t N, uint8_t* out) {
+  static const int map[32] = {0, 1, 8,  9,  16, 17, 24, 25, 2, 3, 10, 11, 18, 19, 26, 27,
+                              4, 5, 12, 13, 20, 21, 28, 29, 6, 7, 14, 15, 22, 23, 30, 31};
+  const size_t row_bytes = N / 2;
+  for (size_t base = 0; base < K; base += 32)
+    for (size_t r = 0; r < 32; ++r) memcpy(out + (base + r) * row_bytes, in + (base + (size_t)map[r]) * row_bytes, row_bytes);
+}
+
+/* :203-323 sub-byte transpose: out is [N][K/2] bytes, nibble k of row n = in nibble n of row k */
+void orc_cutlass_transpose(const uint8_t* in, size_t K, size_t N, uint8_t* out) {
+  for (size_t k = 0; k < K; ++k)
+    for (size_t n = 0; n < N; ++n) set_nib(out, n * K + k, get_nib(in, k * N + n));
+}
+
+/* :426-464 on 32-bit registers of the column-major tensor ([N][K/8] registers): rows_per_tile = 64 ->
+ * 8 registers per tile, interleave = 4 columns */
+void orc_cutlass_interleave_columns(const uint32_t* in, size_t K, size_t N, uint32_t* out) {
+  const size_t vec_rows = K / 8, per_tile = 64 / 8, il = 4;
+  for (size_t col = 0; col < N; ++col) {
+    const size_t wcol = col / il;
+    for (size_t base = 0; base < vec_rows; base += per_tile)
+      for (size_t v = base; v < base + per_tile && v < vec_rows; ++v) {
+        const size_t wv = il * base + per_tile * (col % il) + v % per_tile;
+        out[wcol * vec_rows * il + wv] = in[col * vec_rows + v];
+      }
+  }
+}
+
+/* :352-401 every nibble + 8 (signed -> unsigned), then inside every 32-bit register destination slot d takes
+ * source slot 2d (d < 4) or 2(d - 4) + 1 */
+void orc_cutlass_bias_and_interleave(uint32_t* regs, size_t count) {
+  for (size_t i = 0; i < count; ++i) {
+    const uint32_t r = regs[i];
+    uint32_t biased = 0, t = 0;
+    for (int e = 0; e < 8; ++e) {
+      int v = (int)((r >> (4 * e)) & 0xF);
+      if (v >= 8) v -= 16; /* sign extension of the stored nibble */
+      biased |= (uint32_t)(v + 8) << (4 * e);
+    }
+    for (int d = 0; d < 8; ++d) {
+      const int src = d < 4 ? 2 * d : 2 * (d - 4) + 1;
+      t |= ((biased >> (4 * src)) & 0xFu) << (4 * d);
+    }
+    regs[i] = t;
+  }
+}
+
+/* rowmajor: [K][N/2] bytes; out: K*N/2 bytes.  arch 80: all four steps; arch 90: the transpose only. */
+void orc_cutlass_preprocess(const uint8_t* rowmajor, size_t K, size_t N, int arch, uint8_t* out) {
+  const size_t bytes = K * N / 2;
+  uint8_t* a = (uint8_t*)malloc(bytes);
+  uint8_t* b = (uint8_t*)malloc(bytes);
+  memcpy(a, rowmajor, bytes);
+  if (arch < 90) {
+    orc_cutlass_permute_rows(a, K, N, b);
+    uint8_t* t = a; a = b; b = t;
+  }
+  memset(b, 0, bytes);
+  orc_cutlass_transpose(a, K, N, b);
+  { uint8_t* t = a; a = b; b = t; }
+  if (arch < 90) {
+    orc_cutlass_interleave_columns((const uint32_t*)a, K, N, (uint32_t*)b);
+    uint8_t* t = a; a = b; b = t;
+    orc_cutlass_bias_and_interleave((uint32_t*)a, bytes / 4);
+  }
+  memcpy(out, a, bytes);
+  free(a);
+  free(b);
+}
+
+/* ---------------------------------------------------------------- desc_act (F3)
+ * perm = stable argsort of g_idx (MarlinSortGIdx, KS/models/quant/quant_weight.cpp:455-460: torch::argsort with
+ * stable = true); the activations' columns are gathered through it (permute_cols_kernel,
+ * LK/gptq_marlin/gptq_marlin.cu:380-384) and the weight rows stored in the same order.  Insertion sort: stable
+ * by construction, written independently of the product's counting sort. */
+void orc_act_order_perm(const int32_t* g_idx, size_t K, int32_t* perm) {
+  for (size_t i = 0; i < K; ++i) {
+    size_t j = i;
+    while (j > 0 && g_idx[perm[j - 1]] > g_idx[i]) {
+      perm[j] = perm[j - 1];
+      --j;
+    }
+    perm[j] = (int32_t)i;
+  }
+}
+
+/* ---------------------------------------------------------------- epilogues (F2), on the fp32 GEMM result
+ * SiLU-mul: KS/models/common/common_model.cpp:540-547 runs gate and up GEMMs and then silu(gate) * up
+ * (LK/activation: silu(x) = x / (1 + exp(-x))); here gate = acc[:, :H], up = acc[:, H:] of one [M, 2H] result.
+ * Bias: out + bias[n] (common_model.cpp:456-459). */
+void orc_silu_mul(const float* acc, size_t M, size_t H, float* out) {
+  for (size_t m = 0; m < M; ++m)
+    for (size_t h = 0; h < H; ++h) {
+      const double g = acc[m * 2 * H + h], u = acc[m * 2 * H + H + h];
+      out[m * H + h] = (float)(g / (1.0 + exp(-g)) * u);
+    }
+}
+
 int orc_num_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

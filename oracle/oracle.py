@@ -269,6 +269,46 @@ def fp8_merge_qkv_max(wq, q_scale, k_scale, v_scale, nq, nk, nv):
     return out, merged
 
 
+# ---------------------------------------------------------------- layouts the loader's back ends leave behind
+def cutlass_preprocess(rowmajor, arch=80):
+    """Output bytes of preprocess_weights_for_mixed_gemm (W4_A16) for a row-major signed int4 tensor [K, N/2]."""
+    rowmajor = _c(rowmajor, np.uint8)
+    K, N = rowmajor.shape[0], rowmajor.shape[1] * 2
+    out = np.empty(K * N // 2, dtype=np.uint8)
+    lib().orc_cutlass_preprocess(_p(rowmajor), _sz(K), _sz(N), int(arch), _p(out))
+    return out
+
+
+def cutlass_step(step, data, K, N):
+    """One step of the preprocessor on a whole buffer of K*N/2 bytes: 'permute_rows', 'transpose',
+    'interleave_columns' or 'bias_and_interleave'."""
+    data = _c(data, np.uint8).reshape(-1)
+    assert data.size == K * N // 2
+    if step == "bias_and_interleave":
+        out = data.copy()
+        lib().orc_cutlass_bias_and_interleave(_p(out), _sz(out.size // 4))
+        return out
+    out = np.zeros_like(data)
+    getattr(lib(), "orc_cutlass_" + step)(_p(data), _sz(K), _sz(N), _p(out))
+    return out
+
+
+def act_order_perm(g_idx):
+    g_idx = _c(g_idx, np.int32)
+    perm = np.empty(g_idx.shape[0], dtype=np.int32)
+    lib().orc_act_order_perm(_p(g_idx), _sz(g_idx.shape[0]), _p(perm))
+    return perm
+
+
+def silu_mul(acc):
+    """acc [M, 2H] fp32 = [gate | up] -> silu(gate) * up, [M, H] fp32."""
+    acc = _c(acc, np.float32)
+    M, H = acc.shape[0], acc.shape[1] // 2
+    out = np.empty((M, H), dtype=np.float32)
+    lib().orc_silu_mul(_p(acc), _sz(M), _sz(H), _p(out))
+    return out
+
+
 def num_threads():
     return int(lib().orc_num_threads())
 
