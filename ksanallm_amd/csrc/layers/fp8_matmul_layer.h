@@ -20,12 +20,18 @@ class Fp8MatMulLayer : public BaseLayer {
 
   size_t GetWorkSpaceSize(const int m, const int k);
 
+  // Not in the reference: fold a bias row (KSQ_EPILOGUE_BIAS, bias = T [n]) or SiLU(gate) * up of a row-interleaved
+  // gate/up weight (KSQ_EPILOGUE_SILU_MUL; output [m, n/2]) into the GEMM.  The bias tensor must outlive the layer.
+  void SetEpilogue(int kind, const Tensor* bias = nullptr);
+
   size_t GetWorkSpaceSize() override;
 
  private:
   int max_m_ = 0;
   int max_k_ = 0;
   size_t max_n_hint_ = 0;
+  int epilogue_ = 0;
+  const Tensor* bias_ = nullptr;
 };
 
 // Load-time half (replaces the device work of QuantWeight::ConvertFp8E4m3Tensor and BindFp8E4m3ScaleOfQkvWeight,

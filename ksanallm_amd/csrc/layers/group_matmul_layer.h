@@ -21,8 +21,16 @@ class GroupMatMulLayer : public BaseLayer {
   Status Preprocess(const ModelConfig& model_config_) override;
 
   // input_tensors[0]: activations [m, k] T.  input_tensors[1]: weight in fragment order (ksq_w4a16_repack) whose
-  // .scales points at the repacked scale/zero words.  output_tensors[0]: [m, n] T; shape and dtype are set here.
+  // .scales points at the repacked scale/zero words; for a desc_act layer its .perm is the int32 [k] row order the
+  // weight was repacked with (the activations' columns are gathered through it, as the reference's Marlin back end
+  // does: LK/gptq_marlin/gptq_marlin.cu:380-392).  output_tensors[0]: [m, n] T (n/2 columns with the SiLU-mul
+  // epilogue); shape and dtype are set here.
   Status Forward(const std::vector<Tensor>& input_tensors, std::vector<Tensor>& output_tensors) override;
+
+  // Not in the reference, which runs these as layers of their own (KS/models/common/common_model.cpp:456-459,
+  // 540-547): fold a bias row (kind = KSQ_EPILOGUE_BIAS, bias = T [n]) or SiLU(gate) * up of a fused, column
+  // interleaved gate/up weight (KSQ_EPILOGUE_SILU_MUL) into the GEMM.  The bias tensor must outlive the layer.
+  void SetEpilogue(int kind, const Tensor* bias = nullptr);
 
  private:
   bool is_awq_ = false;
@@ -32,15 +40,33 @@ class GroupMatMulLayer : public BaseLayer {
   size_t max_m_ = 0, max_n_ = 0, max_k_ = 0;
   size_t groupsize_ = 128;
   bool cutlass_use_gemv_cuda_core_ = true;
+  int epilogue_ = 0;
+  const Tensor* bias_ = nullptr;
 };
 
 // Load-time half (replaces the CPU layout preprocess + scale / zero binding of QuantWeight::ConvertGroupTensor,
 // KS/models/quant/quant_weight.cpp:530-536, 577-579, 632-636): repacks one checkpoint weight that is already on
 // the device into fragment order and binds `weight.scales`.  `qzeros` may be null (GPTQ).  The tensors that
 // `weight` and `weight_sz` end up owning are allocated here.
-enum GroupWeightLayout { GROUP_WEIGHT_GPTQ_INT32, GROUP_WEIGHT_AWQ_INT32, GROUP_WEIGHT_ROWMAJOR_INT4 };
+// GROUP_WEIGHT_CUTLASS_SM80 / _SM90: what the reference's own loader leaves in "*.weight" after
+// CutlassPreprocessWeightsForMixedGemmWarpper (quant_weight.cpp:331-346) on those architectures, so an untouched
+// loader can be followed by this call.  `perm` (int32 [k] on the device, from SortGptqGIdx) repacks a desc_act
+// checkpoint with its rows grouped and is bound to weight.perm; `interleave_gate_up` repacks a fused [gate | up]
+// weight with its column pairs interleaved for the SiLU-mul epilogue.
+enum GroupWeightLayout {
+  GROUP_WEIGHT_GPTQ_INT32,
+  GROUP_WEIGHT_AWQ_INT32,
+  GROUP_WEIGHT_ROWMAJOR_INT4,
+  GROUP_WEIGHT_CUTLASS_SM80,
+  GROUP_WEIGHT_CUTLASS_SM90
+};
 Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, const Tensor* qzeros, bool zeros_additive,
                               const Tensor& scales, size_t k, size_t n, size_t groupsize, Tensor& weight,
-                              Tensor& weight_sz, int rank, Stream& stream);
+                              Tensor& weight_sz, int rank, Stream& stream, Tensor* perm = nullptr,
+                              bool interleave_gate_up = false);
+
+// perm = stable argsort of a desc_act checkpoint's g_idx (MarlinSortGIdx, quant_weight.cpp:455-460), on the host.
+// Throws unless every group has exactly `groupsize` rows.
+Status SortGptqGIdx(const std::vector<int32_t>& g_idx, size_t groupsize, std::vector<int32_t>& perm);
 
 }  // namespace ksana_llm

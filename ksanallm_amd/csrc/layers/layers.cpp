@@ -81,7 +81,8 @@ template <typename T, DataType WT>
 size_t GroupMatMulLayer<T, WT>::GetWorkSpaceSize() {
   if constexpr (WT == TYPE_I4_GROUP) {
     size_t bytes = 0;
-    ThrowOnKsqError(ksq_w4a16_workspace_bytes(max_m_, max_n_, max_k_, &bytes), "ksq_w4a16_workspace_bytes");
+    ThrowOnKsqError(ksq_w4a16_workspace_bytes_ex(max_m_, max_n_, max_k_, is_gptq_desc_ ? 1 : 0, &bytes),
+                    "ksq_w4a16_workspace_bytes_ex");
     return bytes;
   } else {
     KLLM_THROW("Not supported weight data type. GroupMatMul only supports TYPE_I4_GROUP.");
@@ -101,13 +102,17 @@ template <typename T, DataType WT>
 Status GroupMatMulLayer<T, WT>::Forward(const std::vector<Tensor>& input_tensors,
                                         std::vector<Tensor>& output_tensors) {
   if constexpr (WT == TYPE_I4_GROUP) {
-    if (is_gptq_desc_) {
-      // the reference serves desc_act through its Marlin backend only (KS/utils/environment.cpp:105-106)
-      KLLM_THROW("GroupMatMulLayer: desc_act (g_idx / perm) weights are not supported by this backend.");
-    }
     const Tensor& weight_tensor = input_tensors[1];
     if (weight_tensor.scales == nullptr) {
       KLLM_THROW("GroupMatMulLayer: weight tensor has no scales bound.");
+    }
+    const int32_t* act_perm = nullptr;
+    if (is_gptq_desc_) {
+      // the reference serves desc_act through its Marlin back end only (KS/utils/environment.cpp:105-106); here the
+      // rows were grouped at load time and the activations follow them
+      if (!is_k_full_) KLLM_THROW("GroupMatMulLayer: desc_act with a partial K (is_k_full = false) is not supported.");
+      if (weight_tensor.perm == nullptr) KLLM_THROW("GroupMatMulLayer: desc_act weight tensor has no perm bound.");
+      act_perm = weight_tensor.perm->GetPtr<int32_t>();
     }
     void* p_qweight_tensor = weight_tensor.GetPtr<void>();
     void* p_sz_tensor = weight_tensor.scales->GetPtr<void>();
@@ -118,12 +123,14 @@ Status GroupMatMulLayer<T, WT>::Forward(const std::vector<Tensor>& input_tensors
 
     void* ws = workspace_buffer_ ? workspace_buffer_->GetPtr<void>() : nullptr;
     const size_t ws_bytes = workspace_buffer_ ? workspace_buffer_->GetTotalBytes() : 0;
-    ThrowOnKsqError(ksq_w4a16_gemm(KsqDtype<T>(), output_tensors[0].GetPtr<void>(), input_tensors[0].GetPtr<void>(),
-                                   p_qweight_tensor, p_sz_tensor, m, n, k, groupsize_, ws, ws_bytes,
-                                   context_->GetComputeStreams()[rank_].Get()),
-                    "ksq_w4a16_gemm");
+    ThrowOnKsqError(
+        ksq_w4a16_gemm_ex(KsqDtype<T>(), output_tensors[0].GetPtr<void>(), input_tensors[0].GetPtr<void>(),
+                          p_qweight_tensor, p_sz_tensor, m, n, k, groupsize_, act_perm, epilogue_,
+                          bias_ ? bias_->GetPtr<void>() : nullptr, ws, ws_bytes,
+                          context_->GetComputeStreams()[rank_].Get()),
+        "ksq_w4a16_gemm_ex");
 
-    output_tensors[0].shape = {m, n};
+    output_tensors[0].shape = {m, epilogue_ == KSQ_EPILOGUE_SILU_MUL ? n / 2 : n};
     output_tensors[0].dtype = input_tensors[0].dtype;
     return Status();
   } else {
@@ -131,20 +138,33 @@ Status GroupMatMulLayer<T, WT>::Forward(const std::vector<Tensor>& input_tensors
   }
 }
 
+template <typename T, DataType WT>
+void GroupMatMulLayer<T, WT>::SetEpilogue(int kind, const Tensor* bias) {
+  if (kind < KSQ_EPILOGUE_NONE || kind > KSQ_EPILOGUE_SILU_MUL) KLLM_THROW("GroupMatMulLayer: unknown epilogue.");
+  if (kind == KSQ_EPILOGUE_BIAS && bias == nullptr) KLLM_THROW("GroupMatMulLayer: the bias epilogue needs a bias.");
+  epilogue_ = kind;
+  bias_ = kind == KSQ_EPILOGUE_BIAS ? bias : nullptr;
+}
+
 template class GroupMatMulLayer<float16, TYPE_I4_GROUP>;
 template class GroupMatMulLayer<bfloat16, TYPE_I4_GROUP>;
 
 Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, const Tensor* qzeros,
                               bool zeros_additive, const Tensor& scales, size_t k, size_t n, size_t groupsize,
-                              Tensor& weight, Tensor& weight_sz, int rank, Stream& stream) {
+                              Tensor& weight, Tensor& weight_sz, int rank, Stream& stream, Tensor* perm,
+                              bool interleave_gate_up) {
   size_t weight_bytes = 0, sz_bytes = 0;
   ThrowOnKsqError(ksq_w4a16_repack_sizes(k, n, groupsize, &weight_bytes, &sz_bytes), "ksq_w4a16_repack_sizes");
   if (scales.dtype != TYPE_FP16 && scales.dtype != TYPE_BF16) KLLM_THROW("RepackGroupQuantWeight: scales must be fp16 or bf16.");
   CreateTensor(weight, {k, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);  // same shape as ksana's "*.weight"
   CreateTensor(weight_sz, {k / groupsize, n}, TYPE_UINT32, rank, MEMORY_DEVICE);
-  int src = layout == GROUP_WEIGHT_GPTQ_INT32 ? KSQ_W4_GPTQ_INT32_KPACK
-            : layout == GROUP_WEIGHT_AWQ_INT32 ? KSQ_W4_AWQ_INT32_NPACK
-                                               : KSQ_W4_ROWMAJOR_INT4_SIGNED;
+  int src = layout == GROUP_WEIGHT_GPTQ_INT32     ? KSQ_W4_GPTQ_INT32_KPACK
+            : layout == GROUP_WEIGHT_AWQ_INT32    ? KSQ_W4_AWQ_INT32_NPACK
+            : layout == GROUP_WEIGHT_CUTLASS_SM80 ? KSQ_W4_CUTLASS_SM80_INTERLEAVED
+            : layout == GROUP_WEIGHT_CUTLASS_SM90 ? KSQ_W4_CUTLASS_SM90_COLMAJOR
+                                                  : KSQ_W4_ROWMAJOR_INT4_SIGNED;
+  if (perm != nullptr && (perm->dtype != TYPE_INT32 || perm->GetElementNumber() != k))
+    KLLM_THROW("RepackGroupQuantWeight: perm must be int32 [k].");
   int zero_kind = KSQ_ZERO_NONE;
   if (qzeros != nullptr) {
     if (zeros_additive) zero_kind = KSQ_ZERO_ADDITIVE;
@@ -152,12 +172,22 @@ Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, c
     else zero_kind = KSQ_ZERO_UINT8;
   }
   ThrowOnKsqError(
-      ksq_w4a16_repack(src, qweight.GetPtr<void>(), zero_kind, qzeros ? qzeros->GetPtr<void>() : nullptr,
-                       scales.GetPtr<void>(), scales.dtype == TYPE_FP16 ? KSQ_F16 : KSQ_BF16, k, n, groupsize,
-                       weight.GetPtr<void>(), weight_sz.GetPtr<void>(), stream.Get()),
-      "ksq_w4a16_repack");
+      ksq_w4a16_repack_ex(src, qweight.GetPtr<void>(), zero_kind, qzeros ? qzeros->GetPtr<void>() : nullptr,
+                          scales.GetPtr<void>(), scales.dtype == TYPE_FP16 ? KSQ_F16 : KSQ_BF16, k, n, groupsize,
+                          perm ? perm->GetPtr<int32_t>() : nullptr,
+                          interleave_gate_up ? KSQ_COLS_HALVES_INTERLEAVED : KSQ_COLS_NATURAL, weight.GetPtr<void>(),
+                          weight_sz.GetPtr<void>(), stream.Get()),
+      "ksq_w4a16_repack_ex");
   weight.dtype = TYPE_I4_GROUP;
   weight.scales = &weight_sz;
+  weight.perm = perm;
+  return Status();
+}
+
+Status SortGptqGIdx(const std::vector<int32_t>& g_idx, size_t groupsize, std::vector<int32_t>& perm) {
+  perm.assign(g_idx.size(), 0);
+  ThrowOnKsqError(ksq_gptq_act_order_perm(g_idx.data(), g_idx.size(), groupsize, perm.data()),
+                  "ksq_gptq_act_order_perm");
   return Status();
 }
 
@@ -209,7 +239,8 @@ Status Fp8MatMulLayer<T>::Forward(const std::vector<Tensor>& input_tensors, std:
   }
   const size_t weight_scale_count = input_tensors[1].weight_scales->GetElementNumber() == (size_t)n && n > 1 ? n : 1;
   void* output = output_tensors[0].GetPtr<void>();
-  output_tensors[0].shape = {static_cast<size_t>(m), static_cast<size_t>(n)};
+  output_tensors[0].shape = {static_cast<size_t>(m),
+                             static_cast<size_t>(epilogue_ == KSQ_EPILOGUE_SILU_MUL ? n / 2 : n)};
   output_tensors[0].dtype = input_tensors[0].dtype;
   void* stream = context_->GetComputeStreams()[rank_].Get();
   float* input_scale = nullptr;
@@ -227,10 +258,19 @@ Status Fp8MatMulLayer<T>::Forward(const std::vector<Tensor>& input_tensors, std:
                                      per_token ? KSQ_FP8_PER_TOKEN_DYNAMIC : KSQ_FP8_PER_TENSOR_DYNAMIC, input_quant,
                                      input_scale, stream), "ksq_fp8_quantize");
   }
-  ThrowOnKsqError(ksq_fp8_gemm(KsqDtype<T>(), output, input_quant, input_scale, input_scale_count, weight_quant,
-                               weight_scale, weight_scale_count, m, n, k, gemm_workspace, kFp8GemmWorkspaceBytes,
-                               stream), "ksq_fp8_gemm");
+  ThrowOnKsqError(ksq_fp8_gemm_ex(KsqDtype<T>(), output, input_quant, input_scale, input_scale_count, weight_quant,
+                                  weight_scale, weight_scale_count, m, n, k, epilogue_,
+                                  bias_ ? bias_->GetPtr<void>() : nullptr, gemm_workspace, kFp8GemmWorkspaceBytes,
+                                  stream), "ksq_fp8_gemm_ex");
   return Status();
+}
+
+template <typename T>
+void Fp8MatMulLayer<T>::SetEpilogue(int kind, const Tensor* bias) {
+  if (kind < KSQ_EPILOGUE_NONE || kind > KSQ_EPILOGUE_SILU_MUL) KLLM_THROW("Fp8MatMulLayer: unknown epilogue.");
+  if (kind == KSQ_EPILOGUE_BIAS && bias == nullptr) KLLM_THROW("Fp8MatMulLayer: the bias epilogue needs a bias.");
+  epilogue_ = kind;
+  bias_ = kind == KSQ_EPILOGUE_BIAS ? bias : nullptr;
 }
 
 Status ConvertFp8Weight(const Tensor& weight, bool per_channel, Tensor& weight_fp8, Tensor& weight_scale, int rank,

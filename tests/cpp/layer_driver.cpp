@@ -20,6 +20,7 @@
 #include <string>
 #include <vector>
 
+#include "ksq.h"
 #include "matmul_layer_factory.h"
 
 using namespace ksana_llm;
@@ -60,6 +61,7 @@ static int RunW4(int argc, char** argv) {
   const std::string dir = argv[2];
   const size_t m = atol(argv[4]), k = atol(argv[5]), n = atol(argv[6]), g = atol(argv[7]);
   const std::string method = argv[8], layout = argv[9], zeros = argv[10];
+  const std::string extra = argc > 11 ? argv[11] : "none";  // none | desc | silu | bias
   const DataType dt = TypeTraits<T>::kDataType;
   auto context = std::make_shared<Context>(1);
 
@@ -73,7 +75,8 @@ static int RunW4(int argc, char** argv) {
     lay = GROUP_WEIGHT_AWQ_INT32;
     qweight = Upload(ReadFile(dir + "/qweight.bin"), TYPE_INT32, {k, n / 8});
   } else {
-    lay = GROUP_WEIGHT_ROWMAJOR_INT4;
+    lay = layout == "cutlass80" ? GROUP_WEIGHT_CUTLASS_SM80 : layout == "cutlass90" ? GROUP_WEIGHT_CUTLASS_SM90
+                                                                                  : GROUP_WEIGHT_ROWMAJOR_INT4;
     qweight = Upload(ReadFile(dir + "/qweight.bin"), TYPE_INT8, {k, n / 2});
   }
   const Tensor* zp = nullptr;
@@ -89,13 +92,25 @@ static int RunW4(int argc, char** argv) {
     zp = &qzeros;
     additive = true;
   }
+  Tensor perm;
+  if (extra == "desc") {
+    // what a loader does with a desc_act checkpoint: sort g_idx on the host, keep the permutation on the device
+    std::vector<char> raw = ReadFile(dir + "/g_idx.bin");
+    std::vector<int32_t> g_idx(raw.size() / 4), order;
+    memcpy(g_idx.data(), raw.data(), raw.size());
+    SortGptqGIdx(g_idx, g, order);
+    std::vector<char> bytes(order.size() * 4);
+    memcpy(bytes.data(), order.data(), bytes.size());
+    perm = Upload(bytes, TYPE_INT32, {k});
+  }
   RepackGroupQuantWeight(lay, qweight, zp, additive, scales, k, n, g, weight, weight_sz, 0,
-                         context->GetComputeStreams()[0]);
+                         context->GetComputeStreams()[0], extra == "desc" ? &perm : nullptr, extra == "silu");
 
   ModelConfig cfg;
   cfg.is_quant = true;
   cfg.quant_config.method = method == "awq" ? QUANT_AWQ : QUANT_GPTQ;
   cfg.quant_config.group_size = g;
+  cfg.quant_config.desc_act = extra == "desc";
   cfg.hidden_units = k;
   cfg.size_per_head = n;  // query_key_value: k = hidden_units, n = size_per_head * (head_num + 2 * kv heads)
   cfg.head_num = 1;
@@ -106,6 +121,18 @@ static int RunW4(int argc, char** argv) {
   auto holder = std::make_shared<OneWeight>();
   holder->t = weight;
   auto layer = factory.AutoCreateLayer(holder, "model.layers.0.self_attn.query_key_value.weight", TYPE_I4_GROUP, dt, dt, {});
+
+  Tensor bias;
+  if (extra == "silu" || extra == "bias") {
+    auto group = std::dynamic_pointer_cast<GroupMatMulLayer<T, TYPE_I4_GROUP>>(layer);
+    if (!group) throw std::runtime_error("factory did not build a GroupMatMulLayer");
+    if (extra == "bias") {
+      bias = Upload(ReadFile(dir + "/bias.bin"), dt, {n});
+      group->SetEpilogue(KSQ_EPILOGUE_BIAS, &bias);
+    } else {
+      group->SetEpilogue(KSQ_EPILOGUE_SILU_MUL);
+    }
+  }
 
   Tensor act = Upload(ReadFile(dir + "/act.bin"), dt, {m, k});
   Tensor out;
@@ -251,7 +278,7 @@ static int RunErrors() {
     p[6] = size_t(192);
     factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
   });
-  Expect("desc_act weights are refused at Forward", true, [&] {
+  Expect("desc_act weight without a bound perm throws at Forward", true, [&] {
     std::vector<std::any> p = good;
     p[1] = true;
     auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
@@ -310,7 +337,7 @@ static int RunErrors() {
 int main(int argc, char** argv) {
   try {
     if (argc >= 2 && std::string(argv[1]) == "errors") return RunErrors();
-    if (argc == 11 && std::string(argv[1]) == "w4a16")
+    if ((argc == 11 || argc == 12) && std::string(argv[1]) == "w4a16")
       return std::string(argv[3]) == "f16" ? RunW4<float16>(argc, argv) : RunW4<bfloat16>(argc, argv);
     if (argc == 9 && std::string(argv[1]) == "fp8")
       return std::string(argv[3]) == "f16" ? RunFp8<float16>(argc, argv) : RunFp8<bfloat16>(argc, argv);

@@ -51,6 +51,57 @@ def test_group_matmul_layer_forward(gpu, tmp_path, dtype, method, layout, zeros,
     orc.assert_parity(got, case.oracle(), f"GroupMatMulLayer {method}/{layout}/{zeros} {dtype}")
 
 
+@pytest.mark.parametrize("dtype,extra,layout,M", [
+    ("f16", "none", "cutlass80", 16),    # the reference loader's own output, accepted as it is
+    ("bf16", "none", "cutlass90", 70),
+    ("f16", "desc", "gptq", 24),         # desc_act checkpoint: perm from g_idx, activations gathered at run time
+    ("bf16", "desc", "gptq", 130),
+    ("f16", "silu", "awq", 16),          # fused gate/up with the SiLU-mul epilogue
+    ("bf16", "silu", "awq", 200),
+    ("f16", "bias", "awq", 40),
+])
+def test_group_matmul_layer_widened(gpu, tmp_path, dtype, extra, layout, M):
+    """The same layer fed by an untouched CUTLASS-backend loader, serving a desc_act checkpoint, and with the step
+    after the GEMM folded in."""
+    K, N, g = 1024, 384, 128
+    method = "gptq" if layout == "gptq" else "awq"
+    case = W4Case(600 + M, M, K, N, g=g, kind=method, dtype=dtype)
+    d = str(tmp_path)
+    zeros = "none"
+    if layout.startswith("cutlass"):
+        orc.cutlass_preprocess(case.rowmajor(), int(layout[-2:])).tofile(d + "/qweight.bin")
+        orc.awq_additive_zeros(case.scales, ORC_DT[dtype], case.z).tofile(d + "/qzeros.bin")
+        zeros = "additive"
+    elif layout == "gptq":
+        case.gptq_qweight().tofile(d + "/qweight.bin")
+    else:
+        case.awq_qweight().tofile(d + "/qweight.bin")
+        case.awq_qzeros().tofile(d + "/qzeros.bin")
+        zeros = "awq"
+    case.scales.tofile(d + "/scales.bin")
+    case.act.tofile(d + "/act.bin")
+    want, cols = case.oracle(), N
+    if extra == "desc":
+        rng = np.random.default_rng(601)
+        order = rng.permutation(K)
+        g_idx = np.empty(K, dtype=np.int32)
+        g_idx[order] = np.arange(K, dtype=np.int32) // g
+        g_idx.tofile(d + "/g_idx.bin")
+        s = orc.from_bits(case.scales, ORC_DT[dtype])
+        wdq = (s[g_idx] * (case.u.astype(np.float32) - 8.0)).astype(np.float32)
+        want = orc.gemm_f32(orc.from_bits(case.act, ORC_DT[dtype]), wdq)
+    elif extra == "silu":
+        want, cols = orc.silu_mul(want), N // 2
+    elif extra == "bias":
+        bias = orc.to_bits(np.random.default_rng(602).standard_normal(N).astype(np.float32), ORC_DT[dtype])
+        bias.tofile(d + "/bias.bin")
+        want = want + orc.from_bits(bias, ORC_DT[dtype])[None, :]
+    rc, out = _run(["w4a16", d, dtype, M, K, N, g, method, layout, zeros, extra])
+    assert rc == 0 and out.splitlines()[-1] == f"OK {M} {cols} {DTYPE_ENUM[dtype]}", out
+    got = orc.from_bits(np.fromfile(d + "/out.bin", dtype=np.uint16).reshape(M, cols), ORC_DT[dtype])
+    orc.assert_parity(got, want, f"GroupMatMulLayer {layout} {extra} {dtype}")
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("wscales,static,M", [("1", 0, 7), ("1", 1, 7), ("n", 0, 40)])
 def test_fp8_matmul_layer_forward(gpu, tmp_path, dtype, wscales, static, M):
