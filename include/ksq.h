@@ -55,7 +55,16 @@ typedef enum ksq_w4_layout {
   KSQ_W4_CUTLASS_SM80_INTERLEAVED = 3,
   /* The same preprocessor's output on sm90 (only the transpose runs: :487-490; the bias step is skipped,
    * :497-499): int8 [N, K/2], low nibble = even k, signed q = u - 8. */
-  KSQ_W4_CUTLASS_SM90_COLMAJOR = 4
+  KSQ_W4_CUTLASS_SM90_COLMAJOR = 4,
+  /* What the loader's Marlin back end leaves behind (gptq_marlin_repack / awq_marlin_repack,
+   * LK/gptq_marlin/gptq_marlin_repack.cu:31-233, awq_marlin_repack.cu:30-170; both write the same format):
+   * int32 [K/16, N*16/8], tiles of 16 k x 64 n = 128 words; word th*4 + w of a tile (th 0..31, w 0..3) holds, in
+   * nibble slots [0,2,4,6,1,3,5,7] -> values 0..7, the elements k = 2*(th%4) + {0,1,8,9}, n = 16*w + th/4 (values
+   * 0..3) and n + 8 (values 4..7), unsigned.  With this layout the scales are read in the Marlin order too
+   * (MarlinPermuteScales, KS/models/quant/quant_weight.cpp:350-375) and AWQ zero points must be given as
+   * KSQ_ZERO_MARLIN_INT32.  Needs N % 64 == 0.  A desc_act Marlin weight already has its rows in sorted order:
+   * pass row_perm = NULL to the repack and the loader's perm as act_perm to the GEMM. */
+  KSQ_W4_MARLIN = 5
 } ksq_w4_layout;
 
 /* Order of the columns in the repacked weight (and in its scale / zero words). */
@@ -83,8 +92,11 @@ typedef enum ksq_zero_kind {
   KSQ_ZERO_NONE = 0,          /* symmetric: z = 8 for every group (GPTQ) */
   KSQ_ZERO_AWQ_INT32 = 1,     /* AWQ qzeros int32 [K/g, N/8], as in the checkpoint */
   KSQ_ZERO_UINT8 = 2,         /* unpacked z in [0,15], uint8 [K/g, N] */
-  KSQ_ZERO_ADDITIVE = 3       /* ksana's layer-boundary form: T [K/g, N] holding scales * (8 - z)
+  KSQ_ZERO_ADDITIVE = 3,      /* ksana's layer-boundary form: T [K/g, N] holding scales * (8 - z)
                                  (KS/models/quant/quant_weight.cpp:530-536); z is recovered exactly */
+  KSQ_ZERO_MARLIN_INT32 = 4   /* Marlin zero points int32 [K/g, N/8] (MarlinZeroPoints, quant_weight.cpp:397-426):
+                                 the scale permutation on blocks of 64, [0,2,4,6,1,3,5,7] on blocks of 8, packed
+                                 eight columns per word in order */
 } ksq_zero_kind;
 
 typedef enum ksq_fp8_merge_mode {

@@ -13,10 +13,10 @@ LIB_PATH = os.path.join(_HERE, "libksq.so")
 # enums of include/ksq.h
 F16, BF16 = 0, 1
 W4_GPTQ_INT32_KPACK, W4_AWQ_INT32_NPACK, W4_ROWMAJOR_INT4_SIGNED = 0, 1, 2
-W4_CUTLASS_SM80_INTERLEAVED, W4_CUTLASS_SM90_COLMAJOR = 3, 4
+W4_CUTLASS_SM80_INTERLEAVED, W4_CUTLASS_SM90_COLMAJOR, W4_MARLIN = 3, 4, 5
 COLS_NATURAL, COLS_HALVES_INTERLEAVED = 0, 1
 EPILOGUE_NONE, EPILOGUE_BIAS, EPILOGUE_SILU_MUL = 0, 1, 2
-ZERO_NONE, ZERO_AWQ_INT32, ZERO_UINT8, ZERO_ADDITIVE = 0, 1, 2, 3
+ZERO_NONE, ZERO_AWQ_INT32, ZERO_UINT8, ZERO_ADDITIVE, ZERO_MARLIN_INT32 = 0, 1, 2, 3, 4
 FP8_PER_TENSOR_DYNAMIC, FP8_PER_TENSOR_STATIC, FP8_PER_TOKEN_DYNAMIC = 0, 1, 2
 FP8_MERGE_MAX, FP8_MERGE_PER_CHANNEL = 0, 1
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_HIP = 0, -1, -2, -3, -4

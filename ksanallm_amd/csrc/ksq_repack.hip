@@ -88,6 +88,17 @@ __host__ __device__ inline uint32_t source_nibble(const RepackArgs& a, size_t k,
       const int slot = (e & 1) ? 4 + (int)(e >> 1) : (int)(e >> 1);
       return (w >> (4 * slot)) & 0xFu;  // already unsigned
     }
+    case KSQ_W4_MARLIN: {
+      // inverse of repack_tile (LK/gptq_marlin/gptq_marlin_repack.cu:128-206): thread th of warp w packs
+      // k = 2 * (th % 4) + {0, 1, 8, 9} of columns 16 w + th / 4 and + 8 into word th * 4 + w of the 16 x 64 tile
+      const size_t kk = k & 15, nn = n & 63;
+      const size_t w = nn >> 4, blk = (nn >> 3) & 1, tc_col = nn & 7;
+      const size_t th = tc_col * 4 + ((kk >> 1) & 3);
+      const int v = (int)((kk & 1) + 2 * (kk >> 3) + 4 * blk);   // index into vals[8]
+      const int slot = (v & 1) ? 4 + (v >> 1) : (v >> 1);        // pack_idx[slot] == v
+      const size_t word = ((k >> 4) * (a.N >> 6) + (n >> 6)) * 128 + th * 4 + w;
+      return (static_cast<const uint32_t*>(a.qweight)[word] >> (4 * slot)) & 0xFu;
+    }
     case KSQ_W4_CUTLASS_SM90_COLMAJOR: {  // transpose only: int8 [N, K/2], signed
       uint8_t b = static_cast<const uint8_t*>(a.qweight)[n * (a.K >> 1) + (k >> 1)];
       uint32_t nib = (k & 1) ? (b >> 4) : (b & 0xFu);
@@ -130,7 +141,20 @@ __host__ __device__ inline uint32_t build_sz_word(const RepackArgs& a, size_t id
   size_t c = idx & 15, rest = idx >> 4;
   size_t gi = rest % G, nt = rest / G;
   size_t n = source_column(a, nt * kTileN + c);
-  uint16_t sbits = static_cast<const uint16_t*>(a.scales)[gi * a.N + n];
+  // Marlin keeps scales (and zero points) permuted inside blocks of 64 columns, or of 32 when there is a single
+  // group (MarlinPermuteScales, KS/models/quant/quant_weight.cpp:350-375): entry p of a block is column
+  // p / 8 + 8 * (p % 8), resp. 2 * (p / 8) + {0,1,8,9,16,17,24,25}[p % 8]
+  size_t ns = n;
+  if (a.layout == KSQ_W4_MARLIN) {
+    if (G > 1) {
+      const size_t q = n & 63;
+      ns = (n & ~(size_t)63) + 8 * (q & 7) + (q >> 3);
+    } else {
+      const size_t q = n & 31, pair = q >> 1, odd = q & 1;  // q = 2 i + (8 h + odd): i = pair & 3, h = pair >> 2
+      ns = (n & ~(size_t)31) + 8 * (pair & 3) + 2 * (pair >> 2) + odd;
+    }
+  }
+  uint16_t sbits = static_cast<const uint16_t*>(a.scales)[gi * a.N + ns];
   uint32_t z = 8;
   switch (a.zero_kind) {
     case KSQ_ZERO_AWQ_INT32: {
@@ -138,6 +162,16 @@ __host__ __device__ inline uint32_t build_sz_word(const RepackArgs& a, size_t id
       int i = (int)(n & 7);
       int slot = (i >> 1) + 4 * (i & 1);
       z = (w >> (4 * slot)) & 0xFu;
+      break;
+    }
+    case KSQ_ZERO_MARLIN_INT32: {
+      // MarlinZeroPoints (quant_weight.cpp:397-426): the grouped scale permutation on blocks of 64, then
+      // [0,2,4,6,1,3,5,7] on blocks of 8, then eight consecutive columns per word
+      const size_t q = n & 63, p = 8 * (q & 7) + (q >> 3), r = p & 7;
+      const size_t t = (r & 1) ? 4 + (r >> 1) : (r >> 1);
+      const size_t col = (n & ~(size_t)63) + (p & ~(size_t)7) + t;
+      uint32_t w = static_cast<const uint32_t*>(a.zeros)[gi * (a.N >> 3) + (col >> 3)];
+      z = (w >> (4 * (col & 7))) & 0xFu;
       break;
     }
     case KSQ_ZERO_UINT8:
@@ -172,10 +206,14 @@ __global__ __launch_bounds__(256) void repack_sz_kernel(RepackArgs a, size_t cou
 
 int validate(int layout, const void* qweight, int zero_kind, const void* zeros, const void* scales, int scale_dtype,
              size_t k, size_t n, size_t g, int column_order, const void* dw, const void* dsz) {
-  KSQ_REQUIRE(layout >= KSQ_W4_GPTQ_INT32_KPACK && layout <= KSQ_W4_CUTLASS_SM90_COLMAJOR, KSQ_ERR_INVALID_ARGUMENT,
+  KSQ_REQUIRE(layout >= KSQ_W4_GPTQ_INT32_KPACK && layout <= KSQ_W4_MARLIN, KSQ_ERR_INVALID_ARGUMENT,
               "bad source layout %d", layout);
-  KSQ_REQUIRE(zero_kind >= KSQ_ZERO_NONE && zero_kind <= KSQ_ZERO_ADDITIVE, KSQ_ERR_INVALID_ARGUMENT,
+  KSQ_REQUIRE(zero_kind >= KSQ_ZERO_NONE && zero_kind <= KSQ_ZERO_MARLIN_INT32, KSQ_ERR_INVALID_ARGUMENT,
               "bad zero kind %d", zero_kind);
+  KSQ_REQUIRE(layout != KSQ_W4_MARLIN || n % 64 == 0, KSQ_ERR_UNSUPPORTED,
+              "the Marlin layout needs n %% 64 == 0 (got %zu)", n);
+  KSQ_REQUIRE((zero_kind == KSQ_ZERO_MARLIN_INT32) == (layout == KSQ_W4_MARLIN && zero_kind != KSQ_ZERO_NONE),
+              KSQ_ERR_INVALID_ARGUMENT, "Marlin zero points go with the Marlin weight layout and with no other");
   KSQ_REQUIRE(scale_dtype == KSQ_F16 || scale_dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad scale dtype %d",
               scale_dtype);
   KSQ_REQUIRE(column_order == KSQ_COLS_NATURAL || column_order == KSQ_COLS_HALVES_INTERLEAVED,

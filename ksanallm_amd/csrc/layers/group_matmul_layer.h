@@ -58,7 +58,8 @@ enum GroupWeightLayout {
   GROUP_WEIGHT_AWQ_INT32,
   GROUP_WEIGHT_ROWMAJOR_INT4,
   GROUP_WEIGHT_CUTLASS_SM80,
-  GROUP_WEIGHT_CUTLASS_SM90
+  GROUP_WEIGHT_CUTLASS_SM90,
+  GROUP_WEIGHT_MARLIN  // Marlin tiles; scales in Marlin order; qzeros (AWQ) as Marlin zero points
 };
 Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, const Tensor* qzeros, bool zeros_additive,
                               const Tensor& scales, size_t k, size_t n, size_t groupsize, Tensor& weight,

@@ -162,12 +162,14 @@ Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, c
             : layout == GROUP_WEIGHT_AWQ_INT32    ? KSQ_W4_AWQ_INT32_NPACK
             : layout == GROUP_WEIGHT_CUTLASS_SM80 ? KSQ_W4_CUTLASS_SM80_INTERLEAVED
             : layout == GROUP_WEIGHT_CUTLASS_SM90 ? KSQ_W4_CUTLASS_SM90_COLMAJOR
+            : layout == GROUP_WEIGHT_MARLIN       ? KSQ_W4_MARLIN
                                                   : KSQ_W4_ROWMAJOR_INT4_SIGNED;
   if (perm != nullptr && (perm->dtype != TYPE_INT32 || perm->GetElementNumber() != k))
     KLLM_THROW("RepackGroupQuantWeight: perm must be int32 [k].");
   int zero_kind = KSQ_ZERO_NONE;
   if (qzeros != nullptr) {
-    if (zeros_additive) zero_kind = KSQ_ZERO_ADDITIVE;
+    if (layout == GROUP_WEIGHT_MARLIN) zero_kind = KSQ_ZERO_MARLIN_INT32;
+    else if (zeros_additive) zero_kind = KSQ_ZERO_ADDITIVE;
     else if (qzeros->dtype == TYPE_INT32 || qzeros->dtype == TYPE_UINT32) zero_kind = KSQ_ZERO_AWQ_INT32;
     else zero_kind = KSQ_ZERO_UINT8;
   }

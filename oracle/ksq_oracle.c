@@ -491,6 +491,66 @@ void orc_cutlass_preprocess(const uint8_t* rowmajor, size_t K, size_t N, int arc
   free(b);
 }
 
+/* ---------------------------------------------------------------- Marlin weight layout (F1 input layout)
+ *
+ * gptq_marlin_repack_kernel<256, 4, false> (LK/gptq_marlin/gptq_marlin_repack.cu:31-233) and
+ * awq_marlin_repack_kernel<256, 4> (LK/gptq_marlin/awq_marlin_repack.cu:30-170) with the CUDA launch geometry
+ * written out as loops: tiles of tile_k_size = 16 by tile_n_size = 64 (marlin_params.h:44-45), four warps of 32
+ * threads per tile, one output word per thread.  Pinned by the formulation published with the format
+ * (vLLM's marlin_permute_weights / get_weight_perm, which the reference cites at quant_weight.cpp:348), written
+ * out in the tests with numpy, and by the library's closed-form inverse reproducing the plain repack.
+ */
+static const int MARLIN_TC_OFFSETS[4] = {0, 1, 8, 9};
+static const int MARLIN_PACK_IDX[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+
+static void marlin_store(const uint32_t vals[8], size_t k_tile, size_t n_tile, size_t n_tiles, int th_id, int warp_id,
+                         uint32_t* out) {
+  uint32_t res = 0;
+  for (int i = 0; i < 8; ++i) res |= vals[MARLIN_PACK_IDX[i]] << (i * 4);
+  out[(k_tile * n_tiles + n_tile) * 128 + (size_t)th_id * 4 + (size_t)warp_id] = res; /* :199-206 */
+}
+
+/* qweight: GPTQ int32 [K/8][N] */
+void orc_marlin_repack_gptq(const uint32_t* qweight, size_t K, size_t N, uint32_t* out) {
+  const size_t k_tiles = K / 16, n_tiles = N / 64;
+  for (size_t k_tile = 0; k_tile < k_tiles; ++k_tile)
+    for (size_t n_tile = 0; n_tile < n_tiles; ++n_tile)
+      for (int warp_id = 0; warp_id < 4; ++warp_id)
+        for (int th_id = 0; th_id < 32; ++th_id) {
+          const int tc_col = th_id / 4, tc_row = (th_id % 4) * 2; /* :142-143 */
+          const size_t cur_n = n_tile * 64 + (size_t)warp_id * 16 + (size_t)tc_col;
+          uint32_t vals[8];
+          for (int i = 0; i < 4; ++i) { /* :185-193: the tile's two packed rows, element cur_elem of the tile */
+            const size_t k = k_tile * 16 + (size_t)(tc_row + MARLIN_TC_OFFSETS[i]);
+            vals[i] = (qweight[(k / 8) * N + cur_n] >> (4 * (k % 8))) & 0xF;
+            vals[4 + i] = (qweight[(k / 8) * N + cur_n + 8] >> (4 * (k % 8))) & 0xF;
+          }
+          marlin_store(vals, k_tile, n_tile, n_tiles, th_id, warp_id, out);
+        }
+}
+
+/* qweight: AWQ int32 [K][N/8], AutoAWQ nibble order */
+void orc_marlin_repack_awq(const uint32_t* qweight, size_t K, size_t N, uint32_t* out) {
+  static const int undo_pack[8] = {0, 4, 1, 5, 2, 6, 3, 7}; /* awq_marlin_repack.cu:119-121 */
+  const size_t k_tiles = K / 16, n_tiles = N / 64;
+  for (size_t k_tile = 0; k_tile < k_tiles; ++k_tile)
+    for (size_t n_tile = 0; n_tile < n_tiles; ++n_tile)
+      for (int warp_id = 0; warp_id < 4; ++warp_id)
+        for (int th_id = 0; th_id < 32; ++th_id) {
+          const int tc_col = th_id / 4, tc_row = (th_id % 4) * 2;
+          const int cur_n = warp_id * 16 + tc_col; /* inside the tile */
+          const size_t packed = (n_tile * 64 + (size_t)cur_n) / 8;
+          const int pos = undo_pack[cur_n % 8];
+          uint32_t vals[8];
+          for (int i = 0; i < 4; ++i) { /* :129-138 */
+            const size_t k = k_tile * 16 + (size_t)(tc_row + MARLIN_TC_OFFSETS[i]);
+            vals[i] = (qweight[k * (N / 8) + packed] >> (4 * pos)) & 0xF;
+            vals[4 + i] = (qweight[k * (N / 8) + packed + 1] >> (4 * pos)) & 0xF;
+          }
+          marlin_store(vals, k_tile, n_tile, n_tiles, th_id, warp_id, out);
+        }
+}
+
 /* ---------------------------------------------------------------- desc_act (F3)
  * perm = stable argsort of g_idx (MarlinSortGIdx, KS/models/quant/quant_weight.cpp:455-460: torch::argsort with
  * stable = true); the activations' columns are gathered through it (permute_cols_kernel,

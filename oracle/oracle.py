@@ -293,6 +293,38 @@ def cutlass_step(step, data, K, N):
     return out
 
 
+def marlin_repack(qweight, K, N, kind):
+    """kind 'gptq': int32 [K/8, N]; 'awq': int32 [K, N/8].  Returns the Marlin weight, int32 [K/16, N*2]."""
+    q = _c(qweight).view(np.uint32)
+    out = np.zeros((K // 16, N * 2), dtype=np.uint32)
+    getattr(lib(), "orc_marlin_repack_" + kind)(_p(q), _sz(K), _sz(N), _p(out))
+    return out.view(np.int32)
+
+
+def marlin_permute_scales(s, K, group_size):
+    """MarlinPermuteScales (KS/models/quant/quant_weight.cpp:350-375) on a [G, N] array of any 16-bit dtype."""
+    s = np.ascontiguousarray(s)
+    N = s.shape[1]
+    if group_size < K and group_size != -1:
+        perm = [i + 8 * j for i in range(8) for j in range(8)]
+    else:
+        perm = [2 * i + j for i in range(4) for j in (0, 1, 8, 9, 16, 17, 24, 25)]
+    return np.ascontiguousarray(s.reshape(-1, len(perm))[:, perm].reshape(-1, N))
+
+
+def marlin_zero_points(z):
+    """MarlinZeroPoints (quant_weight.cpp:397-426) for 4 bits: z uint8 [G, N] -> int32 [G, N/8]."""
+    z = _c(z, np.uint8)
+    G, N = z.shape
+    perm = [i + 8 * j for i in range(8) for j in range(8)]
+    zp = z.reshape(-1, 64)[:, perm]
+    zp = zp.reshape(-1, 8)[:, [0, 2, 4, 6, 1, 3, 5, 7]].reshape(G, N).astype(np.uint32)
+    packed = np.zeros((G, N // 8), dtype=np.uint32)
+    for i in range(8):  # MarlinPackCols (:385-395)
+        packed |= zp[:, i::8] << np.uint32(4 * i)
+    return packed.view(np.int32)
+
+
 def act_order_perm(g_idx):
     g_idx = _c(g_idx, np.int32)
     perm = np.empty(g_idx.shape[0], dtype=np.int32)

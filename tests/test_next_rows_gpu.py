@@ -67,10 +67,20 @@ def _repack_ex(case, gpu, layout="gptq", perm=None, order=0):
         src, lay = orc.cutlass_preprocess(c.rowmajor(), 80), capi.W4_CUTLASS_SM80_INTERLEAVED
     elif layout == "cutlass90":
         src, lay = orc.cutlass_preprocess(c.rowmajor(), 90), capi.W4_CUTLASS_SM90_COLMAJOR
+    elif layout == "marlin":
+        lay = capi.W4_MARLIN
+        if c.kind == "gptq":
+            src = orc.marlin_repack(c.gptq_qweight(), c.K, c.N, "gptq")
+        else:
+            src = orc.marlin_repack(c.awq_qweight(), c.K, c.N, "awq")
     else:
         src, lay = c.rowmajor(), capi.W4_ROWMAJOR_INT4_SIGNED
     zk, zeros = (capi.ZERO_NONE, None) if c.z is None else (capi.ZERO_UINT8, _dev(c.z, gpu))
     scales = _dev(c.scales.view(np.int16), gpu)
+    if layout == "marlin":
+        scales = _dev(orc.marlin_permute_scales(c.scales, c.K, c.g).view(np.int16), gpu)
+        if c.z is not None:
+            zk, zeros = capi.ZERO_MARLIN_INT32, _dev(orc.marlin_zero_points(c.z), gpu)
     p = None if perm is None else _dev(perm.astype(np.int32), gpu)
     capi.w4a16_repack_ex(lay, _dev(src, gpu), zk, zeros, scales, capi_dtype(c.dtype), c.K, c.N, c.g, p, order, w, sz)
     torch.cuda.synchronize()
@@ -124,6 +134,38 @@ def test_gemm_from_preprocessed_weights(gpu, layout, dtype, M):
     w, sz = _repack_ex(case, gpu, layout=layout)
     got = _gemm_ex(case, gpu, w, sz)
     orc.assert_parity(got, case.oracle(), f"{layout} {dtype} M={M}")
+
+
+@pytest.mark.parametrize("kind,dtype,M,g", [("gptq", "f16", 16, 128), ("awq", "bf16", 40, 64), ("awq", "f16", 150, 128)])
+def test_gemm_from_marlin_weights(gpu, kind, dtype, M, g):
+    """What the loader's Marlin back end leaves behind (weight tiles, permuted scales, Marlin zero points)."""
+    case = W4Case(2015 + M, M, 768, 192, g=g, kind=kind, dtype=dtype)
+    w, sz = _repack_ex(case, gpu, layout="marlin")
+    got = _gemm_ex(case, gpu, w, sz)
+    orc.assert_parity(got, case.oracle(), f"marlin {kind} {dtype} M={M}")
+
+
+def test_desc_act_marlin_weights(gpu):
+    """The Marlin repack of a desc_act checkpoint already stores the rows in sorted order (has_perm,
+    gptq_marlin_repack.cu:100-114): no row permutation at repack, the loader's perm at run time."""
+    from ksanallm_amd import capi
+
+    K, N, g, M = 512, 128, 128, 20
+    rng = np.random.default_rng(2017)
+    case = W4Case(2018, M, K, N, g=g, kind="gptq", dtype="f16")
+    order = rng.permutation(K)
+    g_idx = np.empty(K, dtype=np.int32)
+    g_idx[order] = np.arange(K, dtype=np.int32) // g
+    perm = np.empty(K, dtype=np.int32)
+    capi.gptq_act_order_perm(g_idx, K, g, perm)
+    sorted_case = W4Case(2018, M, K, N, g=g, kind="gptq", dtype="f16")
+    sorted_case.u = np.ascontiguousarray(case.u[perm])  # what gptq_marlin_repack reads through perm
+    w, sz = _repack_ex(sorted_case, gpu, layout="marlin")
+    got = _gemm_ex(case, gpu, w, sz, perm=perm)
+    s = orc.from_bits(case.scales, orc.F16)
+    wdq = (s[g_idx] * (case.u.astype(np.float32) - 8.0)).astype(np.float32)
+    want = orc.gemm_f32(orc.from_bits(case.act, orc.F16), wdq)
+    orc.assert_parity(got, want, "desc_act through Marlin weights")
 
 
 def test_one_hot_rows_through_cutlass_layout_are_exact(gpu):

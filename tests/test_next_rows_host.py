@@ -211,3 +211,102 @@ def test_silu_mul_oracle_against_library_routine():
     want = (torch.nn.functional.silu(torch.from_numpy(acc[:, :32]).double()) * torch.from_numpy(acc[:, 32:]).double())
     got = orc.silu_mul(acc)
     assert np.allclose(got, want.numpy(), rtol=1e-6, atol=1e-30)
+
+
+# ---- Marlin
+
+def _published_marlin_weights(u):
+    """The Marlin 4-bit weight format as published with it (vLLM's marlin_permute_weights + get_weight_perm + pack_cols,
+    the file the reference cites at quant_weight.cpp:348), in numpy: u [K, N] unsigned nibbles -> int32 [K/16, N*2]."""
+    K, N = u.shape
+    perm = []
+    for i in range(32):
+        perm1 = []
+        col = i // 4
+        for block in (0, 1):
+            for row in (2 * (i % 4), 2 * (i % 4) + 1, 2 * (i % 4 + 4), 2 * (i % 4 + 4) + 1):
+                perm1.append(16 * row + col + 8 * block)
+        for j in range(4):
+            perm.extend(p + 256 * j for p in perm1)
+    perm = np.array(perm).reshape(-1, 8)[:, [0, 2, 4, 6, 1, 3, 5, 7]].ravel()
+    q = u.astype(np.uint32).reshape(K // 16, 16, N // 16, 16).transpose(0, 2, 1, 3).reshape(K // 16, N * 16)
+    q = q.reshape(-1, perm.size)[:, perm].reshape(K // 16, N * 16)
+    packed = np.zeros((K // 16, N * 2), dtype=np.uint32)
+    for i in range(8):
+        packed |= q[:, i::8] << np.uint32(4 * i)
+    return packed.view(np.int32)
+
+
+@pytest.mark.parametrize("K,N", [(128, 64), (256, 192)])
+def test_marlin_repack_restatements_match_the_published_format(K, N):
+    rng = np.random.default_rng(70 + K)
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    want = _published_marlin_weights(u)
+    assert np.array_equal(orc.marlin_repack(orc.gptq_pack(u), K, N, "gptq"), want)
+    assert np.array_equal(orc.marlin_repack(orc.awq_pack(u), K, N, "awq"), want)
+
+
+def test_marlin_scale_and_zero_point_restatements():
+    # each block of 64 columns is read as an 8 x 8 matrix and transposed; a single group uses blocks of 32 instead
+    s = np.arange(2 * 128, dtype=np.uint16).reshape(2, 128)
+    got = orc.marlin_permute_scales(s, 256, 128)
+    want = s.reshape(2, 2, 8, 8).transpose(0, 1, 3, 2).reshape(2, 128)
+    assert np.array_equal(got, want)
+    one = np.arange(64, dtype=np.uint16).reshape(1, 64)
+    got1 = orc.marlin_permute_scales(one, 128, 128)
+    assert [int(x) for x in got1[0, :8]] == [0, 1, 8, 9, 16, 17, 24, 25] and int(got1[0, 8]) == 2
+    assert sorted(int(x) for x in got1[0, :32]) == list(range(32))
+    z = (np.arange(64, dtype=np.uint8) % 16).reshape(1, 64)
+    zp = orc.marlin_zero_points(z).view(np.uint32)
+    cols = z.reshape(8, 8).T.reshape(-1)  # after the 8 x 8 transpose
+    for wd in range(8):
+        for nib, src in enumerate([0, 2, 4, 6, 1, 3, 5, 7]):
+            assert (int(zp[0, wd]) >> (4 * nib)) & 15 == int(cols[8 * wd + src])
+
+
+@pytest.mark.parametrize("kind", ["gptq", "awq"])
+@pytest.mark.parametrize("K,N,g", [(128, 64, 128), (256, 192, 128), (256, 128, 64)])
+def test_host_repack_from_marlin_equals_repack_from_checkpoint(kind, K, N, g):
+    rng = np.random.default_rng(80 + K + N)
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    s = orc.to_bits(np.abs(rng.standard_normal((K // g, N))) * 0.02 + 1e-3, orc.F16)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8) if kind == "awq" else None
+    want_w = np.zeros(K * N // 8, dtype=np.uint32)
+    want_sz = np.zeros((K // g) * N, dtype=np.uint32)
+    if kind == "awq":
+        capi.w4a16_repack_host(capi.W4_AWQ_INT32_NPACK, orc.awq_pack(u), capi.ZERO_AWQ_INT32, orc.awq_pack(z), s,
+                               capi.F16, K, N, g, want_w, want_sz)
+        marlin = orc.marlin_repack(orc.awq_pack(u), K, N, "awq")
+        zk, zsrc = capi.ZERO_MARLIN_INT32, orc.marlin_zero_points(z)
+    else:
+        capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, orc.gptq_pack(u), capi.ZERO_NONE, None, s, capi.F16, K, N, g,
+                               want_w, want_sz)
+        marlin = orc.marlin_repack(orc.gptq_pack(u), K, N, "gptq")
+        zk, zsrc = capi.ZERO_NONE, None
+    got_w = np.zeros_like(want_w)
+    got_sz = np.zeros_like(want_sz)
+    capi.w4a16_repack_host(capi.W4_MARLIN, marlin, zk, zsrc, orc.marlin_permute_scales(s, K, g), capi.F16, K, N, g,
+                           got_w, got_sz)
+    assert np.array_equal(got_w, want_w)
+    assert np.array_equal(got_sz, want_sz)
+
+
+def test_marlin_argument_rules():
+    K, N, g = 128, 64, 128
+    w = np.zeros((K // 16, N * 2), dtype=np.int32)
+    s = np.zeros((1, N), dtype=np.uint16)
+    z8 = np.zeros((1, N), dtype=np.uint8)
+    dw = np.zeros(K * N // 8, dtype=np.uint32)
+    dsz = np.zeros(N, dtype=np.uint32)
+    with pytest.raises(capi.KsqError) as e:  # Marlin weights with zero points in another form
+        capi.w4a16_repack_host(capi.W4_MARLIN, w, capi.ZERO_UINT8, z8, s, capi.F16, K, N, g, dw, dsz)
+    assert e.value.code == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(capi.KsqError) as e:  # Marlin zero points with another weight layout
+        capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, np.zeros((K // 8, N), dtype=np.int32), capi.ZERO_MARLIN_INT32,
+                               np.zeros((1, N // 8), dtype=np.int32), s, capi.F16, K, N, g, dw, dsz)
+    assert e.value.code == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(capi.KsqError) as e:  # n must be a multiple of 64
+        capi.w4a16_repack_host(capi.W4_MARLIN, np.zeros((K // 16, 96), dtype=np.int32), capi.ZERO_NONE, None,
+                               np.zeros((1, 48), dtype=np.uint16), capi.F16, K, 48, g, np.zeros(K * 48 // 8, np.uint32),
+                               np.zeros(48, np.uint32))
+    assert e.value.code == capi.ERR_UNSUPPORTED
