@@ -182,6 +182,7 @@ def main():
                 torch.float16) for k in (4096, 11008)}, {n: torch.empty((64, n), dtype=torch.float16, device=dev)
                                                         for n in (12288, 4096, 22016)},
                                             *workspace_for(torch, capi, dev, 64), stream, 64, dtype)
+        extra["fused_m16"] = fused(torch, capi, layers, acts, outs, stream, M, dtype, dev)
         extra["prefill_m4096"] = prefill(torch, capi, layers[0], dev, stream)
         extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], dev, stream, "f16")
         extra["prefill_m2048"] = prefill(torch, capi, layers[0], dev, stream, M=2048)
@@ -326,6 +327,33 @@ def per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, d
         us = time_graph(torch, stream, launch, 64)
         b = w4a16_bytes(M, k, n)
         table[name] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 3)}
+    return table
+
+
+def fused(torch, capi, layers, acts, outs, stream, M, dtype, dev):
+    """The steps either side of the GEMM folded into it, at the decode batch of the headline: gate_up with the
+    SiLU-mul epilogue (one launch instead of GEMM + activation kernel; the output is half as wide), qkv with a bias
+    row, and qkv of a desc_act checkpoint (column gather of the activations + GEMM, two launches)."""
+    table = {}
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(17)
+    cases = [("gate_up_silu_mul", 2, capi.EPILOGUE_SILU_MUL, False), ("qkv_bias", 0, capi.EPILOGUE_BIAS, False),
+             ("qkv_act_order", 0, capi.EPILOGUE_NONE, True)]
+    for label, idx, epi, act_order in cases:
+        name, k, n = SHAPES_7B[idx]
+        out = torch.empty((M, n // 2 if epi == capi.EPILOGUE_SILU_MUL else n), dtype=outs[n].dtype, device=dev)
+        bias = torch.randn((n,), device=dev, generator=gen).to(outs[n].dtype) if epi == capi.EPILOGUE_BIAS else None
+        perm = torch.randperm(k, device=dev, generator=gen).to(torch.int32) if act_order else None
+        wsb = capi.w4a16_workspace_bytes_ex(M, n, k, act_order)
+        wk = torch.empty(max(wsb, 256), dtype=torch.uint8, device=dev)
+
+        def launch(i, idx=idx, k=k, n=n):
+            _, _, _, w, sz = layers[i % len(layers)].weights[idx]
+            capi.w4a16_gemm_ex(dtype, out, acts[k], w, sz, M, n, k, GROUP, perm, epi, bias, wk, wsb, stream.cuda_stream)
+
+        us = time_graph(torch, stream, launch, 64)
+        b = w4a16_bytes(M, k, n) - (M * n if epi == capi.EPILOGUE_SILU_MUL else 0)
+        table[label] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1)}
     return table
 
 
