@@ -13,6 +13,11 @@ follow KsanaLLM's loader and FP8 helpers (KS = src/ksana_llm, LU = 3rdparty/LLM_
                   stored rounded once to float32
   fp8_quant_*     LU/cuda_fp8_utils.cu:27-44, 85-127         scale = max(absmax/448, 1/(448*512)), q = e4m3(clamp(x/scale))
   fp8_gemm_*      KS/kernels/nvidia/kernel_wrapper.cpp:1033-1041  out = (sum_k a*w) * w_scale[n] * a_scale[m] in float64
+  w4a16_next_*    the same weights as the loader's other back ends leave them, and the steps either side of the GEMM:
+                  cutlass80 / cutlass90  LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508 as whole-array reshapes
+                  marlin*                the format as published with vLLM's marlin_utils (cited at quant_weight.cpp:348)
+                  g_idx / perm / out_desc  desc_act: row k uses scales[g_idx[k]]; perm = stable argsort (quant_weight.cpp:455-460)
+                  out_silu / out_bias    silu(gate) * up of [gate | up] and out + bias, in float64
 
 Run from the repository root:  python tests/golden/make_fixtures.py
 """
@@ -109,6 +114,87 @@ def w4a16_case(seed, M, K, N, g, awq, bf16):
     return d
 
 
+CUTLASS_ROW_MAP = [0, 1, 8, 9, 16, 17, 24, 25, 2, 3, 10, 11, 18, 19, 26, 27,
+                   4, 5, 12, 13, 20, 21, 28, 29, 6, 7, 14, 15, 22, 23, 30, 31]
+
+
+def pack_nibbles(n):
+    n = n.reshape(-1).astype(np.uint8)
+    return (n[0::2] | (n[1::2] << 4)).astype(np.uint8)
+
+
+def cutlass_sm80(u):
+    """u [K, N] unsigned -> bytes: rows permuted in groups of 32, column major, tiles of 64 rows with four columns
+    interleaved, elements [0,2,4,6,1,3,5,7] inside every group of eight, unsigned."""
+    K, N = u.shape
+    p1 = u.reshape(K // 32, 32, N)[:, CUTLASS_ROW_MAP, :].reshape(K, N)
+    regs = p1.T.reshape(N // 4, 4, K // 64, 8, 8)            # [column group, column, row tile, register, element]
+    regs = regs.transpose(0, 2, 1, 3, 4)                     # row tile outside the four columns
+    regs = regs[..., AWQ_ORDER]                              # the register relayout is the same order
+    return pack_nibbles(regs)
+
+
+def cutlass_sm90(u):
+    return pack_nibbles(((u.astype(np.int16) - 8) & 0xF).T)  # transpose only, nibbles stay signed
+
+
+def marlin_weights(u):
+    K, N = u.shape
+    perm = []
+    for i in range(32):
+        perm1 = []
+        for block in (0, 1):
+            for row in (2 * (i % 4), 2 * (i % 4) + 1, 2 * (i % 4 + 4), 2 * (i % 4 + 4) + 1):
+                perm1.append(16 * row + i // 4 + 8 * block)
+        for j in range(4):
+            perm.extend(p + 256 * j for p in perm1)
+    perm = np.array(perm).reshape(-1, 8)[:, AWQ_ORDER].ravel()
+    q = u.astype(np.uint32).reshape(K // 16, 16, N // 16, 16).transpose(0, 2, 1, 3).reshape(-1, perm.size)[:, perm]
+    q = q.reshape(K // 16, N * 16)
+    packed = np.zeros((K // 16, N * 2), dtype=np.uint32)
+    for i in range(8):
+        packed |= q[:, i::8] << np.uint32(4 * i)
+    return packed.view(np.int32)
+
+
+def marlin_scales(s):
+    G, N = s.shape
+    return np.ascontiguousarray(s.reshape(G, N // 64, 8, 8).transpose(0, 1, 3, 2).reshape(G, N))
+
+
+def marlin_zero_points(z):
+    G, N = z.shape
+    zp = marlin_scales(z).reshape(-1, 8)[:, AWQ_ORDER].reshape(G, N).astype(np.uint32)
+    packed = np.zeros((G, N // 8), dtype=np.uint32)
+    for i in range(8):
+        packed |= zp[:, i::8] << np.uint32(4 * i)
+    return packed.view(np.int32)
+
+
+def next_case(seed, M, K, N, g):
+    rng = np.random.default_rng(seed)
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8)
+    sb = f16_bits(np.abs(rng.standard_normal((K // g, N))).astype(np.float32) * 0.02 + 1e-3)
+    ab = f16_bits(rng.standard_normal((M, K)).astype(np.float32))
+    bias = f16_bits(rng.standard_normal(N).astype(np.float32))
+    sv, av = f16_value(sb), f16_value(ab)
+    out = av @ ((u.astype(np.float64) - np.repeat(z, g, axis=0)) * np.repeat(sv, g, axis=0))
+    order = rng.permutation(K)
+    g_idx = np.empty(K, dtype=np.int32)
+    g_idx[order] = np.arange(K, dtype=np.int32) // g
+    out_desc = av @ ((u.astype(np.float64) - 8.0) * sv[g_idx])
+    gate, up = out[:, : N // 2], out[:, N // 2:]
+    return dict(u=u, z=z, scales_bits=sb, act_bits=ab, bias_bits=bias, group=np.int64(g),
+                qweight_gptq=gptq_pack(u), qweight_awq=awq_pack(u), qzeros_awq=awq_pack(z),
+                cutlass80=cutlass_sm80(u), cutlass90=cutlass_sm90(u), marlin=marlin_weights(u),
+                marlin_scales_bits=marlin_scales(sb), marlin_zp=marlin_zero_points(z),
+                g_idx=g_idx, perm=np.argsort(g_idx, kind="stable").astype(np.int32),
+                out=out.astype(np.float32), out_desc=out_desc.astype(np.float32),
+                out_silu=(gate / (1.0 + np.exp(-gate)) * up).astype(np.float32),
+                out_bias=(out + f16_value(bias)[None, :]).astype(np.float32))
+
+
 def main():
     rng = np.random.default_rng(20240607)
     table = e4m3_table()
@@ -125,6 +211,8 @@ def main():
     np.savez_compressed(os.path.join(HERE, "w4a16_awq_f16_5x256x64_g64.npz"), **w4a16_case(2, 5, 256, 64, 64, True, False))
     np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_16x384x128.npz"), **w4a16_case(3, 16, 384, 128, 128, True, True))
     np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_130x256x272.npz"), **w4a16_case(4, 130, 256, 272, 128, True, True))
+
+    np.savez_compressed(os.path.join(HERE, "w4a16_next_f16_12x256x128.npz"), **next_case(5, 12, 256, 128, 128))
 
     # FP8 activation quantisation, per token, fp16 input 8 x 256
     x = (rng.standard_normal((8, 256)) * 0.7).astype(np.float32)

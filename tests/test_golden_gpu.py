@@ -76,3 +76,45 @@ def test_fp8_golden(gpu):
         capi.fp8_gemm(odt, out, aq, a_scale, M, wq, w_scale, N, M, N, K, ws, wsb)
         torch.cuda.synchronize()
         orc.assert_parity(out.float().cpu().numpy(), f["out"], "fp8 golden")
+
+
+@pytest.mark.parametrize("source", ["cutlass80", "cutlass90", "marlin", "desc_act", "silu_mul", "bias"])
+def test_w4a16_next_golden(gpu, source):
+    """The widened entry points against the float64 vectors: weights as the other back ends leave them, a desc_act
+    checkpoint, and the two epilogues."""
+    import torch
+
+    from ksanallm_amd import capi
+
+    f = load("w4a16_next_f16_12x256x128")
+    K, N = f["u"].shape
+    M, g = f["act_bits"].shape[0], int(f["group"])
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)  # noqa: E731
+    wb, sb = capi.w4a16_repack_sizes(K, N, g)
+    weight = torch.empty(wb, dtype=torch.uint8, device=gpu)
+    sz = torch.empty(sb // 4, dtype=torch.int32, device=gpu)
+    scales = dev(f["scales_bits"].view(np.int16))
+    lay, src, zk, zeros, perm, order = capi.W4_AWQ_INT32_NPACK, f["qweight_awq"], capi.ZERO_AWQ_INT32, f["qzeros_awq"], None, 0
+    epi, bias, want, cols = capi.EPILOGUE_NONE, None, f["out"], N
+    if source == "cutlass80":
+        lay, src, zk, zeros = capi.W4_CUTLASS_SM80_INTERLEAVED, f["cutlass80"], capi.ZERO_UINT8, f["z"]
+    elif source == "cutlass90":
+        lay, src, zk, zeros = capi.W4_CUTLASS_SM90_COLMAJOR, f["cutlass90"], capi.ZERO_UINT8, f["z"]
+    elif source == "marlin":
+        lay, src, zk, zeros = capi.W4_MARLIN, f["marlin"], capi.ZERO_MARLIN_INT32, f["marlin_zp"]
+        scales = dev(f["marlin_scales_bits"].view(np.int16))
+    elif source == "desc_act":
+        lay, src, zk, zeros, perm, want = capi.W4_GPTQ_INT32_KPACK, f["qweight_gptq"], capi.ZERO_NONE, None, dev(f["perm"]), f["out_desc"]
+    elif source == "silu_mul":
+        order, epi, want, cols = capi.COLS_HALVES_INTERLEAVED, capi.EPILOGUE_SILU_MUL, f["out_silu"], N // 2
+    elif source == "bias":
+        epi, bias, want = capi.EPILOGUE_BIAS, dev(f["bias_bits"].view(np.int16)), f["out_bias"]
+    capi.w4a16_repack_ex(lay, dev(src), zk, None if zeros is None else dev(zeros), scales, capi.F16, K, N, g, perm, order,
+                         weight, sz)
+    act = dev(f["act_bits"].view(np.int16)).view(torch.float16)
+    wsb = capi.w4a16_workspace_bytes_ex(M, N, K, perm is not None)
+    ws = torch.empty(max(wsb, 256), dtype=torch.uint8, device=gpu)
+    out = torch.full((M, cols), float("nan"), dtype=torch.float16, device=gpu)
+    capi.w4a16_gemm_ex(capi.F16, out, act, weight, sz, M, N, K, g, perm, epi, bias, ws, wsb)
+    torch.cuda.synchronize()
+    orc.assert_parity(out.float().cpu().numpy(), want, f"next golden {source}")
