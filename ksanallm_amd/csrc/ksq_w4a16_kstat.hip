@@ -258,6 +258,11 @@ void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
 // Plan of the k-stationary kernel: row tiles (1, 2 or 4), waves per workgroup (16 for one row tile, else 8), k
 // tiles per wave (the activations of waves x tpw k tiles live in registers: at most 48, 32 or 16 k tiles per
 // workgroup for 1, 2 or 4 row tiles), split count, column tiles per workgroup and batch size.
+static bool env_round4() {
+  const char* e = getenv("KSQ_W4_KSTAT_ROUND4");  // tuning / test switch
+  return !(e && atoi(e) == 0);
+}
+
 KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   KstatPlan p{};
   const size_t ntiles = n / kTileN, ktiles = k / kTileK;
@@ -286,6 +291,24 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   if (wgs < 1) wgs = 1;
   if (wgs > ntiles) wgs = ntiles;
   p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
+  // One row tile: whole batches of four column tiles.  Fewer, fatter workgroups than CUs still win (measured at the
+  // Llama-2-7B shapes: 3 -> 4 and 6 -> 8 column tiles per workgroup): every workgroup reads its whole k range of the
+  // activations from the L2, and a short last batch costs a barrier and a reduction like a full one.
+  if (p.mt == 1 && p.nt_per_wg >= 3 && env_round4()) p.nt_per_wg = (p.nt_per_wg + 3) & ~3;
+  if (const char* e = getenv("KSQ_W4_KSTAT_NT_PER_WG")) {  // tuning / test override: "v" or "ntiles:v,ntiles:v"
+    for (const char* q = e; q && *q;) {
+      const long a = strtol(q, const_cast<char**>(&q), 10);
+      long v = a;
+      bool applies = true;
+      if (*q == ':') {
+        v = strtol(q + 1, const_cast<char**>(&q), 10);
+        applies = (size_t)a == ntiles;
+      }
+      if (applies && v >= 1 && (size_t)v <= ntiles) p.nt_per_wg = (int)v;
+      if (*q == ',') ++q;
+      else break;
+    }
+  }
   p.grid_x = (int)((ntiles + p.nt_per_wg - 1) / p.nt_per_wg);
   if (p.mt == 1) {
     p.nb = p.nt_per_wg >= 3 ? 4 : (p.nt_per_wg >= 2 ? 2 : 1);  // ring depth = nb * tpw tiles in flight per wave
