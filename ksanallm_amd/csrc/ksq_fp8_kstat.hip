@@ -297,6 +297,10 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
   if (wgs < 1) wgs = 1;
   if (wgs > ntiles) wgs = ntiles;
   p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
+  if (const char* e = getenv("KSQ_FP8_NT_PER_WG")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v >= 1 && (size_t)v <= ntiles) p.nt_per_wg = v;
+  }
   p.grid_x = (int)((ntiles + p.nt_per_wg - 1) / p.nt_per_wg);
   // a single row tile reduces after every column tile when the ring is deep enough without batching (measured:
   // finer batches overlap the reduction of one tile with the stream of the next); more row tiles batch by two
