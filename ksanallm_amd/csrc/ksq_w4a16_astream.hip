@@ -12,8 +12,10 @@
 // four lanes reads 64 contiguous bytes (the memory pipeline then takes four lanes per clock instead of one); a lane
 // permutation gives the MFMA operand layout (lane 16 j + c = row c, piece j).
 //
-// Arithmetic as in the other decode kernels: biased nibbles by bit operations, a correction MFMA with -(bias + z),
-// fp32 sums over 64 k scaled by s[g,n].
+// Arithmetic, bf16: biased nibbles by bit operations (every nibble as bias + u with one bias); fp32 sums over 64 k
+// of a (bias + u) by MFMA, the bias and the zero point removed through the row sums of the activations (one more
+// MFMA per row tile and 32-k step, shared by all column tiles), scaled by s[g,n]: the weights stay exact, which bf16
+// needs.  fp16: the weights are dequantised to T((u - z) s) in registers and accumulated directly.
 #include <cstdlib>
 
 #include "ksq_epilogue.h"
@@ -124,28 +126,48 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     for (int mt = 0; mt < MT; ++mt) acc[i][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // 64 k of all column tiles against all row tiles
+  // sum_k a (u - z) = sum_k a (bias + u) - (bias + z) sum_k a: the row sums of the activations (an MFMA against
+  // ones) serve every column tile, so the bias and the zero point cost one multiply-add per output.
   auto compute_half = [&](const u32x4 (&a)[MT][2], const WTile& t, int h) {
+    if constexpr (__is_same(T, _Float16)) {
+      // fp16: the weights are dequantised (T((u - z) s), rounded once) and multiplied straight into the
+      // accumulators: with two or four row tiles that is fewer instructions than scaling every output per group
+#pragma unroll
+      for (int i = 0; i < CNT; ++i) {
+        const typename Dequant<_Float16>::Consts k = Dequant<_Float16>::prepare(t.sz[i][GPT == 2 ? h : 0]);
+#pragma unroll
+        for (int dd = 0; dd < 2; ++dd) {
+          const u32x4 bw = Dequant<_Float16>::run(t.w[i][2 * h + dd], k, m_lo, m_hi, c_lo, c_hi);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[i][mt] = O::mfma(a[mt][dd], bw, acc[i][mt]);
+        }
+      }
+      return;
+    }
+    const u32x4 ones = {O::kOnes, O::kOnes, O::kOnes, O::kOnes};
+    f32x4 S[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) S[mt] = O::mfma(a[mt][0], ones, f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) S[mt] = O::mfma(a[mt][1], ones, S[mt]);
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
       const uint32_t szw = t.sz[i][GPT == 2 ? h : 0];
-      const uint32_t z = szw >> 16;
-      const u32x4 corr = O::correction(z | (z << 16));
       const float s = O::scale_to_float(szw);
+      const float nsz = -s * (O::kBias + (float)(szw >> 16));  // exact: 11 x 11 significant bits
       f32x4 P[MT];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int dd = 0; dd < 2; ++dd) {
-        const u32x4 bw = O::unpack(t.w[i][2 * h + dd], m_lo, m_hi, c_lo, c_hi);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) P[mt] = O::mfma(a[mt][dd], corr, P[mt]);
+        const u32x4 bw = O::unpack_uniform(t.w[i][2 * h + dd], m_lo, c_lo);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) P[mt] = O::mfma(a[mt][dd], bw, P[mt]);
       }
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[i][mt][e] += s * P[mt][e];
+        for (int e = 0; e < 4; ++e) acc[i][mt][e] += s * P[mt][e] + nsz * S[mt][e];
     }
   };
 
@@ -201,9 +223,11 @@ void launch(int mt, int cnt, const AstreamArgs& a, dim3 grid, hipStream_t s) {
     else if (cnt == 3) KSQ_GO(2, 3);
     else KSQ_GO(2, 4);
   } else {
+    constexpr bool kF16 = __is_same(T, _Float16);  // weight-side dequantisation: fewer live registers
     if (cnt == 1) KSQ_GO(4, 1);
-    else if (cnt == 2 || GPT == 2) KSQ_GO(4, 2);
-    else KSQ_GO(4, 3);
+    else if (cnt == 2 || (GPT == 2 && !kF16)) KSQ_GO(4, 2);
+    else if (cnt == 3 || !kF16) KSQ_GO(4, 3);
+    else if constexpr (kF16) KSQ_GO(4, 4);
   }
 #undef KSQ_GO
 }
@@ -233,7 +257,8 @@ int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weig
   // of workgroups that wastes least
   const int mt = m <= 32 ? 2 : 4;
   const int gpt = (int)(kTileK / g);
-  const int cnt_max = mt == 2 ? 4 : (gpt == 1 ? 3 : 2);  // what 256 registers per lane hold without spilling
+  // what 256 registers per lane hold without spilling
+  const int cnt_max = (mt == 2 || dtype == KSQ_F16) ? 4 : (gpt == 1 ? 3 : 2);
   int cnt = (a.ntiles + cus - 1) / cus;
   if (cnt > cnt_max) {
     const int rounds = (a.ntiles + cnt_max * cus - 1) / (cnt_max * cus);

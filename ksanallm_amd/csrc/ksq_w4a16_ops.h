@@ -30,6 +30,18 @@ struct Ops<_Float16> {
   }
   static constexpr uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x00F000F0u;
   static constexpr uint32_t kMagicLo = 0x64006400u, kMagicHi = 0x54005400u;
+  // the same word with every nibble in the 1024 + u form (two more shifts): one bias for all elements, so that
+  // sum a * (bias + z) factors into (bias + z) * sum a
+  static __device__ inline u32x4 unpack_uniform(uint32_t x, uint32_t m_lo, uint32_t c_lo) {
+    u32x4 v;
+    v[0] = (x & m_lo) | c_lo;
+    v[1] = ((x >> 4) & m_lo) | c_lo;
+    v[2] = ((x >> 8) & m_lo) | c_lo;
+    v[3] = ((x >> 12) & m_lo) | c_lo;
+    return v;
+  }
+  static constexpr float kBias = 1024.f;
+  static constexpr uint32_t kOnes = 0x3C003C00u;
   // -(bias + z) per element for the correction MFMA; zc = z replicated into both halves
   static __device__ inline u32x4 correction(uint32_t zc) {
     const uint32_t lo = 0xE400E400u | zc, hi = 0xD400D400u | (zc << 4);
@@ -58,6 +70,11 @@ struct Ops<__bf16> {
   }
   static constexpr uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x000F000Fu;
   static constexpr uint32_t kMagicLo = 0x43004300u, kMagicHi = 0x43004300u;
+  static __device__ inline u32x4 unpack_uniform(uint32_t x, uint32_t m_lo, uint32_t c_lo) {
+    return unpack(x, m_lo, m_lo, c_lo, c_lo);
+  }
+  static constexpr float kBias = 128.f;
+  static constexpr uint32_t kOnes = 0x3F803F80u;
   static __device__ inline u32x4 correction(uint32_t zc) {
     const uint32_t v = 0xC300C300u | zc;
     return u32x4{v, v, v, v};
@@ -68,6 +85,51 @@ struct Ops<__bf16> {
   }
   static __device__ inline float scale_to_float(uint32_t szw) { return __builtin_bit_cast(float, szw << 16); }
   static __device__ inline uint16_t to_bits(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
+};
+
+// Weight-side dequantisation for the kernels with many row tiles: a word of eight nibbles becomes eight fp16
+// values T((u - z) * s), u - z exact and the product rounded once.
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct Dequant;
+
+template <>
+struct Dequant<_Float16> {
+  // per (group, column): packed (s, s), packed (1024 + z), packed (64 + z)
+  struct Consts {
+    uint32_t s2, c_lo, c_hi;
+  };
+  static __device__ inline Consts prepare(uint32_t szw) {
+    const uint32_t z = szw >> 16, zc = z | (z << 16);
+    Consts k;
+    k.s2 = (szw & 0xFFFFu) | (szw << 16);
+    k.c_lo = 0x64006400u | zc;
+    k.c_hi = 0x54005400u | (zc << 4);
+    return k;
+  }
+  static __device__ inline u32x4 run(uint32_t x, const Consts& k, uint32_t m_lo, uint32_t m_hi, uint32_t g_lo,
+                                     uint32_t g_hi) {
+    const uint32_t y = x >> 8;
+    const half2v s = __builtin_bit_cast(half2v, k.s2);
+    const half2v clo = __builtin_bit_cast(half2v, k.c_lo), chi = __builtin_bit_cast(half2v, k.c_hi);
+    half2v r0 = (__builtin_bit_cast(half2v, (x & m_lo) | g_lo) - clo) * s;
+    half2v r1 = (__builtin_bit_cast(half2v, (x & m_hi) | g_hi) - chi) * s;
+    half2v r2 = (__builtin_bit_cast(half2v, (y & m_lo) | g_lo) - clo) * s;
+    half2v r3 = (__builtin_bit_cast(half2v, (y & m_hi) | g_hi) - chi) * s;
+    return u32x4{__builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1), __builtin_bit_cast(uint32_t, r2),
+                 __builtin_bit_cast(uint32_t, r3)};
+  }
+};
+
+template <>
+struct Dequant<__bf16> : Dequant<_Float16> {
+  // scales arrive as bf16 bits; the arithmetic is the fp16 one
+  static __device__ inline Consts prepare(uint32_t szw) {
+    const _Float16 sh = (_Float16)__builtin_bit_cast(float, szw << 16);
+    const uint32_t sb = __builtin_bit_cast(uint16_t, sh);
+    return Dequant<_Float16>::prepare((szw & 0xFFFF0000u) | sb);
+  }
 };
 
 }  // namespace w4

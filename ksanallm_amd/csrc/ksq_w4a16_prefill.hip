@@ -28,7 +28,6 @@ namespace ksq {
 namespace {
 
 using namespace w4;
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
@@ -44,47 +43,6 @@ struct PrefillArgs {
 
 constexpr int kBM = 128;             // rows per workgroup
 constexpr int kMT = 8, kNT = 4;      // MFMA tiles per wave: 8 x 4
-
-template <typename T>
-struct Dequant;
-
-template <>
-struct Dequant<_Float16> {
-  // per (group, column): packed (s, s), packed (1024 + z), packed (64 + z)
-  struct Consts {
-    uint32_t s2, c_lo, c_hi;
-  };
-  static __device__ inline Consts prepare(uint32_t szw) {
-    const uint32_t z = szw >> 16, zc = z | (z << 16);
-    Consts k;
-    k.s2 = (szw & 0xFFFFu) | (szw << 16);
-    k.c_lo = 0x64006400u | zc;
-    k.c_hi = 0x54005400u | (zc << 4);
-    return k;
-  }
-  static __device__ inline u32x4 run(uint32_t x, const Consts& k, uint32_t m_lo, uint32_t m_hi, uint32_t g_lo,
-                                     uint32_t g_hi) {
-    const uint32_t y = x >> 8;
-    const half2v s = __builtin_bit_cast(half2v, k.s2);
-    const half2v clo = __builtin_bit_cast(half2v, k.c_lo), chi = __builtin_bit_cast(half2v, k.c_hi);
-    half2v r0 = (__builtin_bit_cast(half2v, (x & m_lo) | g_lo) - clo) * s;
-    half2v r1 = (__builtin_bit_cast(half2v, (x & m_hi) | g_hi) - chi) * s;
-    half2v r2 = (__builtin_bit_cast(half2v, (y & m_lo) | g_lo) - clo) * s;
-    half2v r3 = (__builtin_bit_cast(half2v, (y & m_hi) | g_hi) - chi) * s;
-    return u32x4{__builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1), __builtin_bit_cast(uint32_t, r2),
-                 __builtin_bit_cast(uint32_t, r3)};
-  }
-};
-
-template <>
-struct Dequant<__bf16> : Dequant<_Float16> {
-  // scales arrive as bf16 bits; the arithmetic is the fp16 one
-  static __device__ inline Consts prepare(uint32_t szw) {
-    const _Float16 sh = (_Float16)__builtin_bit_cast(float, szw << 16);
-    const uint32_t sb = __builtin_bit_cast(uint16_t, sh);
-    return Dequant<_Float16>::prepare((szw & 0xFFFF0000u) | sb);
-  }
-};
 
 // bf16 [M][K] -> fp16 [M][K] * 2^-e[row] (exact: power-of-two shift of an 8-bit significand into 11 bits), with
 // e[row] chosen so that the row maximum lands at 2^14; row_scale[row] = 2^e.  One workgroup per row; the row stays
