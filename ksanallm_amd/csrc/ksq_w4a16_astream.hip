@@ -80,16 +80,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     u32x4 w[CNT];
     uint32_t sz[CNT][GPT];
   };
+  // The per-lane part of every address is a loop constant and the moving part (k tile, column tile) goes into the
+  // scalar offset of the buffer instruction, which costs no vector arithmetic.  The hardware checks only the vector
+  // offset against the resource's range, so whatever must read as zero (a k tile past the slice, a column tile past
+  // the workgroup's range, a row past M) is parked there, at an offset that is out of range by itself.
   auto load_w = [&](WTile& t, int kt) {
     const bool ok = kt < kt_end;
 #pragma unroll
     for (int i = 0; i < CNT; ++i) {
-      t.w[i] = __builtin_bit_cast(
-          u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, ok ? w_lane + kt * 1024u + i * w_stride : 0x80000000u, 0, 2));
+      const bool live = ok && i < count;  // uniform
+      t.w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, live ? w_lane : 0x80000000u,
+                                                                               live ? kt * 1024 + i * (int)w_stride : 0, 2));
 #pragma unroll
       for (int gi = 0; gi < GPT; ++gi)
-        t.sz[i][gi] = __builtin_amdgcn_raw_buffer_load_b32(
-            rs_sz, ok ? sz_lane + (kt * GPT + gi) * 64u + i * sz_stride : 0x80000000u, 0, 0);
+        t.sz[i][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, live ? sz_lane : 0x80000000u,
+                                                           live ? (kt * GPT + gi) * 64 + i * (int)sz_stride : 0, 0);
     }
   };
   // half h of k tile kt: 32-k steps 2h and 2h + 1 of all row tiles, as loaded (before the lane permutation)
@@ -100,9 +105,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
       for (int dd = 0; dd < 2; ++dd)
         a[mt][dd] = __builtin_bit_cast(
-            u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                       rs_a, (ok && a_row[mt] != 0x80000000u) ? a_row[mt] + (kt * kTileK + 32 * (2 * h + dd)) * 2u : 0x80000000u,
-                       0, 0));
+            u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ok ? a_row[mt] : 0x80000000u,
+                                                         ok ? (kt * kTileK + 32 * (2 * h + dd)) * 2 : 0, 0));
   };
   auto permute = [&](u32x4 (&a)[MT][2]) {
 #pragma unroll
