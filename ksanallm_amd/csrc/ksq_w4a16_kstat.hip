@@ -229,9 +229,11 @@ void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
       if (nb >= 4) KSQ_GO(1, 2, 4, 16);
       else if (nb >= 2) KSQ_GO(1, 2, 2, 16);
       else KSQ_GO(1, 2, 1, 16);
-    } else {
+    } else if (tpw == 3) {
       if (nb >= 2) KSQ_GO(1, 3, 2, 16);
       else KSQ_GO(1, 3, 1, 16);
+    } else {
+      KSQ_GO(1, 4, 1, 16);  // 64 registers of activations: room for a ring of one column tile only
     }
   } else if (pl.mt == 2) {
     if (tpw <= 2) {
@@ -256,8 +258,19 @@ void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
 }  // namespace
 
 // Plan of the k-stationary kernel: row tiles (1, 2 or 4), waves per workgroup (16 for one row tile, else 8), k
-// tiles per wave (the activations of waves x tpw k tiles live in registers: at most 48, 32 or 16 k tiles per
+// tiles per wave (the activations of waves x tpw k tiles live in registers: at most 64, 32 or 16 k tiles per
 // workgroup for 1, 2 or 4 row tiles), split count, column tiles per workgroup and batch size.
+// One row tile: three k tiles per wave (48 per workgroup) leave registers for a weight ring of two column tiles.
+// Four (64: K = 8192 without a split across workgroups) leave room for a ring of one, which pays only where N is
+// large (measured at the Llama-2-70B shapes: qkv -13 %, gate_up -6 %, o +10 %; beyond 64 k tiles the split wins).
+static int kstat_tpw_max_one_row_tile(size_t ktiles, size_t ntiles, int cus) {
+  if (const char* e = getenv("KSQ_W4_KSTAT_TPW_MAX")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v >= 1 && v <= 4) return v;
+  }
+  return (ktiles > 48 && ktiles <= 64 && 2 * ntiles >= 5 * (size_t)cus) ? 4 : 3;
+}
+
 static bool env_round4() {
   const char* e = getenv("KSQ_W4_KSTAT_ROUND4");  // tuning / test switch
   return !(e && atoi(e) == 0);
@@ -270,7 +283,7 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   if (!p.ok) return p;
   p.mt = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
   p.nw = p.mt == 1 ? 16 : 8;
-  const size_t tpw_max = p.mt == 1 ? 3 : (p.mt == 2 ? 4 : 2);
+  const size_t tpw_max = p.mt == 1 ? (size_t)kstat_tpw_max_one_row_tile(ktiles, ntiles, cus) : (p.mt == 2 ? 4 : 2);
   const size_t cap = (size_t)p.nw * tpw_max;
   size_t ksplit = (ktiles + cap - 1) / cap;
   if (const char* e = getenv("KSQ_W4_KSPLIT")) {  // tuning / test override; never below what the registers need
@@ -313,6 +326,7 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   if (p.mt == 1) {
     p.nb = p.nt_per_wg >= 3 ? 4 : (p.nt_per_wg >= 2 ? 2 : 1);  // ring depth = nb * tpw tiles in flight per wave
     if (p.tpw >= 3 && p.nb > 2) p.nb = 2;                       // register budget of 16 waves per workgroup
+    if (p.tpw >= 4) p.nb = 1;
   } else {
     p.nb = p.nt_per_wg >= 2 ? 2 : 1;
   }

@@ -97,6 +97,21 @@ def test_m_sweep_both_decode_routes(gpu, dtype, route, M):
     orc.assert_parity(got, case.oracle(), f"M={M} {dtype} route={route}")
 
 
+@pytest.mark.parametrize("dtype,g", [("f16", 128), ("bf16", 64)])
+@pytest.mark.parametrize("tpw_max", [1, 2, 3, 4])
+@pytest.mark.parametrize("M,K", [(1, 8192), (16, 7168), (9, 2048)])
+def test_k_tiles_per_wave(gpu, dtype, g, tpw_max, M, K):
+    """One row tile with 1..4 k tiles per wave (a smaller maximum forces a split of K across workgroups; four covers
+    K = 8192 inside one workgroup with a ring of a single column tile)."""
+    case = W4Case(1400 + K // 128 + M, M, K, 336, g=g, kind="awq", dtype=dtype)
+    dev = W4Device(case, gpu)
+    with _env(KSQ_W4_KSTAT_TPW_MAX=tpw_max):
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"tpw_max={tpw_max} {dtype} M={M} K={K}")
+    assert np.array_equal(got1, got2)
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("kind,g", [("gptq", 128), ("gptq", 64), ("awq", 64)])
 def test_group_sizes_and_kinds(gpu, dtype, kind, g):
