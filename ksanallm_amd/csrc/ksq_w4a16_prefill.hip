@@ -602,7 +602,9 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     a.mblocks = (int)((m + kBM - 1) / kBM);
     // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; measured at
     // M = 4096 they win up to N = 8192 (fewer, fatter workgroups), four waves (128 x 256, two per CU) beyond.
-    nw = ((size_t)a.mblocks * ((a.ntiles + 31) / 32) >= (size_t)di->cus && a.ntiles <= 512) ? 8 : 4;
+    // (and up to N = 12288 when they fill every CU at least twice: qkv of Llama-2-7B at M = 4096, +5 %)
+    const size_t wgs8 = (size_t)a.mblocks * ((a.ntiles + 31) / 32);
+    nw = ((wgs8 >= (size_t)di->cus && a.ntiles <= 512) || (wgs8 >= 2 * (size_t)di->cus && a.ntiles <= 768)) ? 8 : 4;
     if (const char* e = getenv("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 4 || v == 8) nw = v;
