@@ -69,8 +69,16 @@ unsigned* counter_slot_device_ptr() {
   return pd->counters + (size_t)slot * kCountersPerSlot;
 }
 
+const char* tuning_env(const char* name) {
+  static const bool enabled = [] {
+    const char* e = getenv("KSQ_TUNING");
+    return e && atoi(e) != 0;
+  }();
+  return enabled ? getenv(name) : nullptr;
+}
+
 static int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
+  const char* v = tuning_env(name);
   if (!v || !*v) return dflt;
   return atoi(v);
 }

@@ -663,7 +663,7 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
                               static_cast<hipStream_t>(stream), epi);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
   if (m <= 64) {
-    const char* e = getenv("KSQ_FP8_KSTAT");  // tuning / test switch: 0 sends small m to the streaming kernel
+    const char* e = tuning_env("KSQ_FP8_KSTAT");  // tuning / test switch: 0 sends small m to the streaming kernel
     if (!(e && atoi(e) == 0)) {
       const Fp8KstatPlan kp = fp8_kstat_plan(m, n, k, di->cus, workspace ? workspace_bytes : 0);
       if (kp.ok)

@@ -280,7 +280,7 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
   const size_t nw = p.mt == 4 ? 8 : 16;
   const size_t cap = nw * (p.mt == 2 ? 2u : 4u);
   size_t ksplit = (stages + cap - 1) / cap;
-  if (const char* e = getenv("KSQ_FP8_KSPLIT")) {  // tuning / test override; never below what the registers need
+  if (const char* e = tuning_env("KSQ_FP8_KSPLIT")) {  // tuning / test override; never below what the registers need
     const size_t v = (size_t)atoi(e);
     if (v > ksplit && v <= stages) ksplit = v;
   }
@@ -297,7 +297,7 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
   if (wgs < 1) wgs = 1;
   if (wgs > ntiles) wgs = ntiles;
   p.nt_per_wg = (int)((ntiles + wgs - 1) / wgs);
-  if (const char* e = getenv("KSQ_FP8_NT_PER_WG")) {  // tuning / test override
+  if (const char* e = tuning_env("KSQ_FP8_NT_PER_WG")) {  // tuning / test override
     const int v = atoi(e);
     if (v >= 1 && (size_t)v <= ntiles) p.nt_per_wg = v;
   }
@@ -306,7 +306,7 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
   // finer batches overlap the reduction of one tile with the stream of the next); more row tiles batch by two
   p.nb = p.mt >= 2 ? 2 : (p.tpw == 4 ? 1 : (p.tpw == 2 ? 2 : 4));
   if (p.nb > p.nt_per_wg) p.nb = p.nt_per_wg >= 2 ? 2 : 1;
-  if (const char* e = getenv("KSQ_FP8_NB")) {  // tuning override
+  if (const char* e = tuning_env("KSQ_FP8_NB")) {  // tuning override
     const int v = atoi(e);
     if (v == 1 || v == 2 || (v == 4 && p.mt == 1 && p.tpw < 4)) p.nb = v;
   }

@@ -373,7 +373,7 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
   const DeviceInfo* di = device_info();
   KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
   int tile = ((m + 255) / 256) * ((n + 255) / 256) >= (size_t)di->cus ? 256 : 128;
-  if (const char* e = getenv("KSQ_FP8_PREFILL_TILE")) {  // tuning / test override
+  if (const char* e = tuning_env("KSQ_FP8_PREFILL_TILE")) {  // tuning / test override
     const int v = atoi(e);
     if (v == 128 || v == 256) tile = v;
   }

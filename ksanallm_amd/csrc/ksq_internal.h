@@ -23,6 +23,12 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
     if (!(cond)) return ::ksq::fail((code), __VA_ARGS__); \
   } while (0)
 
+// ---- tuning / test overrides -------------------------------------------------------------------------------
+// The launch planners can be overridden through KSQ_* environment variables.  They are looked up only in a process
+// that had KSQ_TUNING=1 in its environment when the library was first used: otherwise this returns nullptr without
+// touching the environment, so the launch path of a serving process makes no getenv calls.
+const char* tuning_env(const char* name);
+
 // ---- fragment-order geometry -------------------------------------------------------------------------------
 constexpr int kTileN = 16;        // columns per weight tile
 constexpr int kTileK = 128;       // k per weight tile

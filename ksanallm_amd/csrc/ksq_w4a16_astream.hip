@@ -268,7 +268,7 @@ int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weig
     const int rounds = (a.ntiles + cnt_max * cus - 1) / (cnt_max * cus);
     cnt = (a.ntiles + rounds * cus - 1) / (rounds * cus);
   }
-  if (const char* e = getenv("KSQ_W4_ASTREAM_CNT")) {  // tuning / test override
+  if (const char* e = tuning_env("KSQ_W4_ASTREAM_CNT")) {  // tuning / test override
     const int v = atoi(e);
     if (v > 0) cnt = v;
   }

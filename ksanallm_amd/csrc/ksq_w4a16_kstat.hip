@@ -264,7 +264,7 @@ void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
 // Four (64: K = 8192 without a split across workgroups) leave room for a ring of one, which pays only where N is
 // large (measured at the Llama-2-70B shapes: qkv -13 %, gate_up -6 %, o +10 %; beyond 64 k tiles the split wins).
 static int kstat_tpw_max_one_row_tile(size_t ktiles, size_t ntiles, int cus) {
-  if (const char* e = getenv("KSQ_W4_KSTAT_TPW_MAX")) {  // tuning / test override
+  if (const char* e = tuning_env("KSQ_W4_KSTAT_TPW_MAX")) {  // tuning / test override
     const int v = atoi(e);
     if (v >= 1 && v <= 4) return v;
   }
@@ -272,7 +272,7 @@ static int kstat_tpw_max_one_row_tile(size_t ktiles, size_t ntiles, int cus) {
 }
 
 static bool env_round4() {
-  const char* e = getenv("KSQ_W4_KSTAT_ROUND4");  // tuning / test switch
+  const char* e = tuning_env("KSQ_W4_KSTAT_ROUND4");  // tuning / test switch
   return !(e && atoi(e) == 0);
 }
 
@@ -286,7 +286,7 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   const size_t tpw_max = p.mt == 1 ? (size_t)kstat_tpw_max_one_row_tile(ktiles, ntiles, cus) : (p.mt == 2 ? 4 : 2);
   const size_t cap = (size_t)p.nw * tpw_max;
   size_t ksplit = (ktiles + cap - 1) / cap;
-  if (const char* e = getenv("KSQ_W4_KSPLIT")) {  // tuning / test override; never below what the registers need
+  if (const char* e = tuning_env("KSQ_W4_KSPLIT")) {  // tuning / test override; never below what the registers need
     const size_t v = (size_t)atoi(e);
     if (v > ksplit && v <= ktiles) ksplit = v;
   }
@@ -308,7 +308,7 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   // Llama-2-7B shapes: 3 -> 4 and 6 -> 8 column tiles per workgroup): every workgroup reads its whole k range of the
   // activations from the L2, and a short last batch costs a barrier and a reduction like a full one.
   if (p.mt == 1 && p.nt_per_wg >= 3 && env_round4()) p.nt_per_wg = (p.nt_per_wg + 3) & ~3;
-  if (const char* e = getenv("KSQ_W4_KSTAT_NT_PER_WG")) {  // tuning / test override: "v" or "ntiles:v,ntiles:v"
+  if (const char* e = tuning_env("KSQ_W4_KSTAT_NT_PER_WG")) {  // tuning / test override: "v" or "ntiles:v,ntiles:v"
     for (const char* q = e; q && *q;) {
       const long a = strtol(q, const_cast<char**>(&q), 10);
       long v = a;

@@ -541,7 +541,7 @@ bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g) 
   (void)g;
   (void)dtype;
   size_t min_m = 65;
-  if (const char* e = getenv("KSQ_W4_PREFILL_MIN_M")) {  // tuning / test override
+  if (const char* e = tuning_env("KSQ_W4_PREFILL_MIN_M")) {  // tuning / test override
     const int v = atoi(e);
     if (v >= 1) min_m = (size_t)v;
   }
@@ -577,7 +577,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   // Row tile of the workgroup: 128 rows when such tiles (128 x 256) give every CU at least two workgroups, else 64
   // rows with deeper prefetch.
   int rows = ((m + 127) / 128) * ((size_t)(a.ntiles + 15) / 16) >= 2 * (size_t)di->cus ? 128 : 64;
-  if (const char* e = getenv("KSQ_W4_PREFILL_ROWS")) {  // tuning / test override
+  if (const char* e = tuning_env("KSQ_W4_PREFILL_ROWS")) {  // tuning / test override
     const int v = atoi(e);
     if (v == 64 || v == 128) rows = v;
   }
@@ -588,7 +588,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     // column tiles per wave: as many (4, 2, 1) as still give every CU two workgroups
     int knt = 4;
     while (knt > 1 && (size_t)a.mblocks * ((a.ntiles + 4 * knt - 1) / (4 * knt)) < 2 * (size_t)di->cus) knt >>= 1;
-    if (const char* e = getenv("KSQ_W4_PREFILL_NT")) {  // tuning / test override
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_NT")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 1 || v == 2 || v == 4) knt = v;
     }
@@ -605,7 +605,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     // (and up to N = 12288 when they fill every CU at least twice: qkv of Llama-2-7B at M = 4096, +5 %)
     const size_t wgs8 = (size_t)a.mblocks * ((a.ntiles + 31) / 32);
     nw = ((wgs8 >= (size_t)di->cus && a.ntiles <= 512) || (wgs8 >= 2 * (size_t)di->cus && a.ntiles <= 768)) ? 8 : 4;
-    if (const char* e = getenv("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 4 || v == 8) nw = v;
     }
