@@ -273,10 +273,12 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, s, epi);
   if (w4a16_astream_supported(m, n, k)) {
     // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
-    // never slower than the k-stationary one; with two it wins only while every workgroup gets one to four
-    // column tiles.
-    const size_t ntiles = n / kTileN;
-    const bool dflt = m > 32 || (ntiles > (size_t)di->cus && ntiles <= 4 * (size_t)di->cus);
+    // never slower than the k-stationary one.  With two it wins while every workgroup gets one to four column
+    // tiles (exactly one only up to 24 rows: every workgroup re-reads all activations from L2, which then weighs
+    // as much as its weights), loses between four and eight where the last round of workgroups is mostly empty,
+    // and wins again from eight tiles per compute unit on.
+    const size_t ntiles = n / kTileN, cus = (size_t)di->cus;
+    const bool dflt = m > 32 || (ntiles > cus && ntiles <= 4 * cus) || ntiles >= 8 * cus || (ntiles == cus && m <= 24);
     if (env_int("KSQ_W4_ASTREAM", dflt ? 1 : 0) != 0)
       return w4a16_launch_astream(dtype, out, act, weight, sz, m, n, k, g, di->cus, s, epi);
   }

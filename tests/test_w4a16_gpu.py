@@ -174,6 +174,7 @@ def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("lds", [0, 1])
 @pytest.mark.parametrize("cnt", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "awq", 128, 17, 640, 528),      # five k tiles over eight waves: three waves idle, odd slices
@@ -182,12 +183,13 @@ def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
     ("bf16", "gptq", 64, 64, 128, 4112),    # a single k tile, more column tiles than compute units
     ("f16", "awq", 64, 48, 2048, 1040),
 ])
-def test_accumulator_stationary_route(gpu, cnt, dtype, kind, g, M, K, N):
+def test_accumulator_stationary_route(gpu, lds, cnt, dtype, kind, g, M, K, N):
     """The 17 <= M <= 64 kernel that keeps only accumulators and streams both operands, with every number of column
-    tiles per workgroup (0 = the launcher's own choice); twice, bit for bit."""
+    tiles per workgroup (0 = the launcher's own choice) and the activations through registers + lane permutation or
+    through LDS; twice, bit for bit."""
     case = W4Case(1300 + cnt + M, M, K, N, g=g, kind=kind, dtype=dtype)
     dev = W4Device(case, gpu)
-    env = dict(KSQ_W4_ASTREAM=1)
+    env = dict(KSQ_W4_ASTREAM=1, KSQ_W4_ASTREAM_LDS=lds)
     if cnt:
         env["KSQ_W4_ASTREAM_CNT"] = cnt
     with _env(**env):
