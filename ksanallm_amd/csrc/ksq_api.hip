@@ -216,6 +216,11 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     if (p.partial_bytes > best) best = p.partial_bytes;
     KstatPlan kp = w4a16_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
     if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
+    const size_t am = mm < max_m ? mm : max_m;
+    if (w4a16_astream_supported(am, n, k)) {
+      const AstreamPlan ap = w4a16_astream_plan(am, n, k, cus, (size_t)-1);
+      if (ap.partial_bytes > best) best = ap.partial_bytes;
+    }
   }
   if (max_m >= 65) {  // the element type is not known here: size for the bf16 route of the prefill kernel
     const size_t pf = w4a16_prefill_workspace_bytes(KSQ_BF16, max_m, k);
@@ -274,13 +279,14 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   if (w4a16_astream_supported(m, n, k)) {
     // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
     // never slower than the k-stationary one.  With two it wins while every workgroup gets one to four column
-    // tiles (exactly one only up to 24 rows: every workgroup re-reads all activations from L2, which then weighs
-    // as much as its weights), loses between four and eight where the last round of workgroups is mostly empty,
-    // and wins again from eight tiles per compute unit on.
+    // tiles and loses beyond that, where its last round of workgroups is mostly empty or, with very wide weights,
+    // it depends on the clock the device happens to hold.
     const size_t ntiles = n / kTileN, cus = (size_t)di->cus;
-    const bool dflt = m > 32 || (ntiles > cus && ntiles <= 4 * cus) || ntiles >= 8 * cus || (ntiles == cus && m <= 24);
-    if (env_int("KSQ_W4_ASTREAM", dflt ? 1 : 0) != 0)
-      return w4a16_launch_astream(dtype, out, act, weight, sz, m, n, k, g, di->cus, s, epi);
+    const bool dflt = m > 32 || (ntiles >= cus && ntiles <= 4 * cus);
+    if (env_int("KSQ_W4_ASTREAM", dflt ? 1 : 0) != 0) {
+      const AstreamPlan ap = w4a16_astream_plan(m, n, k, di->cus, workspace_bytes);
+      return w4a16_launch_astream(dtype, ap, out, act, weight, sz, m, n, k, g, di->cus, workspace, s, epi);
+    }
   }
   if (m <= (size_t)env_int("KSQ_W4_KSTAT_MAX_M", 64) && env_int("KSQ_W4_KSTAT", 1) != 0) {
     KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace_bytes);

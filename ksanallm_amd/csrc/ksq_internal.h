@@ -143,11 +143,17 @@ int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* 
                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
                         const Epilogue& epi = Epilogue());
 
-// accumulator-stationary decode kernel for 17 <= m <= 64 (no workspace, K never split across workgroups)
+// accumulator-stationary decode kernel for 17 <= m <= 64
+struct AstreamPlan {
+  int mt;      // 16-row tiles (2 or 4)
+  int ksplit;  // grid.y
+  size_t partial_bytes;
+};
 bool w4a16_astream_supported(size_t m, size_t n, size_t k);
-int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, int cus, hipStream_t s,
-                         const Epilogue& epi = Epilogue());
+AstreamPlan w4a16_astream_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+int w4a16_launch_astream(int dtype, const AstreamPlan& plan, void* out, const void* act, const void* weight,
+                         const void* sz, size_t m, size_t n, size_t k, size_t g, int cus, void* workspace,
+                         hipStream_t s, const Epilogue& epi = Epilogue());
 
 struct Fp8KstatPlan {
   bool ok;        // the k-stationary kernel takes this shape (m <= 64)

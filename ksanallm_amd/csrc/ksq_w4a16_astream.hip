@@ -6,7 +6,12 @@
 // streams the activation fragments of all MT row tiles (from the L2: every workgroup reads all activations once) and
 // the CNT weight tiles (from HBM, once per device), one k tile ahead for the weights and half a k tile ahead for the
 // activations.  No barrier and no LDS until the end, where the 8 k slices of every (column tile, row tile) are
-// summed through LDS in a fixed order.  K is never split across workgroups: no workspace, no fix-up pass.
+// summed through LDS in a fixed order.
+//
+// Every workgroup reads all activations of its k range from the L2, M x K x 2 bytes for one to four weight tiles of
+// K x 8 bytes each: with few column tiles per compute unit that is most of what a compute unit moves.  K is then
+// split over grid.y as well (two or four ways), which divides that traffic; the partial tiles of the splits go
+// through the workspace and the last workgroup to arrive at a tile adds them in split order (deterministic).
 //
 // Activation loads put lane l on row l / 4 and 16-byte piece l % 4 of a 32-k step, so that every aligned group of
 // four lanes reads 64 contiguous bytes (the memory pipeline then takes four lanes per clock instead of one); a lane
@@ -33,8 +38,53 @@ struct AstreamArgs {
   const void* act;     // [M][K] T
   void* out;           // [M][N] T
   int M, N, K, KT, G, ntiles;
+  int ksplit;          // grid.y
+  f32x4* partial;      // [ksplit][ntiles][MT][64], ksplit > 1 only
+  unsigned* counters;  // [ntiles][MT], zero between launches
   Epilogue epi;
 };
+
+// k tiles [begin, end) of wave `wave` of the workgroup of split blockIdx.y
+struct KRange {
+  int wg_begin, begin, end;
+};
+__device__ inline KRange astream_k_range(const AstreamArgs& p, int wave) {
+  KRange r;
+  r.wg_begin = (int)(((long)p.KT * blockIdx.y) / p.ksplit);
+  const int wg_end = (int)(((long)p.KT * (blockIdx.y + 1)) / p.ksplit);
+  const int slice = (wg_end - r.wg_begin + 7) / 8;
+  r.begin = r.wg_begin + wave * slice;
+  r.end = r.begin + slice < wg_end ? r.begin + slice : wg_end;
+  return r;
+}
+
+// What a wave does with output tile (column tile nt, row tile mt) once the k slices of its workgroup are summed:
+// store it, or with K split over workgroups park it and, as the last split to arrive, add all of them up first.
+// Every lane of the wave makes the call.
+template <typename T, int MT>
+__device__ inline void astream_finish_tile(const AstreamArgs& p, f32x4 sum, int nt, int mt, int lane) {
+  bool store = true;
+  if (p.ksplit > 1) {
+    const size_t stride = (size_t)p.ntiles * MT * 64;
+    const size_t tile = ((size_t)nt * MT + mt) * 64 + lane;
+    store_agent(p.partial + (size_t)blockIdx.y * stride + tile, sum);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned* counter = p.counters + nt * MT + mt;
+    unsigned arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    store = arrived == (unsigned)(p.ksplit - 1);
+    if (store) {
+      asm volatile("" ::: "memory");
+      sum = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + (size_t)sp * stride + tile);
+      if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  if (store)
+    epi_store_acc<T>(p.epi, static_cast<uint16_t*>(p.out), sum, 16 * mt + 4 * (lane >> 4), nt * 16 + (lane & 15), p.M,
+                     p.N, true);
+}
 
 template <typename T, int GPT, int MT, int CNT>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_astream_kernel(AstreamArgs p) {
@@ -49,12 +99,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   const int nt_begin = blockIdx.x * CNT;
   int count = p.ntiles - nt_begin;
   count = count < CNT ? count : CNT;
-  // k slice of this wave, rounded up to an even number of tiles (the loop below runs in pairs; tiles past the end
-  // are parked out of range and read as zero)
-  const int slice = (p.KT + kWaves - 1) / kWaves;
-  const int kt_begin = wave * slice;
-  int kt_end = kt_begin + slice;
-  kt_end = kt_end < p.KT ? kt_end : p.KT;
+  // k slice of this wave (the loop below prefetches one tile ahead; tiles past the end are parked out of range and
+  // read as zero)
+  const KRange kr = astream_k_range(p, wave);
+  const int kt_begin = kr.begin, kt_end = kr.end;
 
   // Resources cover exactly this workgroup's column tiles: tiles past `count` read as zero without traffic.
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
@@ -198,6 +246,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   __builtin_amdgcn_sched_barrier(0);
   for (int kt = kt_begin; kt < kt_end; kt += 2) {
     tile(w0, w1, kt, kt + 1);
+    if (kt + 1 >= kt_end) break;  // odd slice: what was prefetched for the missing tile is zeros
     tile(w1, w0, kt + 1, kt + 2);
   }
 
@@ -207,13 +256,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) red[((i * MT + mt) * kWaves + wave) * 64 + lane] = acc[i][mt];
   __syncthreads();
-  uint16_t* out = static_cast<uint16_t*>(p.out);
   for (int q = wave; q < kTiles; q += kWaves) {
     const int i = q / MT, mt = q - i * MT;
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ww = 0; ww < kWaves; ++ww) sum += red[(q * kWaves + ww) * 64 + lane];
-    if (i < count) epi_store_acc<T>(p.epi, out, sum, 16 * mt + 4 * j, (nt_begin + i) * 16 + c, p.M, p.N, true);
+    if (i < count) astream_finish_tile<T, MT>(p, sum, nt_begin + i, mt, lane);
   }
 }
 
@@ -278,10 +326,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   const int nt_begin = blockIdx.x * CNT;
   int count = p.ntiles - nt_begin;
   count = count < CNT ? count : CNT;
-  const int slice = (p.KT + kWaves - 1) / kWaves;
-  const int kt_begin = wave * slice;
-  int kt_end = kt_begin + slice;
-  kt_end = kt_end < p.KT ? kt_end : p.KT;
+  const KRange kr = astream_k_range(p, wave);
+  const int kt_begin = kr.begin, kt_end = kr.end;
 
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(static_cast<const char*>(p.weight) + (size_t)nt_begin * p.KT * 1024), 0,
@@ -322,10 +368,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
                                                            live ? (kt * GPT + gi) * 64 + i * (int)sz_stride : 0, 0);
     }
   };
-  // half h of k tile kt into this wave's part of `buf`.  A tile past the slice repeats the slice's first tile (tile 0
-  // for a wave whose slice is empty): its weights read as zero, so whatever finite activations stand in for it
+  // half h of k tile kt into this wave's part of `buf`.  A tile past the slice repeats the slice's first tile (the
+  // workgroup's first for a wave whose slice is empty): its weights read as zero, so whatever finite activations stand in for it
   // contribute nothing.  The scalar offset is not range-checked by the hardware, hence the clamp.
-  const int kt_safe = kt_begin < p.KT ? kt_begin : 0;
+  const int kt_safe = kt_begin < kt_end ? kt_begin : kr.wg_begin;
   auto load_a = [&](u32x4* buf, int kt, int h) {
     const int ktc = kt < kt_end ? kt : kt_safe;
 #pragma unroll
@@ -421,6 +467,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   __builtin_amdgcn_sched_barrier(0);
   for (int kt = kt_begin; kt < kt_end; kt += 2) {
     tile(w0, w1, kt, kt + 1);
+    if (kt + 1 >= kt_end) break;  // odd slice: what was prefetched for the missing tile is zeros
     tile(w1, w0, kt + 1, kt + 2);
   }
 
@@ -440,14 +487,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       else red1[((q - kFirst) * kWaves + wave) * 64 + lane] = acc[i][mt];
     }
   __syncthreads();
-  uint16_t* out = static_cast<uint16_t*>(p.out);
   for (int q = wave; q < kTiles; q += kWaves) {
     const int i = q / MT, mt = q - i * MT;
     const f32x4* src = q < kFirst ? red0 + q * kWaves * 64 : red1 + (q - kFirst) * kWaves * 64;
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ww = 0; ww < kWaves; ++ww) sum += src[ww * 64 + lane];
-    if (i < count) epi_store_acc<T>(p.epi, out, sum, 16 * mt + 4 * j, (nt_begin + i) * 16 + c, p.M, p.N, true);
+    if (i < count) astream_finish_tile<T, MT>(p, sum, nt_begin + i, mt, lane);
   }
 }
 
@@ -490,13 +536,14 @@ void launch(int mt, int cnt, bool lds, const AstreamArgs& a, dim3 grid, hipStrea
 
 template <typename T, int GPT>
 void plan_and_launch(int mt, int cus, const AstreamArgs& a, hipStream_t s) {
-  // column tiles per workgroup: one workgroup per CU if that needs no more than fit, else the split into whole
-  // rounds of workgroups that wastes least
+  // column tiles per workgroup: one workgroup per CU (per CU and split) if that needs no more than fit, else the
+  // split into whole rounds of workgroups that wastes least
+  const int wgs = cus / a.ksplit > 0 ? cus / a.ksplit : 1;
   auto plan = [&](int cnt_max) {
-    int cnt = (a.ntiles + cus - 1) / cus;
+    int cnt = (a.ntiles + wgs - 1) / wgs;
     if (cnt > cnt_max) {
-      const int rounds = (a.ntiles + cnt_max * cus - 1) / (cnt_max * cus);
-      cnt = (a.ntiles + rounds * cus - 1) / (rounds * cus);
+      const int rounds = (a.ntiles + cnt_max * wgs - 1) / (cnt_max * wgs);
+      cnt = (a.ntiles + rounds * wgs - 1) / (rounds * wgs);
     }
     if (const char* e = tuning_env("KSQ_W4_ASTREAM_CNT")) {  // tuning / test override
       const int v = atoi(e);
@@ -512,7 +559,7 @@ void plan_and_launch(int mt, int cus, const AstreamArgs& a, hipStream_t s) {
   bool lds = cnt >= 3;
   if (const char* e = tuning_env("KSQ_W4_ASTREAM_LDS")) lds = atoi(e) != 0;  // tuning / test override
   if (!lds) cnt = plan(cnt_max_of<T, GPT>(mt, false));
-  launch<T, GPT>(mt, cnt, lds, a, dim3((unsigned)((a.ntiles + cnt - 1) / cnt)), s);
+  launch<T, GPT>(mt, cnt, lds, a, dim3((unsigned)((a.ntiles + cnt - 1) / cnt), (unsigned)a.ksplit), s);
 }
 
 }  // namespace
@@ -521,9 +568,30 @@ bool w4a16_astream_supported(size_t m, size_t n, size_t k) {
   return m >= 17 && m <= 64 && m * k * 2 < 0x7FFFFF00ull && 4 * (k / kTileK) * 1024 < 0x7FFFFF00ull && n / kTileN < (1u << 30);
 }
 
-int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, int cus, hipStream_t s,
-                         const Epilogue& epi) {
+// K is split in two over workgroups while the column tiles alone give a compute unit at most two of them and the
+// kernel is long enough for the hand-over through memory (about 3 us) to pay: always with four row tiles, from 80 k
+// tiles on with two (measured on the o and down projections of Llama-2 7B and 70B: 3 to 29 % faster, four splits
+// never better than two).  The element type plays no part, so the workspace can be sized without it.
+AstreamPlan w4a16_astream_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  AstreamPlan p{};
+  p.mt = m <= 32 ? 2 : 4;
+  const size_t ntiles = n / kTileN, kt = k / kTileK;
+  size_t ks = (ntiles <= 2 * (size_t)cus && kt >= 16 && (p.mt == 4 || kt >= 80)) ? 2 : 1;
+  if (const char* e = tuning_env("KSQ_W4_ASTREAM_KSPLIT")) {  // tuning / test override
+    const size_t v = (size_t)atoi(e);
+    if (v >= 1 && v <= 8 && v <= kt) ks = v;
+  }
+  if (ntiles * p.mt > (size_t)kCountersPerSlot) ks = 1;
+  auto need = [&](size_t x) { return x <= 1 ? (size_t)0 : x * ntiles * p.mt * 64 * 16; };
+  while (ks > 1 && need(ks) > workspace_bytes) --ks;
+  p.ksplit = (int)ks;
+  p.partial_bytes = need(ks);
+  return p;
+}
+
+int w4a16_launch_astream(int dtype, const AstreamPlan& plan, void* out, const void* act, const void* weight,
+                         const void* sz, size_t m, size_t n, size_t k, size_t g, int cus, void* workspace,
+                         hipStream_t s, const Epilogue& epi) {
   AstreamArgs a{};
   a.epi = epi;
   a.weight = weight;
@@ -536,7 +604,15 @@ int w4a16_launch_astream(int dtype, void* out, const void* act, const void* weig
   a.KT = (int)(k / kTileK);
   a.G = (int)(k / g);
   a.ntiles = (int)(n / kTileN);
-  const int mt = m <= 32 ? 2 : 4;
+  a.ksplit = plan.ksplit;
+  a.partial = static_cast<f32x4*>(workspace);
+  a.counters = nullptr;
+  if (plan.ksplit > 1) {
+    KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
+    a.counters = counter_slot_device_ptr();
+    if (!a.counters) return KSQ_ERR_HIP;
+  }
+  const int mt = plan.mt;
   const int gpt = (int)(kTileK / g);
   if (dtype == KSQ_F16) {
     if (gpt == 1) plan_and_launch<_Float16, 1>(mt, cus, a, s);

@@ -199,6 +199,30 @@ def test_accumulator_stationary_route(gpu, lds, cnt, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("lds", [0, 1])
+@pytest.mark.parametrize("ksplit", [2, 3, 4])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 17, 640, 528),      # five k tiles: splits of one and two tiles, most waves idle
+    ("bf16", "awq", 128, 32, 1152, 272),
+    ("f16", "gptq", 64, 64, 2048, 1040),
+    ("bf16", "gptq", 64, 48, 4096, 272),    # splits of eight to eleven k tiles: odd and even slices per wave
+])
+def test_accumulator_stationary_split_k(gpu, lds, ksplit, dtype, kind, g, M, K, N):
+    """The same kernel with K split over workgroups as well (partial tiles through the workspace, summed in split
+    order by the last workgroup to arrive): parity, bit-identical repeats (the arrival counters return to zero), and
+    the fall-back to one split when the caller gives no workspace."""
+    case = W4Case(1340 + ksplit + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    with _env(KSQ_W4_ASTREAM=1, KSQ_W4_ASTREAM_LDS=lds, KSQ_W4_ASTREAM_KSPLIT=ksplit):
+        dev = W4Device(case, gpu)   # sizes the workspace for the split
+        assert dev.workspace_bytes >= ksplit * (N // 16) * (2 if M <= 32 else 4) * 1024
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+        got3 = dev.gemm_f32(use_workspace=False)
+    orc.assert_parity(got1, case.oracle(), f"astream ksplit={ksplit} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+    orc.assert_parity(got3, case.oracle(), f"astream no workspace {dtype} {kind} g={g} M={M}")
+
+
 def test_prefill_bf16_row_magnitudes(gpu):
     """bf16 activations go through a per-row power-of-two re-encoding on the large-M route: rows of very different
     magnitude (up to 2^100, down to 2^-60, an all-zero row) must each keep full relative accuracy."""
