@@ -369,10 +369,10 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
   a.KS = (int)(k / 128);
   a.a_scale_per_row = act_scale_count > 1;
   a.w_scale_per_col = w_scale_count > 1;
-  // 256 x 256 tiles (one workgroup per CU) when they still cover every CU, else 128 x 256 (two per CU)
-  const DeviceInfo* di = device_info();
-  KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
-  int tile = ((m + 255) / 256) * ((n + 255) / 256) >= (size_t)di->cus ? 256 : 128;
+  // 256 x 256 tiles (one workgroup of eight waves per CU) whenever there is more than one 128-row block: measured
+  // on the Qwen-72B shapes that kernel sustains 1.7 times the rate of the 128 x 256 one and is up to twice as fast
+  // even where its workgroups cover a third of the CUs; never more than 13 % slower.
+  int tile = m > 128 ? 256 : 128;
   if (const char* e = tuning_env("KSQ_FP8_PREFILL_TILE")) {  // tuning / test override
     const int v = atoi(e);
     if (v == 128 || v == 256) tile = v;
