@@ -222,8 +222,15 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
       if (ap.partial_bytes > best) best = ap.partial_bytes;
     }
   }
-  if (max_m >= 65) {  // the element type is not known here: size for the bf16 route of the prefill kernel
-    const size_t pf = w4a16_prefill_workspace_bytes(KSQ_BF16, max_m, k);
+  if (max_m >= 65) {
+    // the element type is not known here: size for the bf16 route of the prefill kernel, plus the largest set of
+    // split-K partial tiles any m up to max_m asks for (the plan depends on the number of 64-row blocks only)
+    size_t partial = 0;
+    for (size_t mb = 2; mb <= (max_m + 63) / 64 && mb <= 2 * (size_t)cus; ++mb) {
+      const PrefillPlan pp = w4a16_prefill_plan(mb * 64, n, k, cus, (size_t)-1);
+      if (pp.partial_bytes > partial) partial = pp.partial_bytes;
+    }
+    const size_t pf = w4a16_prefill_workspace_bytes(KSQ_BF16, max_m, k) + partial;
     if (pf > best) best = pf;
   }
   *bytes = best;
@@ -275,7 +282,7 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   epi.bias = bias;
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g) &&
       workspace_bytes >= w4a16_prefill_workspace_bytes(dtype, m, k))
-    return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, s, epi);
+    return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, workspace_bytes, s, epi);
   if (w4a16_astream_supported(m, n, k)) {
     // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
     // never slower than the k-stationary one.  With two it wins while every workgroup gets one to four column

@@ -120,9 +120,17 @@ W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes)
 int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
                         const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
                         const Epilogue& epi = Epilogue());
+struct PrefillPlan {
+  int rows;    // rows per workgroup tile: 64 or 128
+  int knt;     // 64-row kernel: column tiles per wave (1, 2 or 4)
+  int nw;      // 128-row kernel: waves per workgroup (4 or 8)
+  int ksplit;  // 64-row kernel: grid.y
+  size_t partial_bytes;
+};
+PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
 int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
-                        const Epilogue& epi = Epilogue());
+                         size_t n, size_t k, size_t g, void* workspace, size_t workspace_bytes, hipStream_t s,
+                         const Epilogue& epi = Epilogue());
 size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k);
 bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g);
 int w4a16_stream_max_slices(int mt, int nt);

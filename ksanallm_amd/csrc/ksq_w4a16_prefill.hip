@@ -38,6 +38,9 @@ struct PrefillArgs {
   void* out;
   const float* row_scale;  // bf16 route: 2^e per row of the re-encoded activations
   int M, N, K, KT, G, ntiles, mblocks, nblocks, super_n;
+  int ksplit;          // 64-row kernel only: grid.y
+  float* partial;      // [ksplit][mblocks * 64][N] fp32, ksplit > 1 only
+  unsigned* counters;  // [mblocks][nblocks][4 waves], zero between launches
   Epilogue epi;
 };
 
@@ -323,6 +326,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 // (four waves, every wave 4 x 4 MFMA tiles, two workgroups per CU) and, because such grids run one or two waves
 // per SIMD with nobody to hide a memory round trip behind, everything three k tiles ahead: activations global -> LDS
 // over four stages of 16 KiB (four separate objects), weights in a ring of four register tiles.
+// What bounds such a grid is the length of the k loop (a k tile takes most of a microsecond however little work it
+// carries), so while the output tiles alone leave workgroup slots empty and K is long K is split over grid.y: the fp32 partial tiles
+// go through the workspace and the last wave to arrive at its 64 x (16 KNT) tile adds them in split order
+// (deterministic) and stores the result.
 template <typename T, int GPT, int KNT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_mid_kernel(PrefillArgs p) {
   using O = Ops<_Float16>;
@@ -391,7 +398,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   // which the second is empty when a k tile is one group)
   auto load_item = [&](u32x4* buf, BTile& b, int kt, int q, int item) {
     if (item == 0) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (4 * wave + q) * 64), 16, a_off[q], kt * 256, 0, 0);
+      // the scalar offset is not range-checked: a prefetch past K re-reads the last k tile (nobody uses it)
+      const int kta = kt < p.KT ? kt : p.KT - 1;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (4 * wave + q) * 64), 16, a_off[q], kta * 256, 0, 0);
     } else if (q < KNT) {
       if (item == 1)
         b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
@@ -464,24 +473,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
     }
   };
 
-  load_tile(lds_a0, b0, 0);
-  load_tile(lds_a1, b1, 1);
-  load_tile(lds_a2, b2, 2);
+  // k tiles of this split
+  const int kt0 = (int)(((long)p.KT * blockIdx.y) / p.ksplit), kt1 = (int)(((long)p.KT * (blockIdx.y + 1)) / p.ksplit);
+  load_tile(lds_a0, b0, kt0);
+  load_tile(lds_a1, b1, kt0 + 1);
+  load_tile(lds_a2, b2, kt0 + 2);
   // Whole groups of four tiles run in the steady state: every step issues the loads of the tile three ahead, also
   // past K (weights then read as zero without touching memory, activations as bytes that nobody uses), so that the
   // number of loads in flight at a step's wait is always the same.  The remaining one to three tiles issue nothing.
-  int kt = 0;
-  for (; kt + 4 <= p.KT; kt += 4) {
+  int kt = kt0;
+  for (; kt + 4 <= kt1; kt += 4) {
     step(lds_a0, lds_a3, b0, b3, kt, std::true_type{});
     step(lds_a1, lds_a0, b1, b0, kt + 1, std::true_type{});
     step(lds_a2, lds_a1, b2, b1, kt + 2, std::true_type{});
     step(lds_a3, lds_a2, b3, b2, kt + 3, std::true_type{});
   }
-  if (kt < p.KT) {
+  if (kt < kt1) {
     step(lds_a0, lds_a3, b0, b3, kt, std::false_type{});
-    if (kt + 1 < p.KT) {
+    if (kt + 1 < kt1) {
       step(lds_a1, lds_a0, b1, b0, kt + 1, std::false_type{});
-      if (kt + 2 < p.KT) step(lds_a2, lds_a1, b2, b1, kt + 2, std::false_type{});
+      if (kt + 2 < kt1) step(lds_a2, lds_a1, b2, b1, kt + 2, std::false_type{});
     }
   }
 
@@ -505,13 +516,67 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
       const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
       float rs = 1.f;
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
+      const bool live = cc < 16 * KNT && row < p.M && col + 8 <= p.N;
+      if (p.ksplit > 1) {  // park the fp32 segment; finished below
+        if (live) {
+          f32x4* dst = reinterpret_cast<f32x4*>(p.partial + ((size_t)blockIdx.y * p.mblocks * 64 + row) * p.N + col);
+          store_agent(dst, f32x4{src[0], src[1], src[2], src[3]});
+          store_agent(dst + 1, f32x4{src[4], src[5], src[6], src[7]});
+        }
+        continue;
+      }
       float vals[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs;
-      if (cc < 16 * KNT && row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
+      if (live) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
+  if (p.ksplit == 1) return;
+
+  // ---- K split over workgroups: the last wave to arrive at this 64 x (16 KNT) tile adds the partials in split order
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  unsigned* counter = p.counters + ((size_t)mb * p.nblocks + nb) * 4 + wave;
+  unsigned arrived = 0;
+  if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  arrived = __builtin_amdgcn_readfirstlane(arrived);
+  if (arrived != (unsigned)(p.ksplit - 1)) return;
+  asm volatile("" ::: "memory");
+  if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const size_t split_stride = (size_t)p.mblocks * 64 * p.N / 4;  // in 16-byte units
+  // the loads of all splits of a row segment are independent: with the count a constant they go out together
+  auto reduce = [&](auto ks_tag) {
+    constexpr int KS = decltype(ks_tag)::value;
+#pragma unroll
+    for (int mt = 0; mt < kRows; ++mt) {
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+        const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
+        const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
+        if (!(cc < 16 * KNT && row < p.M && col + 8 <= p.N)) continue;
+        const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + (size_t)row * p.N + col);
+        f32x4 lo[KS], hi[KS];
+#pragma unroll
+        for (int sp = 0; sp < KS; ++sp) {
+          lo[sp] = load_agent(src + sp * split_stride);
+          hi[sp] = load_agent(src + sp * split_stride + 1);
+        }
+#pragma unroll
+        for (int sp = 1; sp < KS; ++sp) {
+          lo[0] += lo[sp];
+          hi[0] += hi[sp];
+        }
+        float rs = 1.f;
+        if constexpr (kBF16) rs = p.row_scale[row];
+        const float vals[8] = {lo[0][0] * rs, lo[0][1] * rs, lo[0][2] * rs, lo[0][3] * rs,
+                               hi[0][0] * rs, hi[0][1] * rs, hi[0][2] * rs, hi[0][3] * rs};
+        epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
+      }
+    }
+  };
+  if (p.ksplit == 2) reduce(std::integral_constant<int, 2>{});
+  else if (p.ksplit == 3) reduce(std::integral_constant<int, 3>{});
+  else reduce(std::integral_constant<int, 4>{});
 }
 
 template <typename T>
@@ -548,14 +613,70 @@ bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g) 
   return m >= min_m && n % 16 == 0 && m * k * 2 < 0x7FFFFF00ull && (k / kTileK) * 1024 < 0x7FFFFF00ull;
 }
 
-// bf16 route: fp16 copy of the activations + one float per row
+// bf16 route: fp16 copy of the activations + one float per row, in front of whatever else the plan needs
 size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k) {
   if (dtype != KSQ_BF16) return 0;
-  return (m * k * 2 + 255) / 256 * 256 + m * 4;
+  return ((m * k * 2 + 255) / 256 * 256 + m * 4 + 255) / 256 * 256;
+}
+
+// Tile shapes and the K split of the 64-row kernel; `workspace_bytes` is what remains behind the bf16 front part.
+PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  PrefillPlan p{};
+  const size_t ntiles = n / kTileN, kt = k / kTileK, mb128 = (m + 127) / 128;
+  // Row tile of the workgroup: 128 rows when such tiles (128 x 256) give every CU a workgroup and every weight tile
+  // is shared by four row blocks or more (that kernel prefetches weights one k tile ahead only, which covers an L2
+  // hit but not a trip to HBM); else 64 rows with deeper prefetch.
+  p.rows = (mb128 * ((ntiles + 15) / 16) >= (size_t)cus && mb128 >= 4) ? 128 : 64;
+  if (const char* e = tuning_env("KSQ_W4_PREFILL_ROWS")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v == 64 || v == 128) p.rows = v;
+  }
+  p.ksplit = 1;
+  if (p.rows == 64) {
+    const size_t mb = (m + 63) / 64;
+    auto wgs = [&](int knt) { return mb * ((ntiles + 4 * knt - 1) / (4 * knt)); };
+    // column tiles per wave (4, 2 or 1): the choice with the most workgroups that still run all at once, two per
+    // CU (measured on the Llama-2 7B and 70B shapes at M = 128 .. 512: within 11 % of the best everywhere); the
+    // widest tiles when even those need several rounds.
+    int knt = 4;
+    if (wgs(4) <= 2 * (size_t)cus) knt = wgs(2) <= 2 * (size_t)cus ? (wgs(1) <= 2 * (size_t)cus ? 1 : 2) : 4;
+    // K split in two: the fp32 partial tiles cost 2 x 2 x M x N x 4 bytes of traffic against K x N / 2 of weights,
+    // which pays only for long K and few rows (K >= 96 M: the 70B down projection up to M = 256, 11 to 17 % faster)
+    size_t ks = 1;
+    if (k >= 96 * mb * 64 && 2 * wgs(2) <= 2 * (size_t)cus && kt >= 16) {
+      ks = 2;
+      knt = 2;
+    }
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_KSPLIT")) {  // tuning / test override
+      const size_t v = (size_t)atoi(e);
+      if (v >= 1 && v <= 4 && v <= kt) ks = v;
+    }
+    auto need = [&](size_t x) { return x <= 1 ? (size_t)0 : x * mb * 64 * n * 4; };
+    while (ks > 1 && need(ks) > workspace_bytes) --ks;
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_NT")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 1 || v == 2 || v == 4) knt = v;
+    }
+    if (mb * ((ntiles + 4 * knt - 1) / (4 * knt)) * 4 > (size_t)kCountersPerSlot) ks = 1;
+    p.knt = knt;
+    p.ksplit = (int)ks;
+    p.partial_bytes = need(ks);
+  } else {
+    // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; measured at
+    // M = 4096 they win up to N = 8192 (fewer, fatter workgroups), four waves (128 x 256, two per CU) beyond.
+    // (and up to N = 12288 when they fill every CU at least twice: qkv of Llama-2-7B at M = 4096, +5 %)
+    const size_t wgs8 = mb128 * ((ntiles + 31) / 32);
+    p.nw = ((wgs8 >= (size_t)cus && ntiles <= 512) || (wgs8 >= 2 * (size_t)cus && ntiles <= 768)) ? 8 : 4;
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 4 || v == 8) p.nw = v;
+    }
+  }
+  return p;
 }
 
 int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
-                         size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
+                         size_t n, size_t k, size_t g, void* workspace, size_t workspace_bytes, hipStream_t s,
                          const Epilogue& epi) {
   KSQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && n % 8 == 0, KSQ_ERR_INVALID_ARGUMENT,
               "prefill output must be 16-byte aligned");
@@ -574,41 +695,32 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   a.ntiles = (int)(n / kTileN);
   const DeviceInfo* di = device_info();
   KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
-  // Row tile of the workgroup: 128 rows when such tiles (128 x 256) give every CU at least two workgroups, else 64
-  // rows with deeper prefetch.
-  int rows = ((m + 127) / 128) * ((size_t)(a.ntiles + 15) / 16) >= 2 * (size_t)di->cus ? 128 : 64;
-  if (const char* e = tuning_env("KSQ_W4_PREFILL_ROWS")) {  // tuning / test override
-    const int v = atoi(e);
-    if (v == 64 || v == 128) rows = v;
+  const size_t front = w4a16_prefill_workspace_bytes(dtype, m, k);
+  KSQ_REQUIRE(front == 0 || (workspace != nullptr && workspace_bytes >= front), KSQ_ERR_WORKSPACE,
+              "bf16 prefill needs its workspace");
+  const PrefillPlan plan = w4a16_prefill_plan(m, n, k, di->cus, workspace ? workspace_bytes - front : 0);
+  a.ksplit = plan.ksplit;
+  a.partial = nullptr;
+  a.counters = nullptr;
+  if (plan.ksplit > 1) {
+    a.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + front);
+    a.counters = counter_slot_device_ptr();
+    if (!a.counters) return KSQ_ERR_HIP;
   }
   int nw = 0;  // > 0: waves of the 128-row kernel; <= 0: minus the column tiles per wave of the 64-row kernel
   dim3 grid, block(256);
-  if (rows == 64) {
+  if (plan.rows == 64) {
     a.mblocks = (int)((m + 63) / 64);
-    // column tiles per wave: as many (4, 2, 1) as still give every CU two workgroups
-    int knt = 4;
-    while (knt > 1 && (size_t)a.mblocks * ((a.ntiles + 4 * knt - 1) / (4 * knt)) < 2 * (size_t)di->cus) knt >>= 1;
-    if (const char* e = tuning_env("KSQ_W4_PREFILL_NT")) {  // tuning / test override
-      const int v = atoi(e);
-      if (v == 1 || v == 2 || v == 4) knt = v;
-    }
+    const int knt = plan.knt;
     nw = -knt;
     a.nblocks = (a.ntiles + 4 * knt - 1) / (4 * knt);
     a.super_n = (a.nblocks + 7) / 8;
     const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
     KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
-    grid = dim3((unsigned)total);
+    grid = dim3((unsigned)total, (unsigned)plan.ksplit);
   } else {
     a.mblocks = (int)((m + kBM - 1) / kBM);
-    // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; measured at
-    // M = 4096 they win up to N = 8192 (fewer, fatter workgroups), four waves (128 x 256, two per CU) beyond.
-    // (and up to N = 12288 when they fill every CU at least twice: qkv of Llama-2-7B at M = 4096, +5 %)
-    const size_t wgs8 = (size_t)a.mblocks * ((a.ntiles + 31) / 32);
-    nw = ((wgs8 >= (size_t)di->cus && a.ntiles <= 512) || (wgs8 >= 2 * (size_t)di->cus && a.ntiles <= 768)) ? 8 : 4;
-    if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
-      const int v = atoi(e);
-      if (v == 4 || v == 8) nw = v;
-    }
+    nw = plan.nw;
     const int bnt = nw * kNT, sn = 32 / nw;
     a.nblocks = (a.ntiles + bnt - 1) / bnt;
     a.super_n = (a.nblocks + sn - 1) / sn;
@@ -621,7 +733,6 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   if (dtype == KSQ_F16) {
     launch_typed<_Float16>(a, gpt, nw, grid, block, s);
   } else {
-    KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "bf16 prefill needs its workspace");
     uint16_t* a16 = static_cast<uint16_t*>(workspace);
     float* row_scale = reinterpret_cast<float*>(static_cast<char*>(workspace) + (m * k * 2 + 255) / 256 * 256);
     const uint16_t* a_in = static_cast<const uint16_t*>(act);

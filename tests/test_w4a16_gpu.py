@@ -174,6 +174,36 @@ def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("ksplit", [2, 3, 4])
+@pytest.mark.parametrize("nt", [1, 4])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 65, 1152, 528),     # nine k tiles: splits of one to five tiles, ragged rows and columns
+    ("bf16", "awq", 128, 200, 2048, 272),
+    ("f16", "gptq", 64, 130, 4096, 512),    # whole groups of four tiles per split (the steady-state loop)
+    ("bf16", "gptq", 64, 512, 1024, 256),
+])
+def test_prefill_split_k(gpu, ksplit, nt, dtype, kind, g, M, K, N):
+    """The 64-row large-M kernel with K split over workgroups (fp32 partial tiles through the workspace, summed in split
+    order by the last wave to arrive): parity, bit-identical repeats (the arrival counters return to zero), and the
+    fall-back to one split when the workspace holds nothing beyond the bf16 front part."""
+    from ksanallm_amd import capi
+
+    case = W4Case(1280 + ksplit + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    with _env(KSQ_W4_PREFILL_ROWS=64, KSQ_W4_PREFILL_NT=nt, KSQ_W4_PREFILL_KSPLIT=ksplit):
+        dev = W4Device(case, gpu)   # sizes the workspace for the split
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+    with _env(KSQ_W4_PREFILL_ROWS=64, KSQ_W4_PREFILL_NT=nt, KSQ_W4_PREFILL_KSPLIT=1):
+        front = capi.w4a16_workspace_bytes(M, N, K)
+    assert dev.workspace_bytes > front
+    dev.workspace_bytes = front
+    with _env(KSQ_W4_PREFILL_ROWS=64, KSQ_W4_PREFILL_NT=nt, KSQ_W4_PREFILL_KSPLIT=ksplit):
+        got3 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"prefill ksplit={ksplit} nt={nt} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+    orc.assert_parity(got3, case.oracle(), f"prefill one split {dtype} {kind} g={g} M={M}")
+
+
 @pytest.mark.parametrize("lds", [0, 1])
 @pytest.mark.parametrize("cnt", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
