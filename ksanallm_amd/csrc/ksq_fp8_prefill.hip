@@ -108,11 +108,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
   };
   BStage b0, b1;
 
-  // item i < 4: activation fragment 4 * wave + i of stage s -> buf (past K: inside the buffer or out of range, never
-  // used either way)
+  // item i < 4: activation fragment 4 * wave + i of stage s -> buf.  The scalar offset is not range-checked: a
+  // prefetch past K re-reads the last stage (nobody uses it).
   auto load_a_item = [&](u32x4* buf, int s, int i) {
+    const int sc = s < p.KS ? s : p.KS - 1;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (4 * wave + i) * 64), 16, a_off[i >> 1],
-                                             s * 128 + (i & 1) * 64, 0, 0);
+                                             sc * 128 + (i & 1) * 64, 0, 0);
   };
   // item i < 8: weight piece (column tile i >> 1, half i & 1) of stage s; a stage past K is never used
   auto load_b_item = [&](BStage& b, int s, int i) {
@@ -269,10 +270,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   // item i < 8 of a stage's loads: i < 4 activations, else weights
   auto load_item = [&](u32x4* abuf, u32x4* bbuf, int s, int i) {
     const int f = i & 3;
+    const int sc = s < p.KS ? s : p.KS - 1;  // the scalar offset is not range-checked: past K, the last stage again
     if (i < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], s * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sc * 128, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], s * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], sc * 128, 0, 0);
   };
   auto read_frag = [&](const u32x4* buf, int tile) {
     return join(buf[tile * 128 + f_lane], buf[tile * 128 + 32 + f_lane]);

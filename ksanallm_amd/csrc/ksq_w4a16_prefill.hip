@@ -216,8 +216,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     if (item < 2) {
       if (item < kFPW / 4) {
         const int i = kFPW / 4 * q + item;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i], kt * 256,
-                                                 0, 0);
+        // the scalar offset is not range-checked: a prefetch past K re-reads the last k tile (nobody uses it)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i],
+                                                 (kt < p.KT ? kt : p.KT - 1) * 256, 0, 0);
       }
     } else if (item == 2) {
       b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
