@@ -171,7 +171,7 @@ int ksq_permute_columns(void* out, const void* in, const int32_t* perm, size_t m
  *   out[m,n] = T( sum_k act[m,k] * s[k/g,n] * (u[k,n] - z[k/g,n]) ),  fp32 accumulation.
  * act is [m,k] row-major T, out is [m,n] row-major T, weight / sz come from ksq_w4a16_repack.
  * The workspace (256-byte aligned, ksq_w4a16_workspace_bytes) holds split-K partial sums and, for bf16
- * activations at m >= 128, the fp16 re-encoding of the activations.  With workspace == NULL, misaligned or too
+ * activations at m >= 65, the fp16 re-encoding of the activations.  With workspace == NULL, misaligned or too
  * small the call still succeeds on a slower route that needs none.  The workspace is scratch for the duration
  * of one call and holds no state between calls; calls that may overlap in time on one device need a workspace
  * each, and at most 16 split-K launches of this library may be in flight on one device at a time (they share
