@@ -253,6 +253,27 @@ def test_accumulator_stationary_split_k(gpu, lds, ksplit, dtype, kind, g, M, K, 
     orc.assert_parity(got3, case.oracle(), f"astream no workspace {dtype} {kind} g={g} M={M}")
 
 
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 40, 2304, 1040),     # 18 k tiles, 65 column tiles, four row tiles: K split in two by the planner
+    ("bf16", "gptq", 64, 24, 10240, 272),    # 80 k tiles with two row tiles: split
+    ("f16", "gptq", 128, 24, 2048, 4112),    # one column tile per CU and a bit: activations through registers
+    ("bf16", "awq", 128, 64, 1152, 16400),   # four tiles per workgroup: activations through LDS, bf16 with CNT = 4
+    ("f16", "awq", 128, 100, 12288, 528),    # M >= 65, K >= 96 M: the 64-row kernel with K split in two
+    ("bf16", "gptq", 128, 128, 12288, 272),
+])
+def test_planner_choices_without_overrides(gpu, dtype, kind, g, M, K, N):
+    """Shapes picked so that the launch planners, left alone, take the split-K and LDS forms of the kernels for
+    17 <= M <= 64 and the split-K form of the 64-row large-M kernel; twice, bit for bit, and without a workspace."""
+    case = W4Case(1400 + M + N, M, K, N, g=g, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    got1 = dev.gemm_f32()
+    got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"planner {dtype} {kind} g={g} M={M} K={K} N={N}")
+    assert np.array_equal(got1, got2)
+    if not (dtype == "bf16" and M >= 65):  # the bf16 large-M route needs its workspace and falls back to a slower kernel
+        orc.assert_parity(dev.gemm_f32(use_workspace=False), case.oracle(), f"planner, no workspace {dtype} M={M}")
+
+
 def test_prefill_bf16_row_magnitudes(gpu):
     """bf16 activations go through a per-row power-of-two re-encoding on the large-M route: rows of very different
     magnitude (up to 2^100, down to 2^-60, an all-zero row) must each keep full relative accuracy."""
