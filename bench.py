@@ -177,11 +177,14 @@ def main():
     extra = {}
     if not args.no_extra:
         extra["per_shape"] = per_shape(torch, capi, layers, acts, outs, workspace, ws_bytes, stream, M, dtype)
-        if M != 64:
-            extra["decode_m64"] = per_shape(torch, capi, layers, {k: torch.randn((64, k), device=dev, generator=gen).to(
-                torch.float16) for k in (4096, 11008)}, {n: torch.empty((64, n), dtype=torch.float16, device=dev)
-                                                        for n in (12288, 4096, 22016)},
-                                            *workspace_for(torch, capi, dev, 64), stream, 64, dtype)
+        for m2 in (1, 4, 64):  # the other batch sizes of configs[1]
+            if m2 == M:
+                continue
+            extra[f"decode_m{m2}"] = per_shape(
+                torch, capi, layers,
+                {k: torch.randn((m2, k), device=dev, generator=gen).to(torch.float16) for k in (4096, 11008)},
+                {n: torch.empty((m2, n), dtype=torch.float16, device=dev) for n in (12288, 4096, 22016)},
+                *workspace_for(torch, capi, dev, m2), stream, m2, dtype)
         extra["fused_m16"] = fused(torch, capi, layers, acts, outs, stream, M, dtype, dev)
         extra["prefill_m4096"] = prefill(torch, capi, layers[0], dev, stream)
         extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], dev, stream, "f16")
