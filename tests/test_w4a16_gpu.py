@@ -336,6 +336,25 @@ def test_config2_awq_bf16_prefill_rows_subset(gpu, K, N):
     orc.assert_parity(got[rows], case.oracle(rows=rows), f"cfg2 K={K} N={N}")
 
 
+@pytest.mark.parametrize("K,N", [(8192, 8192), (28672, 8192)])
+def test_config3_gptq_70b_rows_subset(gpu, K, N):
+    """The o and down projections of Llama-2-70B (configs[3]) at M = 32, 64 and 256 through the product path: these
+    are the shapes where the planners split K over workgroups for 17 <= M <= 64 and (down, M = 256) in the 64-row
+    large-M kernel.  The oracle checks a seeded subset of rows."""
+    import torch
+
+    case = W4Case(3000 + K + N, 256, K, N, kind="gptq", dtype="f16")
+    dev = W4Device(case, gpu)
+    rows = np.unique(np.concatenate([[3, 20, 40, 60], np.random.default_rng(6).choice(256, size=8, replace=False)]))
+    want = case.oracle(rows=rows)
+    for M in (32, 64, 256):
+        sel = rows[rows < M]
+        got = dev.gemm(act=dev.act[:M].contiguous()).float().cpu().numpy()
+        orc.assert_parity(got[sel], want[: len(sel)], f"cfg3 K={K} N={N} M={M}")
+    del dev
+    torch.cuda.empty_cache()
+
+
 def test_linearity_at_full_size(gpu):
     """Size-independent property at a full 7B shape: f(a + b) = f(a) + f(b) when a, b and a + b are exactly
     representable and the fp16 results do not round differently (integer activations, unit scales)."""
