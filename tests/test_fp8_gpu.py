@@ -238,6 +238,28 @@ def test_gemm_small_integers_exact(gpu):
     assert np.array_equal(orc.to_bits(got, orc.F16), orc.to_bits(want.astype(np.float32), orc.F16))
 
 
+@pytest.mark.parametrize("wide", [0, 1])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 272), (5, 8208, 100), (16, 9600, 528), (9, 29568, 272)])
+def test_gemm_one_row_tile_both_workgroup_shapes(gpu, wide, M, K, N):
+    """M <= 16 with 16 waves x 4 stages and with 8 waves x 8 stages per workgroup (what the planner takes for K above
+    8192), including K that is split over workgroups and K that is not a multiple of 128; twice, bit for bit."""
+    import os
+
+    xq, xs, wq, ws = _fp8_case(440 + M, M, K, N)
+    old = os.environ.get("KSQ_FP8_WIDE")
+    os.environ["KSQ_FP8_WIDE"] = str(wide)
+    try:
+        got = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+        got2 = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+    finally:
+        if old is None:
+            os.environ.pop("KSQ_FP8_WIDE", None)
+        else:
+            os.environ["KSQ_FP8_WIDE"] = old
+    orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"fp8 wide={wide} M={M} K={K} N={N}")
+    assert np.array_equal(got, got2)
+
+
 @pytest.mark.parametrize("M", [1, 64])
 def test_config4_qwen72b_shape(gpu, M):
     xq, xs, wq, ws = _fp8_case(403, M, 8192, 8192)
