@@ -41,7 +41,8 @@ def test_graph_capture_and_replay(gpu):
     cases = [W4Case(3000, 16, 11008, 256, kind="awq", dtype="f16"),    # K beyond one workgroup: split over grid.y
              W4Case(3001, 40, 2048, 1024, kind="gptq", dtype="f16"),
              W4Case(3002, 200, 1024, 512, kind="awq", dtype="bf16"),
-             W4Case(3003, 24, 1024, 512, kind="gptq", dtype="bf16")]
+             W4Case(3003, 24, 1024, 512, kind="gptq", dtype="bf16"),
+             W4Case(3004, 100, 12288, 272, kind="awq", dtype="f16")]   # 64-row large-M kernel, K split in two
     devs = [W4Device(c, gpu) for c in cases]
     perm = torch.from_numpy(np.random.default_rng(3004).permutation(1024).astype(np.int32)).to(gpu)
     bias = torch.from_numpy(orc.to_bits(np.random.default_rng(3005).standard_normal(512).astype(np.float32),
