@@ -251,13 +251,15 @@ ROUTES = {
     "auto": {},
     "kstat": {"KSQ_W4_ASTREAM": 0},
     "astream": {"KSQ_W4_ASTREAM": 1},
+    "astream_splitk": {"KSQ_W4_ASTREAM": 1, "KSQ_W4_ASTREAM_KSPLIT": 2},
+    "astream_lds": {"KSQ_W4_ASTREAM": 1, "KSQ_W4_ASTREAM_LDS": 1, "KSQ_W4_ASTREAM_KSPLIT": 3},
     "stream": {"KSQ_W4_ASTREAM": 0, "KSQ_W4_KSTAT": 0, "KSQ_W4_FORCE_STREAM": 1},
     "stream_splitk": {"KSQ_W4_ASTREAM": 0, "KSQ_W4_KSTAT": 0, "KSQ_W4_FORCE_STREAM": 1, "KSQ_W4_KSPLIT": 3},
     "rows64": {"KSQ_W4_PREFILL_ROWS": 64, "KSQ_W4_PREFILL_KSPLIT": 1},
     "rows64_splitk": {"KSQ_W4_PREFILL_ROWS": 64, "KSQ_W4_PREFILL_KSPLIT": 3},
     "rows128": {"KSQ_W4_PREFILL_ROWS": 128},
 }
-EPI_CASES = [("auto", 1), ("auto", 16), ("kstat", 24), ("astream", 24), ("kstat", 64), ("astream", 64), ("stream", 9),
+EPI_CASES = [("auto", 1), ("auto", 16), ("kstat", 24), ("astream", 24), ("kstat", 64), ("astream", 64), ("astream_splitk", 24), ("astream_splitk", 64), ("astream_lds", 40), ("stream", 9),
              ("stream", 100), ("stream_splitk", 33), ("rows64", 100), ("rows64_splitk", 100), ("rows128", 200), ("auto", 300)]
 
 
