@@ -205,7 +205,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 
 
 // The same GEMM with a 256 x 256 workgroup tile: eight waves as 2 x 4, every wave 128 rows x 64 columns.  Both
-// operands go from global memory straight into LDS (one stage = 256 rows x 128 k of each = 64 KiB, two stages), so
+// operands go from global memory straight into LDS (one stage = 256 rows x 128 k of each = 32 KiB per operand; two
+// stages of activations, three of weights = all 160 KiB), so
 // each byte crosses the CU's vector memory path once per workgroup: 128 x 256 tiles need 46 B/clk per CU at the
 // matrix cores' FP8 rate, this one 32.  One workgroup per CU.
 template <typename T>
@@ -213,9 +214,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   constexpr int kHalf = 16 * 2 * 64;  // 16-byte elements of one operand of one stage (32 KiB)
   constexpr int kEpiStride = 68;
   __shared__ u32x4 lds_a0[kHalf];
-  __shared__ u32x4 lds_b0[kHalf];
   __shared__ u32x4 lds_a1[kHalf];
+  __shared__ u32x4 lds_b0[kHalf];
   __shared__ u32x4 lds_b1[kHalf];
+  __shared__ u32x4 lds_b2[kHalf];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -267,22 +269,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
     for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // item i < 8 of a stage's loads: i < 4 activations, else weights
-  auto load_item = [&](u32x4* abuf, u32x4* bbuf, int s, int i) {
+  // item i < 8 of a step's loads: i < 4 activations of stage sa, else weights of stage sb
+  auto load_item = [&](u32x4* abuf, u32x4* bbuf, int sa, int sb, int i) {
     const int f = i & 3;
-    const int sc = s < p.KS ? s : p.KS - 1;  // the scalar offset is not range-checked: past K, the last stage again
+    // the scalar offset is not range-checked: past K, the last stage again (nobody uses it)
+    const int sac = sa < p.KS ? sa : p.KS - 1, sbc = sb < p.KS ? sb : p.KS - 1;
     if (i < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sc * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sac * 128, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], sc * 128, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], sbc * 128, 0, 0);
   };
   auto read_frag = [&](const u32x4* buf, int tile) {
     return join(buf[tile * 128 + f_lane], buf[tile * 128 + 32 + f_lane]);
   };
 
-  auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt, int s) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of stage s has landed
-    __builtin_amdgcn_s_barrier();        // ... everyone's has, and everyone is done with the other stage
+  // One stage.  Weights (they come from HBM) are requested two stages ahead into a ring of three buffers, activations
+  // (mostly L2 hits: every row block is shared by all column blocks) one stage ahead into a ring of two.  Loads
+  // retire in order and a step issues its activation loads before its weight loads, so on entry everything but the
+  // four weight loads of the previous step (stage s + 1) has to have landed.
+  auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt2, int s) {
+    __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+    __builtin_amdgcn_s_barrier();        // ... everyone's share has landed, and everyone is done with the stage before
     __builtin_amdgcn_sched_barrier(0);
     i32x8 bf[kNT];
 #pragma unroll
@@ -293,9 +300,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       const i32x8 af = a_cur;
       a_cur = a_nxt;
       if (mt + 2 < kMT) a_nxt = read_frag(acur, 8 * wm + mt + 2);
-      if (mt < 4) {  // the next stage's loads go out in the first half, to have the second half to land
-        load_item(anxt, bnxt, s + 1, 2 * mt);
-        load_item(anxt, bnxt, s + 1, 2 * mt + 1);
+      if (mt < 4) {  // the loads go out in the first half: activations first, then weights
+        load_item(anxt, bnxt2, s + 1, s + 2, mt < 2 ? 2 * mt : 4 + 2 * (mt - 2));
+        load_item(anxt, bnxt2, s + 1, s + 2, mt < 2 ? 2 * mt + 1 : 4 + 2 * (mt - 2) + 1);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -306,13 +313,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   };
 
 #pragma unroll
-  for (int i = 0; i < 8; ++i) load_item(lds_a0, lds_b0, 0, i);
+  for (int i = 0; i < 4; ++i) load_item(lds_a0, lds_b0, 0, 0, i);
+#pragma unroll
+  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b0, 0, 0, i);
+#pragma unroll
+  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b1, 0, 1, i);
   int s = 0;
-  for (; s + 2 <= p.KS; s += 2) {
-    step(lds_a0, lds_b0, lds_a1, lds_b1, s);
+  for (; s + 6 <= p.KS; s += 6) {
+    step(lds_a0, lds_b0, lds_a1, lds_b2, s);
     step(lds_a1, lds_b1, lds_a0, lds_b0, s + 1);
+    step(lds_a0, lds_b2, lds_a1, lds_b1, s + 2);
+    step(lds_a1, lds_b0, lds_a0, lds_b2, s + 3);
+    step(lds_a0, lds_b1, lds_a1, lds_b0, s + 4);
+    step(lds_a1, lds_b2, lds_a0, lds_b1, s + 5);
   }
-  if (s < p.KS) step(lds_a0, lds_b0, lds_a1, lds_b1, s);
+  // the remaining zero to five stages, same rotation (their prefetches past K re-read the last stage)
+  if (s < p.KS) step(lds_a0, lds_b0, lds_a1, lds_b2, s);
+  if (s + 1 < p.KS) step(lds_a1, lds_b1, lds_a0, lds_b0, s + 1);
+  if (s + 2 < p.KS) step(lds_a0, lds_b2, lds_a1, lds_b1, s + 2);
+  if (s + 3 < p.KS) step(lds_a1, lds_b0, lds_a0, lds_b2, s + 3);
+  if (s + 4 < p.KS) step(lds_a0, lds_b1, lds_a1, lds_b0, s + 4);
 
   // ---- epilogue: scales, then a transpose through LDS so that every lane stores 16 contiguous bytes
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
