@@ -40,7 +40,6 @@ struct PrefillArgs {
   int M, N, K, KT, G, ntiles, mblocks, nblocks, super_n;
   int ksplit;          // 64-row kernel only: grid.y
   float* partial;      // [ksplit][mblocks * 64][N] fp32, ksplit > 1 only
-  unsigned* counters;  // [mblocks][nblocks][4 waves], zero between launches
   Epilogue epi;
 };
 
@@ -328,9 +327,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 // per SIMD with nobody to hide a memory round trip behind, everything three k tiles ahead: activations global -> LDS
 // over four stages of 16 KiB (four separate objects), weights in a ring of four register tiles.
 // What bounds such a grid is the length of the k loop (a k tile takes most of a microsecond however little work it
-// carries), so while the output tiles alone leave workgroup slots empty and K is long K is split over grid.y: the fp32 partial tiles
-// go through the workspace and the last wave to arrive at its 64 x (16 KNT) tile adds them in split order
-// (deterministic) and stores the result.
+// carries), so while the output tiles alone leave workgroup slots empty K is split over grid.y: every split stores
+// its fp32 partial tile into the workspace with plain stores and a second, ordinary kernel adds the splits in order
+// (deterministic) and applies the epilogue.  Tens of megabytes of partial tiles through the agent-scope atomics that
+// the decode kernels hand their few partial tiles over with were measured several times slower than the GEMM itself.
 template <typename T, int GPT, int KNT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_mid_kernel(PrefillArgs p) {
   using O = Ops<_Float16>;
@@ -518,11 +518,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
       float rs = 1.f;
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
       const bool live = cc < 16 * KNT && row < p.M && col + 8 <= p.N;
-      if (p.ksplit > 1) {  // park the fp32 segment; finished below
+      if (p.ksplit > 1) {  // the fp32 segment of this split; the reduction kernel finishes it
         if (live) {
           f32x4* dst = reinterpret_cast<f32x4*>(p.partial + ((size_t)blockIdx.y * p.mblocks * 64 + row) * p.N + col);
-          store_agent(dst, f32x4{src[0], src[1], src[2], src[3]});
-          store_agent(dst + 1, f32x4{src[4], src[5], src[6], src[7]});
+          dst[0] = f32x4{src[0], src[1], src[2], src[3]};
+          dst[1] = f32x4{src[4], src[5], src[6], src[7]};
         }
         continue;
       }
@@ -533,51 +533,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
-  if (p.ksplit == 1) return;
+}
 
-  // ---- K split over workgroups: the last wave to arrive at this 64 x (16 KNT) tile adds the partials in split order
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  unsigned* counter = p.counters + ((size_t)mb * p.nblocks + nb) * 4 + wave;
-  unsigned arrived = 0;
-  if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  arrived = __builtin_amdgcn_readfirstlane(arrived);
-  if (arrived != (unsigned)(p.ksplit - 1)) return;
-  asm volatile("" ::: "memory");
-  if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const size_t split_stride = (size_t)p.mblocks * 64 * p.N / 4;  // in 16-byte units
-  // the loads of all splits of a row segment are independent: with the count a constant they go out together
-  auto reduce = [&](auto ks_tag) {
-    constexpr int KS = decltype(ks_tag)::value;
-#pragma unroll
-    for (int mt = 0; mt < kRows; ++mt) {
-#pragma unroll
-      for (int pass = 0; pass < 2; ++pass) {
-        const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
-        const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
-        if (!(cc < 16 * KNT && row < p.M && col + 8 <= p.N)) continue;
-        const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + (size_t)row * p.N + col);
-        f32x4 lo[KS], hi[KS];
-#pragma unroll
-        for (int sp = 0; sp < KS; ++sp) {
-          lo[sp] = load_agent(src + sp * split_stride);
-          hi[sp] = load_agent(src + sp * split_stride + 1);
-        }
-#pragma unroll
-        for (int sp = 1; sp < KS; ++sp) {
-          lo[0] += lo[sp];
-          hi[0] += hi[sp];
-        }
-        float rs = 1.f;
-        if constexpr (kBF16) rs = p.row_scale[row];
-        const float vals[8] = {lo[0][0] * rs, lo[0][1] * rs, lo[0][2] * rs, lo[0][3] * rs,
-                               hi[0][0] * rs, hi[0][1] * rs, hi[0][2] * rs, hi[0][3] * rs};
-        epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
-      }
-    }
-  };
-  if (p.ksplit == 2) reduce(std::integral_constant<int, 2>{});
-  else if (p.ksplit == 3) reduce(std::integral_constant<int, 3>{});
-  else reduce(std::integral_constant<int, 4>{});
+// Second half of a K split of the 64-row kernel: out[row, col .. col + 7] = epilogue(row factor x sum over the splits,
+// in split order), one thread per segment of eight columns.
+template <typename T>
+__global__ __launch_bounds__(256) void w4a16_splitk_reduce_kernel(const float* __restrict__ partial, size_t split_stride,
+                                                                  int ksplit, const float* __restrict__ row_scale,
+                                                                  uint16_t* out, int M, int N, Epilogue epi) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t segs = (size_t)N / 8;
+  const size_t row = idx / segs;
+  if (row >= (size_t)M) return;
+  const int col = (int)(idx - row * segs) * 8;
+  const f32x4* src = reinterpret_cast<const f32x4*>(partial + row * N + col);
+  f32x4 lo = src[0], hi = src[1];
+  for (int sp = 1; sp < ksplit; ++sp) {
+    lo += src[sp * (split_stride / 4)];
+    hi += src[sp * (split_stride / 4) + 1];
+  }
+  const float rs = row_scale ? row_scale[row] : 1.f;
+  const float vals[8] = {lo[0] * rs, lo[1] * rs, lo[2] * rs, lo[3] * rs, hi[0] * rs, hi[1] * rs, hi[2] * rs, hi[3] * rs};
+  epi_store_row8<T>(epi, out, vals, (int)row, col, N);
 }
 
 template <typename T>
@@ -641,24 +618,32 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     // widest tiles when even those need several rounds.
     int knt = 4;
     if (wgs(4) <= 2 * (size_t)cus) knt = wgs(2) <= 2 * (size_t)cus ? (wgs(1) <= 2 * (size_t)cus ? 1 : 2) : 4;
-    // K split in two: the fp32 partial tiles cost 2 x 2 x M x N x 4 bytes of traffic against K x N / 2 of weights,
-    // which pays only for long K and few rows (K >= 96 M: the 70B down projection up to M = 256, 11 to 17 % faster)
+    // K split over workgroups, with the widest tiles.  Those are bound by their own instruction stream (about a
+    // microsecond per k tile and workgroup), so a split pays where they leave CUs empty and K is long: from 64 k
+    // tiles on and fewer workgroups than CUs, as many splits as fill two workgroup slots per CU, at least twelve k
+    // tiles each, and the partial tiles (written and read once, about 4 TB/s) at most 40 % of the unsplit estimate
+    // of 0.7 us per k tile.  Measured at the Llama-2 shapes, M = 128 .. 512: 7B down 52 -> 31, 54 -> 38, 61 -> 57 us;
+    // 70B qkv 61 -> 46, 65 -> 55; 70B o 41 -> 39, 51 -> 47; 70B down 130 -> 100, 159 -> 125 us; K = 4096 never gains.
     size_t ks = 1;
-    if (k >= 96 * mb * 64 && 2 * wgs(2) <= 2 * (size_t)cus && kt >= 16) {
-      ks = 2;
-      knt = 2;
+    if (kt >= 64 && wgs(4) < (size_t)cus) {
+      ks = 2 * (size_t)cus / wgs(4);
+      if (ks > 8) ks = 8;
+      if (ks > kt / 12) ks = kt / 12;
+      auto traffic_us = [&](size_t c) { return 2.0 * (double)c * (double)(mb * 64) * (double)n * 4.0 / 4e6; };
+      while (ks > 1 && traffic_us(ks) > 0.4 * 0.7 * (double)kt) --ks;
+      if (ks < 1) ks = 1;
     }
     if (const char* e = tuning_env("KSQ_W4_PREFILL_KSPLIT")) {  // tuning / test override
       const size_t v = (size_t)atoi(e);
-      if (v >= 1 && v <= 4 && v <= kt) ks = v;
+      if (v >= 1 && v <= 8 && v <= kt) ks = v;
     }
     auto need = [&](size_t x) { return x <= 1 ? (size_t)0 : x * mb * 64 * n * 4; };
     while (ks > 1 && need(ks) > workspace_bytes) --ks;
+    if (ks > 1) knt = 4;
     if (const char* e = tuning_env("KSQ_W4_PREFILL_NT")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 1 || v == 2 || v == 4) knt = v;
     }
-    if (mb * ((ntiles + 4 * knt - 1) / (4 * knt)) * 4 > (size_t)kCountersPerSlot) ks = 1;
     p.knt = knt;
     p.ksplit = (int)ks;
     p.partial_bytes = need(ks);
@@ -701,13 +686,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
               "bf16 prefill needs its workspace");
   const PrefillPlan plan = w4a16_prefill_plan(m, n, k, di->cus, workspace ? workspace_bytes - front : 0);
   a.ksplit = plan.ksplit;
-  a.partial = nullptr;
-  a.counters = nullptr;
-  if (plan.ksplit > 1) {
-    a.partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + front);
-    a.counters = counter_slot_device_ptr();
-    if (!a.counters) return KSQ_ERR_HIP;
-  }
+  a.partial = plan.ksplit > 1 ? reinterpret_cast<float*>(static_cast<char*>(workspace) + front) : nullptr;
   int nw = 0;  // > 0: waves of the 128-row kernel; <= 0: minus the column tiles per wave of the 64-row kernel
   dim3 grid, block(256);
   if (plan.rows == 64) {
@@ -746,6 +725,17 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     a.act = a16;
     a.row_scale = row_scale;
     launch_typed<__bf16>(a, gpt, nw, grid, block, s);
+  }
+  if (plan.ksplit > 1) {  // add the splits up and store
+    const size_t stride = (size_t)a.mblocks * 64 * n;
+    const dim3 rgrid((unsigned)((m * (n / 8) + 255) / 256));
+    uint16_t* o = static_cast<uint16_t*>(out);
+    if (dtype == KSQ_F16)
+      hipLaunchKernelGGL(w4a16_splitk_reduce_kernel<_Float16>, rgrid, dim3(256), 0, s, a.partial, stride, plan.ksplit,
+                         a.row_scale, o, (int)m, (int)n, epi);
+    else
+      hipLaunchKernelGGL(w4a16_splitk_reduce_kernel<__bf16>, rgrid, dim3(256), 0, s, a.partial, stride, plan.ksplit,
+                         a.row_scale, o, (int)m, (int)n, epi);
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
