@@ -192,6 +192,21 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
                       size_t n, size_t k, size_t group_size, const int32_t* act_perm, int epilogue,
                       const void* bias, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ksq_w4a16_gemm for callers that cannot allocate device memory (code under HIP graph capture that owns no
+ * buffer, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * layers always receive a workspace from their factory.  The split-K partial tiles and, for bf16 activations at
+ * m >= 65, the re-encoded activations go to a file-scope device array of KSQ_STATIC_SCRATCH_BYTES inside the library
+ * (every GPU the library runs on holds its own copy until the process ends); the call allocates and frees nothing.
+ * A shape whose ksq_w4a16_workspace_bytes(m, n, k) exceeds KSQ_STATIC_SCRATCH_BYTES fails with KSQ_ERR_WORKSPACE
+ * (every shape of Llama-2-7B / Llama-3-70B width fits up to m = 64).  All calls on one GPU share the one array:
+ * calls that may overlap in time on one GPU (different streams, different threads) race; serialise them or use
+ * ksq_w4a16_gemm with a workspace each.  The result is bit-identical to ksq_w4a16_gemm given a workspace of
+ * ksq_w4a16_workspace_bytes(m, n, k) bytes.  The first call of the library on a device resolves the array's
+ * address: make one call (ksq_device_compute_units() will do) on every device before capturing a graph. */
+#define KSQ_STATIC_SCRATCH_BYTES (64u << 20)
+int ksq_w4a16_gemm_static_scratch(int dtype, void* out, const void* act, const void* weight, const void* sz,
+                                  size_t m, size_t n, size_t k, size_t group_size, void* stream);
+
 /* ------------------------------------------------------------------ FP8 e4m3 (OCP: bias 7, max 448, no inf)
  *
  * ksq_fp8_quantize replaces Fp8E4m3Quantize (KS/kernels/nvidia/kernel_wrapper.cpp:1015-1027) =

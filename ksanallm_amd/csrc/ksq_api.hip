@@ -21,6 +21,9 @@ int fail(int code, const char* fmt, ...) {
 
 // ---- per-device state -----------------------------------------------------------------------------------------
 static __device__ __align__(256) unsigned g_splitk_counters[kCounterSlots * kCountersPerSlot];
+// Scratch of ksq_w4a16_gemm_static_scratch: stands in for the caller's workspace.  In host code this name is only a
+// handle for hipGetSymbolAddress; the address kept per device below is what kernels and copies get.
+static __device__ __align__(256) unsigned char g_static_scratch[KSQ_STATIC_SCRATCH_BYTES];
 
 namespace {
 constexpr int kMaxDevices = 16;
@@ -29,6 +32,7 @@ struct PerDevice {
   bool ok = false;
   DeviceInfo info{};
   unsigned* counters = nullptr;
+  unsigned char* static_scratch = nullptr;
   std::atomic<unsigned> next_slot{0};
 };
 PerDevice g_dev[kMaxDevices];
@@ -47,10 +51,13 @@ PerDevice* current_device_state() {
     void* p = nullptr;
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_splitk_counters)) != hipSuccess || p == nullptr) return;
     pd->counters = static_cast<unsigned*>(p);
+    void* q = nullptr;
+    if (hipGetSymbolAddress(&q, HIP_SYMBOL(g_static_scratch)) != hipSuccess || q == nullptr) return;
+    pd->static_scratch = static_cast<unsigned char*>(q);
     pd->ok = true;
   });
   if (!pd->ok) {
-    fail(KSQ_ERR_HIP, "device %d: could not query properties or resolve the split-K counters", dev);
+    fail(KSQ_ERR_HIP, "device %d: could not query properties or resolve the library's device arrays", dev);
     return nullptr;
   }
   return pd;
@@ -67,6 +74,11 @@ unsigned* counter_slot_device_ptr() {
   if (!pd) return nullptr;
   unsigned slot = pd->next_slot.fetch_add(1, std::memory_order_relaxed) % kCounterSlots;
   return pd->counters + (size_t)slot * kCountersPerSlot;
+}
+
+static unsigned char* static_scratch_device_ptr() {
+  PerDevice* pd = current_device_state();
+  return pd ? pd->static_scratch : nullptr;
 }
 
 const char* tuning_env(const char* name) {
@@ -307,6 +319,24 @@ int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, co
                    size_t k, size_t g, void* workspace, size_t workspace_bytes, void* stream) {
   return ksq_w4a16_gemm_ex(dtype, out, act, weight, sz, m, n, k, g, nullptr, KSQ_EPILOGUE_NONE, nullptr, workspace,
                            workspace_bytes, stream);
+}
+
+int ksq_w4a16_gemm_static_scratch(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m,
+                                  size_t n, size_t k, size_t g, void* stream) {
+  if (m == 0) return KSQ_OK;
+  size_t need = 0;
+  int rc = ksq_w4a16_workspace_bytes(m, n, k, &need);
+  if (rc != KSQ_OK) return rc;
+  KSQ_REQUIRE(need <= (size_t)KSQ_STATIC_SCRATCH_BYTES, KSQ_ERR_WORKSPACE,
+              "m=%zu n=%zu k=%zu needs %zu bytes of scratch; the library's static scratch holds %zu: use "
+              "ksq_w4a16_gemm with a workspace of the caller's",
+              m, n, k, need, (size_t)KSQ_STATIC_SCRATCH_BYTES);
+  unsigned char* scratch = static_scratch_device_ptr();  // this device's copy of the array
+  if (!scratch) return KSQ_ERR_HIP;
+  // Nothing in the scratch has to start at zero: split-K partial tiles and the re-encoded activations are written
+  // in full before they are read, and the arrival counters live elsewhere and return to zero by themselves.
+  return ksq_w4a16_gemm_ex(dtype, out, act, weight, sz, m, n, k, g, nullptr, KSQ_EPILOGUE_NONE, nullptr, scratch,
+                           need, stream);
 }
 
 }  // extern "C"
