@@ -29,7 +29,7 @@ struct KstatArgs {
   void* out;           // [M][N] T
   f32x4* partial;      // [ksplit][ntiles][MT][64]
   unsigned* counters;  // [ntiles][MT]
-  int M, N, K, KT, G, ntiles, ksplit, nt_per_wg;
+  int M, N, K, KT, G, ntiles, ksplit, nt_per_wg, act_barrier;
   Epilogue epi;
 };
 
@@ -66,14 +66,24 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
       const_cast<char*>(sb), 0, any ? ((count - 1) * p.G + TPW * GPT) * 64 : 0, 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
-  unsigned w_off[TPW], sz_off[TPW];
+  unsigned w_off[TPW];
 #pragma unroll
-  for (int t = 0; t < TPW; ++t) {
-    const bool ok = kt0 + t < wg_end;
-    w_off[t] = ok ? t * 1024u + lane * 16u : 0x80000000u;
-    sz_off[t] = ok ? t * GPT * 64u + c * 4u : 0x80000000u;
-  }
+  for (int t = 0; t < TPW; ++t) w_off[t] = kt0 + t < wg_end ? t * 1024u + lane * 16u : 0x80000000u;
   const unsigned w_stride = (unsigned)p.KT * 1024u, sz_stride = (unsigned)p.G * 64u;
+  // The scale/zero words of one batch -- NB column tiles x the wave's TPW * GPT groups x 16 columns -- are fetched
+  // with one word per lane: the words of one column tile are contiguous (its groups follow each other), so SZR
+  // instructions cover the batch instead of one instruction per (column tile, group).  Flat word f = 64 r + lane
+  // belongs to column tile f / (16 GW), group (f / 16) % GW, column f % 16.  The memory pipeline takes about as long
+  // for a one-word-per-lane instruction as for a weight tile, so this matters.
+  constexpr int GW = TPW * GPT;                  // groups per column tile that this wave needs
+  constexpr int SZR = (NB * GW * 16 + 63) / 64;  // instructions per batch
+  unsigned sz_off[SZR];
+#pragma unroll
+  for (int r = 0; r < SZR; ++r) {
+    const int f = 64 * r + lane, i = f / (16 * GW), gq = (f >> 4) % GW;
+    const bool ok = i < NB && kt0 + gq / GPT < wg_end;
+    sz_off[r] = ok ? (unsigned)i * sz_stride + (unsigned)gq * 64u + (unsigned)c * 4u : 0x80000000u;
+  }
 
   // Activation fragments of this wave's k tiles: registers for the whole kernel.  They are loaded with lane l on
   // row l / 4, 16-byte piece l % 4 of a 32-k step, so that every aligned group of four lanes reads 64 contiguous
@@ -96,12 +106,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 
   u32x4 wq[D];
-  uint32_t szq[D][GPT];
+  uint32_t szraw[SZR];  // the next batch's words as loaded, one per lane
   auto fetch = [&](int slot, int i /* column tile inside the workgroup */, int t) {
     wq[slot] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_off[t] + i * w_stride, 0, 2));
+  };
+  auto fetch_sz = [&](int batch) {
 #pragma unroll
-    for (int gi = 0; gi < GPT; ++gi)
-      szq[slot][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, sz_off[t] + gi * 64u + i * sz_stride, 0, 0);
+    for (int r = 0; r < SZR; ++r)
+      szraw[r] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, sz_off[r] + (unsigned)(batch * NB) * sz_stride, 0, 0);
   };
 
   uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
@@ -110,6 +122,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   asm volatile("" : "+v"(c_hi));
   asm volatile("" : "+v"(m_hi));
 
+  __builtin_amdgcn_sched_barrier(0);
+  // With more than one batch per workgroup, every wave's activation loads are issued before any wave's weight
+  // loads: the memory pipeline of a compute unit returns data in the order of issue, so activations (cache hits)
+  // queued behind another wave's weight tiles (HBM) would hold their wave back by the whole first batch.
+  if (p.act_barrier) __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_sz(0);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int q = 0; q < D; ++q) {
@@ -131,7 +150,23 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 
   uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int sz_lane = c * 4;
   for (int b = 0; b < nbatches; ++b) {
+    // every lane takes the words of its column: word (i, gq) sits in lane 16 * (f / 16 % 4) + c of instruction f / 64
+    uint32_t szq[D][GPT];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int gi = 0; gi < GPT; ++gi) {
+          const int f16 = (i * TPW + t) * GPT + gi;  // flat word index / 16
+          szq[i * TPW + t][gi] =
+              (uint32_t)__builtin_amdgcn_ds_bpermute(sz_lane + 64 * (f16 & 3), (int)szraw[f16 >> 2]);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+    fetch_sz(b + 1);
+    __builtin_amdgcn_sched_barrier(0);
     f32x4 accb[NB][MT];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
@@ -355,6 +390,7 @@ int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* 
   a.ntiles = (int)(n / kTileN);
   a.ksplit = plan.ksplit;
   a.nt_per_wg = plan.nt_per_wg;
+  a.act_barrier = (plan.nt_per_wg + plan.nb - 1) / plan.nb >= 2 ? 1 : 0;
   a.counters = nullptr;
   if (plan.ksplit > 1) {
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
