@@ -176,7 +176,7 @@ struct ModelConfig {
   size_t max_scheduler_token_num = 4096;
 };
 
-// Just enough of BaseWeight for MatMulLayerFactory::AutoCreateLayer.
+// Just enough of BaseWeight for a caller that looks a weight tensor up by name, as KsanaLLM's layer factory does.
 class BaseWeight {
  public:
   virtual ~BaseWeight() {}

@@ -8,7 +8,6 @@
 #include "fp8_matmul_layer.h"
 #include "group_matmul_layer.h"
 #include "ksq.h"
-#include "matmul_layer_factory.h"
 
 namespace ksana_llm {
 
@@ -313,7 +312,5 @@ Status MergeFp8QkvScales(Tensor& qkv_weight, const Tensor& q_scale, const Tensor
 template class Fp8MatMulLayer<float16>;
 template class Fp8MatMulLayer<bfloat16>;
 
-template class MatMulLayerFactory<float16>;
-template class MatMulLayerFactory<bfloat16>;
 
 }  // namespace ksana_llm

@@ -1,5 +1,5 @@
-// Test driver of the C++ layer shims: builds the layers through MatMulLayerFactory exactly as CommonModel does
-// (AutoCreateLayer by weight name), runs Forward on the device and writes the result for the Python parity tests.
+// Test driver of the C++ layer shims: builds the layers by weight name through the test harness that stands in for
+// KsanaLLM's layer factory, runs Forward on the device and writes the result for the Python parity tests.
 //
 //   layer_driver w4a16 <dir> <f16|bf16> <m> <k> <n> <g> <gptq|awq> <gptq|awq|rowmajor> <none|awq|uint8|additive>
 //       reads <dir>/qweight.bin, qzeros.bin (unless none), scales.bin, act.bin; writes <dir>/out.bin
@@ -21,7 +21,7 @@
 #include <vector>
 
 #include "ksq.h"
-#include "matmul_layer_factory.h"
+#include "layer_harness.h"
 
 using namespace ksana_llm;
 
@@ -116,16 +116,15 @@ static int RunW4(int argc, char** argv) {
   cfg.head_num = 1;
   cfg.num_key_value_heads = 0;
   cfg.max_scheduler_token_num = m;
-  std::shared_ptr<Tensor> workspace;
-  MatMulLayerFactory<T> factory(workspace, cfg, 0, context);
+  LayerHarness<T> factory(cfg, context);
   auto holder = std::make_shared<OneWeight>();
   holder->t = weight;
-  auto layer = factory.AutoCreateLayer(holder, "model.layers.0.self_attn.query_key_value.weight", TYPE_I4_GROUP, dt, dt, {});
+  auto layer = factory.ForWeight(*holder, "model.layers.0.self_attn.query_key_value.weight", dt);
 
   Tensor bias;
   if (extra == "silu" || extra == "bias") {
     auto group = std::dynamic_pointer_cast<GroupMatMulLayer<T, TYPE_I4_GROUP>>(layer);
-    if (!group) throw std::runtime_error("factory did not build a GroupMatMulLayer");
+    if (!group) throw std::runtime_error("harness did not build a GroupMatMulLayer");
     if (extra == "bias") {
       bias = Upload(ReadFile(dir + "/bias.bin"), dt, {n});
       group->SetEpilogue(KSQ_EPILOGUE_BIAS, &bias);
@@ -164,11 +163,10 @@ static int RunFp8(int argc, char** argv) {
   }
   ModelConfig cfg;
   cfg.max_scheduler_token_num = m;
-  std::shared_ptr<Tensor> workspace;
-  MatMulLayerFactory<T> factory(workspace, cfg, 0, context);
+  LayerHarness<T> factory(cfg, context);
   auto holder = std::make_shared<OneWeight>();
   holder->t = wq;
-  auto layer = factory.AutoCreateLayer(holder, "model.layers.0.mlp.down_proj.weight", TYPE_FP8_E4M3, dt, dt, {});
+  auto layer = factory.ForWeight(*holder, "model.layers.0.mlp.down_proj.weight", dt);
   Tensor act = Upload(ReadFile(dir + "/act.bin"), dt, {m, k});
   Tensor out;
   CreateTensor(out, {m, n}, dt, 0, MEMORY_DEVICE);
@@ -213,11 +211,10 @@ static int RunFp8Load(int argc, char** argv) {
 
   ModelConfig cfg;
   cfg.max_scheduler_token_num = m;
-  std::shared_ptr<Tensor> workspace;
-  MatMulLayerFactory<T> factory(workspace, cfg, 0, context);
+  LayerHarness<T> factory(cfg, context);
   auto holder = std::make_shared<OneWeight>();
   holder->t = fused;
-  auto layer = factory.AutoCreateLayer(holder, "model.layers.0.self_attn.query_key_value.weight", TYPE_FP8_E4M3, dt, dt, {});
+  auto layer = factory.ForWeight(*holder, "model.layers.0.self_attn.query_key_value.weight", dt);
   Tensor act = Upload(ReadFile(dir + "/act.bin"), dt, {m, k});
   Tensor out;
   CreateTensor(out, {m, n}, dt, 0, MEMORY_DEVICE);
@@ -250,20 +247,19 @@ static int RunErrors() {
   ModelConfig cfg;
   cfg.is_quant = true;
   cfg.quant_config.method = QUANT_GPTQ;
-  std::shared_ptr<Tensor> workspace;
-  MatMulLayerFactory<float16> factory(workspace, cfg, 0, context);
+  LayerHarness<float16> factory(cfg, context);
   std::vector<std::any> good = {false, false, true, CUTLASS_BACKEND, size_t(16), size_t(256), size_t(256), size_t(128), true};
 
-  Expect("unregistered (weight,input,output,quant) key throws", true,
-         [&] { factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP32, TYPE_FP32, good, QUANT_GPTQ); });
+  Expect("activation type without a layer class throws", true,
+         [&] { factory.Make(TYPE_I4_GROUP, TYPE_FP32, good); });
   Expect("parameter pack in the wrong order throws", true, [&] {
     std::vector<std::any> bad = {size_t(16), false, true};
-    factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, bad, QUANT_GPTQ);
+    factory.Make(TYPE_I4_GROUP, TYPE_FP16, bad);
   });
   Expect("group size 32 is refused when the workspace is sized", true, [&] {
     std::vector<std::any> p = good;
     p[7] = size_t(32);
-    auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
+    auto l = factory.Make(TYPE_I4_GROUP, TYPE_FP16, p);
     Tensor a, w, s, o;
     CreateTensor(a, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
     CreateTensor(w, {256, 128}, TYPE_UINT8, 0, MEMORY_DEVICE);
@@ -276,12 +272,12 @@ static int RunErrors() {
   Expect("k not a multiple of 128 is refused", true, [&] {
     std::vector<std::any> p = good;
     p[6] = size_t(192);
-    factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
+    factory.Make(TYPE_I4_GROUP, TYPE_FP16, p);
   });
   Expect("desc_act weight without a bound perm throws at Forward", true, [&] {
     std::vector<std::any> p = good;
     p[1] = true;
-    auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, p, QUANT_GPTQ);
+    auto l = factory.Make(TYPE_I4_GROUP, TYPE_FP16, p);
     Tensor a, w, s, o;
     CreateTensor(a, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
     CreateTensor(w, {256, 128}, TYPE_UINT8, 0, MEMORY_DEVICE);
@@ -292,7 +288,7 @@ static int RunErrors() {
     l->Forward({a, w}, outs);
   });
   Expect("weight without bound scales throws", true, [&] {
-    auto l = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, good, QUANT_GPTQ);
+    auto l = factory.Make(TYPE_I4_GROUP, TYPE_FP16, good);
     Tensor a, w, o;
     CreateTensor(a, {1, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
     CreateTensor(w, {256, 128}, TYPE_UINT8, 0, MEMORY_DEVICE);
@@ -302,7 +298,7 @@ static int RunErrors() {
   });
   Expect("fp8: null weight scale throws", true, [&] {
     std::vector<std::any> p = {size_t(4), size_t(256)};
-    auto l = factory.CreateLayer(TYPE_FP8_E4M3, TYPE_FP16, TYPE_FP16, p, QUANT_FP8_E4M3);
+    auto l = factory.Make(TYPE_FP8_E4M3, TYPE_FP16, p);
     Tensor a, w, o;
     CreateTensor(a, {4, 256}, TYPE_FP16, 0, MEMORY_DEVICE);
     CreateTensor(w, {64, 256}, TYPE_FP8_E4M3, 0, MEMORY_DEVICE);
@@ -312,7 +308,7 @@ static int RunErrors() {
   });
   Expect("fp8: workspace smaller than the request throws", true, [&] {
     std::vector<std::any> p = {size_t(4), size_t(256)};
-    auto l = factory.CreateLayer(TYPE_FP8_E4M3, TYPE_FP16, TYPE_FP16, p, QUANT_FP8_E4M3);
+    auto l = factory.Make(TYPE_FP8_E4M3, TYPE_FP16, p);
     Tensor a, w, o, sc;
     CreateTensor(a, {64, 256}, TYPE_FP16, 0, MEMORY_DEVICE);  // m = 64 > max_m = 4
     CreateTensor(w, {64, 256}, TYPE_FP8_E4M3, 0, MEMORY_DEVICE);
@@ -323,12 +319,12 @@ static int RunErrors() {
     l->Forward({a, w}, outs);
   });
   Expect("well-formed group layer builds and shares one workspace", false, [&] {
-    auto l1 = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, good, QUANT_GPTQ);
+    auto l1 = factory.Make(TYPE_I4_GROUP, TYPE_FP16, good);
     std::vector<std::any> big = good;
     big[5] = size_t(4096);
     big[6] = size_t(4096);
-    auto l2 = factory.CreateLayer(TYPE_I4_GROUP, TYPE_FP16, TYPE_FP16, big, QUANT_AWQ);
-    if (!factory.GetWorkSpaceBuffer() || factory.GetWorkSpaceBuffer()->GetTotalBytes() < l2->GetWorkSpaceSize())
+    auto l2 = factory.Make(TYPE_I4_GROUP, TYPE_FP16, big);
+    if (!factory.Workspace() || factory.Workspace()->GetTotalBytes() < l2->GetWorkSpaceSize())
       throw std::runtime_error("shared workspace was not grown to the largest request");
   });
   return 0;

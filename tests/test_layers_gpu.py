@@ -1,4 +1,4 @@
-"""The C++ layer shims (GroupMatMulLayer / Fp8MatMulLayer built through MatMulLayerFactory::AutoCreateLayer, with
+"""The C++ layer shims (GroupMatMulLayer / Fp8MatMulLayer built by weight name through the test harness that stands in for KsanaLLM's layer factory, with
 the reference's Init / Forward(input_tensors, output_tensors) interface) against the CPU oracle, through the test
 driver tests/cpp/layer_driver.cpp.  Also their error conventions (misuse throws std::runtime_error)."""
 import os
