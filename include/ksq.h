@@ -127,7 +127,8 @@ int ksq_device_compute_units(void);
  *            owns column n = 16*nt + c; 32-bit word d (0..3) of the lane covers k = 128*kt + 32*d + 8*j + e,
  *            e = 0..7, with element e in nibble e/2 when e is even and nibble 4 + e/2 when e is odd; nibbles are
  *            the unsigned u in [0,15].  One 128-bit load per lane is the B operand of four 16x16x32 MFMAs.
- *   sz     : (K/g)*N 32-bit words = [N/16][K/g][16]; word = scale bits (T) | z << 16 with z in [0,15]. */
+ *   sz     : (K/g)*N 32-bit words = [N/16][K/g][16]; word = scale bits (T) | z << 16 with z in [0,15]
+ *            | E << 24, E (int8) = the largest binary exponent among the column's scales when they are bf16, else 0. */
 int ksq_w4a16_repack_sizes(size_t k, size_t n, size_t group_size, size_t* weight_bytes, size_t* sz_bytes);
 
 int ksq_w4a16_repack(int src_layout, const void* qweight, int zero_kind, const void* zeros, const void* scales,
@@ -174,8 +175,10 @@ int ksq_permute_columns(void* out, const void* in, const int32_t* perm, size_t m
  * activations at m >= 65, the fp16 re-encoding of the activations.  With workspace == NULL, misaligned or too
  * small the call still succeeds on a slower route that needs none.  The workspace is scratch for the duration
  * of one call and holds no state between calls; calls that may overlap in time on one device need a workspace
- * each, and at most 16 split-K launches of this library may be in flight on one device at a time (they share
- * 16 rotating sets of arrival counters in library-owned device memory). */
+ * each.  The arrival counters of the split-K kernels are library-owned device memory, one region per stream (the
+ * first 64 streams per device that launch a split-K kernel; later streams get the same results without split-K):
+ * launches on one stream never overlap, so no launch shares counters with one in flight -- with one exception:
+ * two HIP graphs captured from the same stream and replayed at the same time on different streams would. */
 int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
 
 int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,

@@ -33,7 +33,9 @@ struct PerDevice {
   DeviceInfo info{};
   unsigned* counters = nullptr;
   unsigned char* static_scratch = nullptr;
-  std::atomic<unsigned> next_slot{0};
+  std::mutex slot_mutex;
+  int slots_used = 0;
+  hipStream_t slot_owner[kCounterSlots] = {};
 };
 PerDevice g_dev[kMaxDevices];
 
@@ -69,10 +71,16 @@ const DeviceInfo* device_info() {
   return pd ? &pd->info : nullptr;
 }
 
-unsigned* counter_slot_device_ptr() {
+unsigned* counter_slot_device_ptr(hipStream_t stream) {
   PerDevice* pd = current_device_state();
   if (!pd) return nullptr;
-  unsigned slot = pd->next_slot.fetch_add(1, std::memory_order_relaxed) % kCounterSlots;
+  std::lock_guard<std::mutex> lock(pd->slot_mutex);
+  int slot = 0;
+  while (slot < pd->slots_used && pd->slot_owner[slot] != stream) ++slot;
+  if (slot == pd->slots_used) {
+    if (slot == kCounterSlots) return nullptr;  // every region has an owner: this stream runs without split-K
+    pd->slot_owner[pd->slots_used++] = stream;
+  }
   return pd->counters + (size_t)slot * kCountersPerSlot;
 }
 
@@ -295,6 +303,9 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g) &&
       workspace_bytes >= w4a16_prefill_workspace_bytes(dtype, m, k))
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, workspace_bytes, s, epi);
+  // The kernels below split K across workgroups through arrival counters owned per stream; a stream that got none
+  // (more streams than counter regions) is planned as if it had no workspace: same results, no split.
+  if (workspace_bytes && !counter_slot_device_ptr(s)) workspace_bytes = 0;
   if (w4a16_astream_supported(m, n, k)) {
     // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
     // never slower than the k-stationary one.  With two it wins while every workgroup gets one to four column

@@ -662,6 +662,8 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
     return fp8_launch_prefill(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
                               static_cast<hipStream_t>(stream), epi);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
+  // split-K needs the stream's arrival counters; a stream that got none is planned as if it had no workspace
+  if (workspace && !counter_slot_device_ptr(static_cast<hipStream_t>(stream))) workspace = nullptr;
   if (m <= 64) {
     const char* e = tuning_env("KSQ_FP8_KSTAT");  // tuning / test switch: 0 sends small m to the streaming kernel
     if (!(e && atoi(e) == 0)) {
@@ -692,8 +694,8 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
   if (w_scale_count == n && n == 1) a.w_scale_per_col = 0;
   a.counters = nullptr;
   if (plan.ksplit > 1) {
-    a.counters = counter_slot_device_ptr();
-    if (!a.counters) return KSQ_ERR_HIP;
+    a.counters = counter_slot_device_ptr(static_cast<hipStream_t>(stream));
+    KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   KSQ_REQUIRE(plan.mblocks <= 65535, KSQ_ERR_UNSUPPORTED, "m too large");
   dim3 grid((unsigned)((a.ntiles + 3) / 4), (unsigned)plan.ksplit, (unsigned)plan.mblocks);

@@ -349,8 +349,8 @@ int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const v
   a.counters = nullptr;
   if (plan.ksplit > 1) {
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
-    a.counters = counter_slot_device_ptr();
-    if (!a.counters) return KSQ_ERR_HIP;
+    a.counters = counter_slot_device_ptr(s);
+    KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
   if (out_dtype == KSQ_F16) launch<_Float16>(plan.mt, plan.tpw, plan.nb, a, grid, s);

@@ -64,12 +64,13 @@ __host__ __device__ inline int frag_nibble_of(int e) { return (e & 1) ? 4 + (e >
 
 // ---- split-K bookkeeping -----------------------------------------------------------------------------------
 // Arrival counters of the split-K fix-up.  They live in library-owned device memory (zero at load, returned
-// to zero by the last-arriving wave of every tile), so no launch has to clear anything.  Launches rotate over
-// kCounterSlots regions so that calls in flight on different streams do not share counters unless more than
-// kCounterSlots overlap.
-constexpr int kCounterSlots = 16;
+// to zero by the last-arriving wave of every tile), so no launch has to clear anything.  Every stream that launches
+// a split-K kernel owns one of kCounterSlots regions for good: launches on one stream run one after the other, so
+// they never share counters with a launch still in flight.  A device's first kCounterSlots streams get a region;
+// for any later stream this returns nullptr and the caller plans without a split across workgroups.
+constexpr int kCounterSlots = 64;
 constexpr int kCountersPerSlot = 16384;
-unsigned* counter_slot_device_ptr();  // next slot (device address), or nullptr on failure
+unsigned* counter_slot_device_ptr(hipStream_t stream);  // the stream's region (device address) or nullptr
 
 #if defined(__HIPCC__)
 // Split-K partial tiles cross workgroups (and XCDs, each with its own L2) through agent-scope relaxed atomics:

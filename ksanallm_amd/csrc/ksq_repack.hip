@@ -17,7 +17,24 @@ struct RepackArgs {
   int layout, zero_kind, scale_dtype;
   const int32_t* row_perm;  // destination row i holds source row row_perm[i]; null = identity
   int column_order;
+  const int8_t* col_exp;    // host repack: column_exponent() of every source scale column, computed once; else null
 };
+
+// bf16 scales only: the largest binary exponent among the finite, non-zero scales of source scale column `ns` (0
+// when there is none).  The kernels that run their matrix instructions in fp16 divide a column's scales by 2 to
+// this power, which keeps them inside the fp16 range whatever their magnitude, and put the factor back on the fp32
+// result of the column.
+__host__ __device__ inline int column_exponent(const RepackArgs& a, size_t ns) {
+  if (a.scale_dtype != KSQ_BF16) return 0;
+  if (a.col_exp) return a.col_exp[ns];
+  const size_t G = a.K / a.g;
+  int best = -1000;
+  for (size_t gi = 0; gi < G; ++gi) {
+    const int e = (static_cast<const uint16_t*>(a.scales)[gi * a.N + ns] >> 7) & 0xFF;
+    if (e != 0 && e != 255 && e - 127 > best) best = e - 127;
+  }
+  return best == -1000 ? 0 : best;
+}
 
 // source column of destination column n
 __host__ __device__ inline size_t source_column(const RepackArgs& a, size_t n) {
@@ -191,7 +208,7 @@ __host__ __device__ inline uint32_t build_sz_word(const RepackArgs& a, size_t id
     default:
       break;
   }
-  return (uint32_t)sbits | (z << 16);
+  return (uint32_t)sbits | (z << 16) | ((uint32_t)(uint8_t)(int8_t)column_exponent(a, ns) << 24);
 }
 
 __global__ __launch_bounds__(256) void repack_weight_kernel(RepackArgs a, size_t words) {
@@ -319,6 +336,12 @@ extern "C" int ksq_w4a16_repack_ex_host(int layout, const void* qweight, int zer
   RepackArgs a = make_args(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, row_perm, column_order,
                            dst_weight, dst_sz);
   const size_t words = k * n / 8, count = (k / g) * n;
+  std::vector<int8_t> col_exp;
+  if (scale_dtype == KSQ_BF16) {
+    col_exp.resize(n);
+    for (size_t ns = 0; ns < n; ++ns) col_exp[ns] = (int8_t)column_exponent(a, ns);
+    a.col_exp = col_exp.data();
+  }
   for (size_t i = 0; i < words; ++i) a.dst_weight[i] = build_weight_word(a, i);
   for (size_t i = 0; i < count; ++i) a.dst_sz[i] = build_sz_word(a, i);
   return KSQ_OK;

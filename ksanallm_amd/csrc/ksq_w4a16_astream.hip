@@ -206,7 +206,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     for (int i = 0; i < CNT; ++i) {
       const uint32_t szw = t.sz[i][GPT == 2 ? h : 0];
       const float s = O::scale_to_float(szw);
-      const float nsz = -s * (O::kBias + (float)(szw >> 16));  // exact: 11 x 11 significant bits
+      const float nsz = -s * (O::kBias + (float)((szw >> 16) & 15u));  // exact: 11 x 11 significant bits
       f32x4 P[MT];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -424,7 +424,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     for (int i = 0; i < CNT; ++i) {
       const uint32_t szw = t.sz[i][GPT == 2 ? h : 0];
       const float s = O::scale_to_float(szw);
-      const float nsz = -s * (O::kBias + (float)(szw >> 16));
+      const float nsz = -s * (O::kBias + (float)((szw >> 16) & 15u));
       f32x4 P[MT];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -609,8 +609,8 @@ int w4a16_launch_astream(int dtype, const AstreamPlan& plan, void* out, const vo
   a.counters = nullptr;
   if (plan.ksplit > 1) {
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
-    a.counters = counter_slot_device_ptr();
-    if (!a.counters) return KSQ_ERR_HIP;
+    a.counters = counter_slot_device_ptr(s);
+    KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   const int mt = plan.mt;
   const int gpt = (int)(kTileK / g);

@@ -178,7 +178,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
 #pragma unroll
         for (int gi = 0; gi < GPT; ++gi) {
           const uint32_t szw = szq[slot][gi];
-          const uint32_t z = szw >> 16;
+          const uint32_t z = (szw >> 16) & 15u;
           const u32x4 corr = O::correction(z | (z << 16));
           const float s = O::scale_to_float(szw);
           f32x4 P[MT];
@@ -394,8 +394,8 @@ int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* 
   a.counters = nullptr;
   if (plan.ksplit > 1) {
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
-    a.counters = counter_slot_device_ptr();
-    if (!a.counters) return KSQ_ERR_HIP;
+    a.counters = counter_slot_device_ptr(s);
+    KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
   const int gpt = (int)(kTileK / g);

@@ -101,7 +101,7 @@ struct Dequant<_Float16> {
     uint32_t s2, c_lo, c_hi;
   };
   static __device__ inline Consts prepare(uint32_t szw) {
-    const uint32_t z = szw >> 16, zc = z | (z << 16);
+    const uint32_t z = (szw >> 16) & 15u, zc = z | (z << 16);
     Consts k;
     k.s2 = (szw & 0xFFFFu) | (szw << 16);
     k.c_lo = 0x64006400u | zc;
@@ -124,13 +124,28 @@ struct Dequant<_Float16> {
 
 template <>
 struct Dequant<__bf16> : Dequant<_Float16> {
-  // scales arrive as bf16 bits; the arithmetic is the fp16 one
+  // Scales arrive as bf16 bits; the arithmetic is the fp16 one.  A bf16 scale can lie far outside the fp16 range, so
+  // the scale is first divided by 2^E, E = the column's largest scale exponent (bits 24..31 of every scale/zero word
+  // of the column, written by the repack): the column's largest scale becomes 1.x, smaller ones keep all their
+  // bits down to 2^-14 of it.  column_factors() below gives the 2^E that the fp32 result of the column is owed.
   static __device__ inline Consts prepare(uint32_t szw) {
-    const _Float16 sh = (_Float16)__builtin_bit_cast(float, szw << 16);
+    const _Float16 sh = (_Float16)__builtin_ldexpf(__builtin_bit_cast(float, szw << 16), -((int)szw >> 24));
     const uint32_t sb = __builtin_bit_cast(uint16_t, sh);
-    return Dequant<_Float16>::prepare((szw & 0xFFFF0000u) | sb);
+    return Dequant<_Float16>::prepare((szw & 0x000F0000u) | sb);
   }
 };
+
+// 2^E of the eight columns col .. col + 7 (col a multiple of 8, col + 8 <= N) of a weight with bf16 scales; sz is the
+// scale/zero buffer [N/16][G][16].
+__device__ inline void column_factors(const void* sz, int G, int col, float (&f)[8]) {
+  const uint32_t* w = static_cast<const uint32_t*>(sz) + ((size_t)(col >> 4) * G) * 16 + (col & 15);
+  const u32x4 lo = *reinterpret_cast<const u32x4*>(w), hi = *reinterpret_cast<const u32x4*>(w + 4);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    f[q] = __builtin_bit_cast(float, (uint32_t)(((int)lo[q] >> 24) + 127) << 23);
+    f[4 + q] = __builtin_bit_cast(float, (uint32_t)(((int)hi[q] >> 24) + 127) << 23);
+  }
+}
 
 }  // namespace w4
 }  // namespace ksq

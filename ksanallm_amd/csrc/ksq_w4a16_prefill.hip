@@ -14,8 +14,9 @@
 // 2^-8 per weight -- together with the bf16 rounding of the output more than the 1e-2 bound on the maximum relative
 // error allows -- so bf16 activations are first re-encoded, exactly, as fp16 with one power-of-two exponent per row
 // (a bf16 significand fits into fp16; the row exponent keeps every row inside the fp16 range whatever its
-// magnitude); the row factor 2^e is applied to the fp32 accumulators in the epilogue, and the bf16 group scales
-// are converted to fp16.
+// magnitude); the row factor 2^e is applied to the fp32 accumulators in the epilogue.  The bf16 group scales are
+// converted to fp16 after division by a power of two per column (the column's largest scale exponent, kept in
+// every scale/zero word by the repack), which the epilogue puts back, so scales far outside the fp16 range work.
 // Workgroups are numbered so that those sharing a row block of the activations run on the same XCD (own L2).
 #include <cstdlib>
 #include <type_traits>
@@ -299,6 +300,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   float* epi = reinterpret_cast<float*>(wave < 4 ? lds_a0 : lds_a1) + (wave & 3) * (16 * kEpiStride);  // 4352 B
   uint16_t* out = static_cast<uint16_t*>(p.out);
   const int ncol0 = nt0 * 16;
+  float cf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // bf16 scales: 2^E of this lane's eight columns
+  if constexpr (kBF16) {
+    const int col = ncol0 + (lane & 7) * 8;
+    if (col + 8 <= p.N) column_factors(p.sz, p.G, col, cf);
+  }
 #pragma unroll
   for (int mt = 0; mt < kMT; ++mt) {
 #pragma unroll
@@ -315,7 +321,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
       float vals[8];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs;
+      for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs * cf[q];
       if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -503,6 +509,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   float* epi = reinterpret_cast<float*>(wave == 0 ? lds_a0 : wave == 1 ? lds_a1 : wave == 2 ? lds_a2 : lds_a3);
   uint16_t* out = static_cast<uint16_t*>(p.out);
   const int ncol0 = nt0 * 16;
+  float cf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // bf16 scales: 2^E of this lane's eight columns
+  if constexpr (kBF16) {
+    const int col = ncol0 + (lane & 7) * 8;
+    if ((lane & 7) * 8 < 16 * KNT && col + 8 <= p.N) column_factors(p.sz, p.G, col, cf);
+  }
 #pragma unroll
   for (int mt = 0; mt < kRows; ++mt) {
 #pragma unroll
@@ -528,7 +539,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
       }
       float vals[8];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs;
+      for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs * cf[q];
       if (live) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -540,7 +551,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
 template <typename T>
 __global__ __launch_bounds__(256) void w4a16_splitk_reduce_kernel(const float* __restrict__ partial, size_t split_stride,
                                                                   int ksplit, const float* __restrict__ row_scale,
-                                                                  uint16_t* out, int M, int N, Epilogue epi) {
+                                                                  const void* sz, int G, uint16_t* out, int M, int N,
+                                                                  Epilogue epi) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t segs = (size_t)N / 8;
   const size_t row = idx / segs;
@@ -553,7 +565,10 @@ __global__ __launch_bounds__(256) void w4a16_splitk_reduce_kernel(const float* _
     hi += src[sp * (split_stride / 4) + 1];
   }
   const float rs = row_scale ? row_scale[row] : 1.f;
-  const float vals[8] = {lo[0] * rs, lo[1] * rs, lo[2] * rs, lo[3] * rs, hi[0] * rs, hi[1] * rs, hi[2] * rs, hi[3] * rs};
+  float cf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+  if (sz) column_factors(sz, G, col, cf);  // bf16 scales: the column's 2^E
+  const float vals[8] = {lo[0] * rs * cf[0], lo[1] * rs * cf[1], lo[2] * rs * cf[2], lo[3] * rs * cf[3],
+                         hi[0] * rs * cf[4], hi[1] * rs * cf[5], hi[2] * rs * cf[6], hi[3] * rs * cf[7]};
   epi_store_row8<T>(epi, out, vals, (int)row, col, N);
 }
 
@@ -732,10 +747,10 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     uint16_t* o = static_cast<uint16_t*>(out);
     if (dtype == KSQ_F16)
       hipLaunchKernelGGL(w4a16_splitk_reduce_kernel<_Float16>, rgrid, dim3(256), 0, s, a.partial, stride, plan.ksplit,
-                         a.row_scale, o, (int)m, (int)n, epi);
+                         a.row_scale, (const void*)nullptr, a.G, o, (int)m, (int)n, epi);
     else
       hipLaunchKernelGGL(w4a16_splitk_reduce_kernel<__bf16>, rgrid, dim3(256), 0, s, a.partial, stride, plan.ksplit,
-                         a.row_scale, o, (int)m, (int)n, epi);
+                         a.row_scale, sz, a.G, o, (int)m, (int)n, epi);
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;

@@ -188,7 +188,7 @@ w4a16_stream_kernel(StreamArgs p) {
 #pragma unroll
       for (int gi = 0; gi < GPT; ++gi) {
         const uint32_t szw = szq[slot][t][gi];
-        const uint32_t z = szw >> 16;
+        const uint32_t z = (szw >> 16) & 15u;
         const u32x4 corr = O::correction(z | (z << 16));
         cur_s[t][gi] = O::scale_to_float(szw);
 #pragma unroll
@@ -400,8 +400,8 @@ int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* ac
     KSQ_REQUIRE(workspace != nullptr, KSQ_ERR_WORKSPACE, "split-K planned without a workspace");
     KSQ_REQUIRE((size_t)a.ngroups * plan.mblocks <= (size_t)kCountersPerSlot, KSQ_ERR_UNSUPPORTED,
                 "too many tiles for the split-K counters");
-    a.counters = counter_slot_device_ptr();
-    if (!a.counters) return KSQ_ERR_HIP;
+    a.counters = counter_slot_device_ptr(s);
+    KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   KSQ_REQUIRE(plan.mblocks <= 65535 && plan.ksplit <= 65535, KSQ_ERR_UNSUPPORTED, "grid too large");
   dim3 grid((unsigned)((a.ngroups + 3) / 4), (unsigned)plan.ksplit, (unsigned)plan.mblocks);

@@ -65,7 +65,35 @@ def test_host_repack_fragment_order(g):
             assert np.array_equal(dw, want)
             szw = dsz.reshape(N // 16, K // g, 16).transpose(1, 0, 2).reshape(K // g, N)
             assert np.array_equal((szw & 0xFFFF).astype(np.uint16), s)
-            assert np.array_equal((szw >> 16).astype(np.uint8), zwant)
+            assert np.array_equal(((szw >> 16) & 0xFF).astype(np.uint8), zwant)
+            # bits 24..31: with bf16 scales, the largest binary exponent of the column's scales in every word of it
+            col_exp = np.floor(np.log2(orc.from_bits(s, orc.BF16))).max(axis=0).astype(np.int64)
+            assert np.array_equal((szw >> 24).astype(np.uint8).view(np.int8), np.tile(col_exp.astype(np.int8), (K // g, 1)))
+
+
+def test_host_repack_column_exponent_of_bf16_scales():
+    """Bits 24..31 of a scale/zero word: zero for fp16 scales; for bf16 scales the largest exponent among the column's
+    finite non-zero scales (zero for a column of zeros), whatever the magnitudes."""
+    rng = np.random.default_rng(32)
+    K, N, g = 512, 32, 128
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    sv = np.exp2(rng.integers(-120, 120, size=(K // g, N)).astype(np.float64)) * (1 + rng.random((K // g, N)))
+    sv[:, 3] = 0.0
+    sv[1, 5] = 0.0
+    s = orc.to_bits(sv.astype(np.float32), orc.BF16)
+    back = orc.from_bits(s, orc.BF16).astype(np.float64)
+    want = np.zeros(N, dtype=np.int64)
+    for n in range(N):
+        nz = back[:, n][back[:, n] > 0]
+        want[n] = int(np.floor(np.log2(nz)).max()) if nz.size else 0
+    dw = np.zeros(K * N // 8, dtype=np.uint32)
+    dsz = np.zeros((K // g) * N, dtype=np.uint32)
+    capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, orc.gptq_pack(u), capi.ZERO_NONE, None, s, capi.BF16, K, N, g, dw, dsz)
+    szw = dsz.reshape(N // 16, K // g, 16).transpose(1, 0, 2).reshape(K // g, N)
+    assert np.array_equal((szw >> 24).astype(np.uint8).view(np.int8).astype(np.int64), np.tile(want, (K // g, 1)))
+    s16 = orc.to_bits(np.clip(sv, 0, 6e4).astype(np.float32), orc.F16)
+    capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, orc.gptq_pack(u), capi.ZERO_NONE, None, s16, capi.F16, K, N, g, dw, dsz)
+    assert np.all(dsz >> 24 == 0)
 
 
 def test_additive_zero_recovery_fp16_all_values():
@@ -82,7 +110,7 @@ def test_additive_zero_recovery_fp16_all_values():
     dsz = np.zeros(N, dtype=np.uint32)
     capi.w4a16_repack_host(capi.W4_GPTQ_INT32_KPACK, orc.gptq_pack(u), capi.ZERO_ADDITIVE, za, s, capi.F16, K, N, g,
                            dw, dsz)
-    got = (dsz.reshape(N // 16, 1, 16) >> 16).astype(np.uint8).transpose(1, 0, 2).reshape(1, N)
+    got = ((dsz.reshape(N // 16, 1, 16) >> 16) & 0xFF).astype(np.uint8).transpose(1, 0, 2).reshape(1, N)
     assert np.array_equal(got, z)
 
 

@@ -292,6 +292,26 @@ def test_prefill_bf16_row_magnitudes(gpu):
             orc.assert_parity(got[row:row + 1], want[row:row + 1], f"row {row} (2^{exps[row]})")
 
 
+@pytest.mark.parametrize("M", [16, 65, 600])
+def test_bf16_scales_far_outside_the_fp16_range(gpu, M):
+    """bf16 group scales from 1e-6 to 1e5, different per column block and with a wide spread inside some columns: the
+    decode kernels (M = 16) keep scales in fp32, the 64-row and 128-row kernels (M = 65, 600) run their matrix
+    instructions in fp16 and must still be right, column block by column block."""
+    K, N = 1024, 1024
+    rng = np.random.default_rng(1290 + M)
+    G = K // 128
+    base = np.repeat(np.array([1e-6, 3e-5, 1e-3, 0.02, 7.0, 3e3, 1e5, 2e-2], dtype=np.float32), N // 8)[None, :]
+    sv = base * (1 + rng.random((G, N), dtype=np.float32))
+    sv[:, -128:] *= np.exp2(rng.integers(-10, 1, size=(G, 128))).astype(np.float32)  # spread inside a column
+    case = W4Case(1291, M, K, N, kind="awq", dtype="bf16", scales=sv)
+    got = W4Device(case, gpu).gemm_f32()
+    want = case.oracle()
+    assert np.all(np.isfinite(got))
+    for b in range(8):
+        cols = slice(b * N // 8, (b + 1) * N // 8)
+        orc.assert_parity(got[:, cols], want[:, cols], f"M={M} column block {b} (scale ~ {base[0, b * N // 8]:g})")
+
+
 def test_no_workspace_still_correct(gpu):
     case = W4Case(1300, 16, 4096, 512, kind="gptq", dtype="f16")
     dev = W4Device(case, gpu)
