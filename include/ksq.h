@@ -122,13 +122,19 @@ int ksq_device_compute_units(void);
  * (KS/models/quant/quant_weight.cpp:331-346, 577-579; LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508)
  * and the scale / zero binding of ConvertGroupTensor (quant_weight.cpp:530-536, 632-636).
  *
- * Output "fragment order" (K % 128 == 0, N % 16 == 0, g in {64,128}):
+ * Output "fragment order" (K % 128 == 0, N % 16 == 0, g in {64,128}; the reference's kernels take K % 64 == 0,
+ * LK/asymmetric_gemm/fpA_intB_gemm/fpA_intB_gemm_template.h:168-171: a K that is an odd multiple of 64 is refused
+ * here with KSQ_ERR_UNSUPPORTED):
  *   weight : K*N/2 bytes = tiles [N/16][K/128] of 1024 B.  Tile (nt,kt) is 64 lanes x 16 B; lane l = 16*j + c
  *            owns column n = 16*nt + c; 32-bit word d (0..3) of the lane covers k = 128*kt + 32*d + 8*j + e,
  *            e = 0..7, with element e in nibble e/2 when e is even and nibble 4 + e/2 when e is odd; nibbles are
  *            the unsigned u in [0,15].  One 128-bit load per lane is the B operand of four 16x16x32 MFMAs.
  *   sz     : (K/g)*N 32-bit words = [N/16][K/g][16]; word = scale bits (T) | z << 16 with z in [0,15]
  *            | E << 24, E (int8) = the largest binary exponent among the column's scales when they are bf16, else 0. */
+/* Column tiles are contiguous in both buffers: tensors that share K (q_proj / k_proj / v_proj, gate_proj / up_proj)
+ * are fused along N by repacking each, in order, to dst_weight + ksq_w4a16_repack_sizes(k, n_before).weight_bytes and
+ * dst_sz + ...sz_bytes, n_before = the columns already placed (a multiple of 16); no concatenated copy is needed
+ * (replaces the concat of KS/models/quant/quant_weight.cpp:471-513). */
 int ksq_w4a16_repack_sizes(size_t k, size_t n, size_t group_size, size_t* weight_bytes, size_t* sz_bytes);
 
 int ksq_w4a16_repack(int src_layout, const void* qweight, int zero_kind, const void* zeros, const void* scales,

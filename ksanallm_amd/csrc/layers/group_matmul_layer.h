@@ -66,6 +66,21 @@ Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, c
                               Tensor& weight_sz, int rank, Stream& stream, Tensor* perm = nullptr,
                               bool interleave_gate_up = false);
 
+// Several checkpoint tensors that share K, side by side along N in one repacked weight: what the loader's concat of
+// q_proj / k_proj / v_proj into query_key_value (and of gate_proj / up_proj) does before its repack
+// (KS/models/quant/quant_weight.cpp:471-513), without the concatenated copy: column tiles are contiguous in the
+// fragment order, so every part is repacked straight into its own range of the fused buffers.  Every part's width
+// must be a multiple of 16.
+struct GroupWeightPart {
+  const Tensor* qweight;
+  const Tensor* qzeros;  // nullptr = symmetric
+  const Tensor* scales;
+  size_t n;
+};
+Status RepackFusedGroupQuantWeight(GroupWeightLayout layout, const std::vector<GroupWeightPart>& parts,
+                                   bool zeros_additive, size_t k, size_t groupsize, Tensor& weight, Tensor& weight_sz,
+                                   int rank, Stream& stream);
+
 // perm = stable argsort of a desc_act checkpoint's g_idx (MarlinSortGIdx, quant_weight.cpp:455-460), on the host.
 // Throws unless every group has exactly `groupsize` rows.
 Status SortGptqGIdx(const std::vector<int32_t>& g_idx, size_t groupsize, std::vector<int32_t>& perm);

@@ -148,6 +148,26 @@ void GroupMatMulLayer<T, WT>::SetEpilogue(int kind, const Tensor* bias) {
 template class GroupMatMulLayer<float16, TYPE_I4_GROUP>;
 template class GroupMatMulLayer<bfloat16, TYPE_I4_GROUP>;
 
+namespace {
+
+int KsqLayout(GroupWeightLayout layout) {
+  return layout == GROUP_WEIGHT_GPTQ_INT32     ? KSQ_W4_GPTQ_INT32_KPACK
+         : layout == GROUP_WEIGHT_AWQ_INT32    ? KSQ_W4_AWQ_INT32_NPACK
+         : layout == GROUP_WEIGHT_CUTLASS_SM80 ? KSQ_W4_CUTLASS_SM80_INTERLEAVED
+         : layout == GROUP_WEIGHT_CUTLASS_SM90 ? KSQ_W4_CUTLASS_SM90_COLMAJOR
+         : layout == GROUP_WEIGHT_MARLIN       ? KSQ_W4_MARLIN
+                                               : KSQ_W4_ROWMAJOR_INT4_SIGNED;
+}
+
+int KsqZeroKind(GroupWeightLayout layout, const Tensor* qzeros, bool zeros_additive) {
+  if (qzeros == nullptr) return KSQ_ZERO_NONE;
+  if (layout == GROUP_WEIGHT_MARLIN) return KSQ_ZERO_MARLIN_INT32;
+  if (zeros_additive) return KSQ_ZERO_ADDITIVE;
+  return (qzeros->dtype == TYPE_INT32 || qzeros->dtype == TYPE_UINT32) ? KSQ_ZERO_AWQ_INT32 : KSQ_ZERO_UINT8;
+}
+
+}  // namespace
+
 Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, const Tensor* qzeros,
                               bool zeros_additive, const Tensor& scales, size_t k, size_t n, size_t groupsize,
                               Tensor& weight, Tensor& weight_sz, int rank, Stream& stream, Tensor* perm,
@@ -157,21 +177,10 @@ Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, c
   if (scales.dtype != TYPE_FP16 && scales.dtype != TYPE_BF16) KLLM_THROW("RepackGroupQuantWeight: scales must be fp16 or bf16.");
   CreateTensor(weight, {k, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);  // same shape as ksana's "*.weight"
   CreateTensor(weight_sz, {k / groupsize, n}, TYPE_UINT32, rank, MEMORY_DEVICE);
-  int src = layout == GROUP_WEIGHT_GPTQ_INT32     ? KSQ_W4_GPTQ_INT32_KPACK
-            : layout == GROUP_WEIGHT_AWQ_INT32    ? KSQ_W4_AWQ_INT32_NPACK
-            : layout == GROUP_WEIGHT_CUTLASS_SM80 ? KSQ_W4_CUTLASS_SM80_INTERLEAVED
-            : layout == GROUP_WEIGHT_CUTLASS_SM90 ? KSQ_W4_CUTLASS_SM90_COLMAJOR
-            : layout == GROUP_WEIGHT_MARLIN       ? KSQ_W4_MARLIN
-                                                  : KSQ_W4_ROWMAJOR_INT4_SIGNED;
+  const int src = KsqLayout(layout);
   if (perm != nullptr && (perm->dtype != TYPE_INT32 || perm->GetElementNumber() != k))
     KLLM_THROW("RepackGroupQuantWeight: perm must be int32 [k].");
-  int zero_kind = KSQ_ZERO_NONE;
-  if (qzeros != nullptr) {
-    if (layout == GROUP_WEIGHT_MARLIN) zero_kind = KSQ_ZERO_MARLIN_INT32;
-    else if (zeros_additive) zero_kind = KSQ_ZERO_ADDITIVE;
-    else if (qzeros->dtype == TYPE_INT32 || qzeros->dtype == TYPE_UINT32) zero_kind = KSQ_ZERO_AWQ_INT32;
-    else zero_kind = KSQ_ZERO_UINT8;
-  }
+  const int zero_kind = KsqZeroKind(layout, qzeros, zeros_additive);
   ThrowOnKsqError(
       ksq_w4a16_repack_ex(src, qweight.GetPtr<void>(), zero_kind, qzeros ? qzeros->GetPtr<void>() : nullptr,
                           scales.GetPtr<void>(), scales.dtype == TYPE_FP16 ? KSQ_F16 : KSQ_BF16, k, n, groupsize,
@@ -182,6 +191,43 @@ Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, c
   weight.dtype = TYPE_I4_GROUP;
   weight.scales = &weight_sz;
   weight.perm = perm;
+  return Status();
+}
+
+Status RepackFusedGroupQuantWeight(GroupWeightLayout layout, const std::vector<GroupWeightPart>& parts,
+                                   bool zeros_additive, size_t k, size_t groupsize, Tensor& weight, Tensor& weight_sz,
+                                   int rank, Stream& stream) {
+  size_t n = 0;
+  for (const GroupWeightPart& part : parts) {
+    if (part.qweight == nullptr || part.scales == nullptr || part.n == 0 || part.n % 16 != 0)
+      KLLM_THROW("RepackFusedGroupQuantWeight: every part needs a weight, scales and a width that is a multiple of 16.");
+    if (part.scales->dtype != parts[0].scales->dtype || (part.qzeros == nullptr) != (parts[0].qzeros == nullptr))
+      KLLM_THROW("RepackFusedGroupQuantWeight: the parts must agree in scale type and in having zero points.");
+    n += part.n;
+  }
+  if (parts.empty()) KLLM_THROW("RepackFusedGroupQuantWeight: no parts.");
+  const DataType st = parts[0].scales->dtype;
+  if (st != TYPE_FP16 && st != TYPE_BF16) KLLM_THROW("RepackFusedGroupQuantWeight: scales must be fp16 or bf16.");
+  size_t weight_bytes = 0, sz_bytes = 0;
+  ThrowOnKsqError(ksq_w4a16_repack_sizes(k, n, groupsize, &weight_bytes, &sz_bytes), "ksq_w4a16_repack_sizes");
+  CreateTensor(weight, {k, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);
+  CreateTensor(weight_sz, {k / groupsize, n}, TYPE_UINT32, rank, MEMORY_DEVICE);
+  size_t n0 = 0;
+  for (const GroupWeightPart& part : parts) {
+    // columns n0 .. n0 + part.n - 1 are the column tiles n0 / 16 .. of the fused buffers: a contiguous range of each
+    size_t part_w = 0, part_sz = 0;
+    ThrowOnKsqError(ksq_w4a16_repack_sizes(k, n0 == 0 ? part.n : n0, groupsize, &part_w, &part_sz), "ksq_w4a16_repack_sizes");
+    const size_t w_off = n0 == 0 ? 0 : part_w, sz_off = n0 == 0 ? 0 : part_sz;  // bytes taken by the columns before n0
+    ThrowOnKsqError(
+        ksq_w4a16_repack(KsqLayout(layout), part.qweight->GetPtr<void>(), KsqZeroKind(layout, part.qzeros, zeros_additive),
+                         part.qzeros ? part.qzeros->GetPtr<void>() : nullptr, part.scales->GetPtr<void>(),
+                         st == TYPE_FP16 ? KSQ_F16 : KSQ_BF16, k, part.n, groupsize, weight.GetPtr<char>() + w_off,
+                         weight_sz.GetPtr<char>() + sz_off, stream.Get()),
+        "ksq_w4a16_repack");
+    n0 += part.n;
+  }
+  weight.dtype = TYPE_I4_GROUP;
+  weight.scales = &weight_sz;
   return Status();
 }
 

@@ -61,7 +61,7 @@ static int RunW4(int argc, char** argv) {
   const std::string dir = argv[2];
   const size_t m = atol(argv[4]), k = atol(argv[5]), n = atol(argv[6]), g = atol(argv[7]);
   const std::string method = argv[8], layout = argv[9], zeros = argv[10];
-  const std::string extra = argc > 11 ? argv[11] : "none";  // none | desc | silu | bias
+  const std::string extra = argc > 11 ? argv[11] : "none";  // none | desc | silu | bias | parts:n0:n1:..
   const DataType dt = TypeTraits<T>::kDataType;
   auto context = std::make_shared<Context>(1);
 
@@ -103,8 +103,32 @@ static int RunW4(int argc, char** argv) {
     memcpy(bytes.data(), order.data(), bytes.size());
     perm = Upload(bytes, TYPE_INT32, {k});
   }
-  RepackGroupQuantWeight(lay, qweight, zp, additive, scales, k, n, g, weight, weight_sz, 0,
-                         context->GetComputeStreams()[0], extra == "desc" ? &perm : nullptr, extra == "silu");
+  std::vector<Tensor> part_tensors;  // qweight, qzeros, scales of every part (kept alive until the repack ran)
+  if (extra.rfind("parts:", 0) == 0) {
+    // "parts:n0:n1:..": the AWQ checkpoint comes as separate tensors qweight_i.bin / qzeros_i.bin / scales_i.bin that
+    // share K (q_proj, k_proj, v_proj); they are repacked side by side into one fused weight
+    std::vector<size_t> widths;
+    for (size_t pos = 6; pos < extra.size();) {
+      const size_t end = extra.find(':', pos);
+      widths.push_back(std::stoul(extra.substr(pos, end - pos)));
+      pos = end == std::string::npos ? extra.size() : end + 1;
+    }
+    part_tensors.reserve(3 * widths.size());
+    std::vector<GroupWeightPart> parts;
+    for (size_t i = 0; i < widths.size(); ++i) {
+      const std::string tag = "_" + std::to_string(i) + ".bin";
+      part_tensors.push_back(Upload(ReadFile(dir + "/qweight" + tag), TYPE_INT32, {k, widths[i] / 8}));
+      part_tensors.push_back(Upload(ReadFile(dir + "/qzeros" + tag), TYPE_INT32, {k / g, widths[i] / 8}));
+      part_tensors.push_back(Upload(ReadFile(dir + "/scales" + tag), dt, {k / g, widths[i]}));
+      const size_t base = part_tensors.size() - 3;
+      parts.push_back({&part_tensors[base], &part_tensors[base + 1], &part_tensors[base + 2], widths[i]});
+    }
+    RepackFusedGroupQuantWeight(GROUP_WEIGHT_AWQ_INT32, parts, false, k, g, weight, weight_sz, 0,
+                                context->GetComputeStreams()[0]);
+  } else {
+    RepackGroupQuantWeight(lay, qweight, zp, additive, scales, k, n, g, weight, weight_sz, 0,
+                           context->GetComputeStreams()[0], extra == "desc" ? &perm : nullptr, extra == "silu");
+  }
 
   ModelConfig cfg;
   cfg.is_quant = true;

@@ -102,6 +102,31 @@ def test_group_matmul_layer_widened(gpu, tmp_path, dtype, extra, layout, M):
     orc.assert_parity(got, want, f"GroupMatMulLayer {layout} {extra} {dtype}")
 
 
+@pytest.mark.parametrize("dtype,M", [("f16", 16), ("bf16", 70)])
+def test_group_matmul_layer_fused_from_separate_projections(gpu, tmp_path, dtype, M):
+    """q_proj / k_proj / v_proj of an AWQ checkpoint as three tensors, repacked side by side into one fused weight
+    (RepackFusedGroupQuantWeight) and served by one layer: equals the GEMM against the concatenated weight."""
+    K, g = 1024, 128
+    widths = [256, 64, 64]
+    N = sum(widths)
+    case = W4Case(620 + M, M, K, N, g=g, kind="awq", dtype=dtype)
+    d = str(tmp_path)
+    n0 = 0
+    for i, w in enumerate(widths):
+        orc.awq_pack(np.ascontiguousarray(case.u[:, n0:n0 + w])).tofile(f"{d}/qweight_{i}.bin")
+        orc.awq_pack(np.ascontiguousarray(case.z[:, n0:n0 + w])).tofile(f"{d}/qzeros_{i}.bin")
+        np.ascontiguousarray(case.scales[:, n0:n0 + w]).tofile(f"{d}/scales_{i}.bin")
+        n0 += w
+    case.awq_qweight().tofile(d + "/qweight.bin")   # the driver reads these too; the parts are what it repacks
+    case.awq_qzeros().tofile(d + "/qzeros.bin")
+    case.scales.tofile(d + "/scales.bin")
+    case.act.tofile(d + "/act.bin")
+    rc, out = _run(["w4a16", d, dtype, M, K, N, g, "awq", "awq", "awq", "parts:" + ":".join(map(str, widths))])
+    assert rc == 0 and out.splitlines()[-1] == f"OK {M} {N} {DTYPE_ENUM[dtype]}", out
+    got = orc.from_bits(np.fromfile(d + "/out.bin", dtype=np.uint16).reshape(M, N), ORC_DT[dtype])
+    orc.assert_parity(got, case.oracle(), f"fused q/k/v {dtype}")
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("wscales,static,M", [("1", 0, 7), ("1", 1, 7), ("n", 0, 40)])
 def test_fp8_matmul_layer_forward(gpu, tmp_path, dtype, wscales, static, M):

@@ -310,3 +310,33 @@ def test_marlin_argument_rules():
                                np.zeros((1, 48), dtype=np.uint16), capi.F16, K, 48, g, np.zeros(K * 48 // 8, np.uint32),
                                np.zeros(48, np.uint32))
     assert e.value.code == capi.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_parts_repacked_side_by_side_equal_the_concatenated_repack(dtype):
+    """Column tiles are contiguous in the fragment order and in the scale/zero words, so tensors that share K can be
+    repacked one by one into consecutive ranges of the fused buffers (what replaces the loader's q/k/v concat,
+    KS/models/quant/quant_weight.cpp:471-513): bit for bit the repack of the concatenated tensor."""
+    rng = np.random.default_rng(77)
+    K, g = 512, 128
+    widths = [96, 32, 48]
+    N = sum(widths)
+    odt = orc.F16 if dtype == "f16" else orc.BF16
+    cdt = capi.F16 if dtype == "f16" else capi.BF16
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8)
+    s = orc.to_bits((np.abs(rng.standard_normal((K // g, N))) * 0.02 + 1e-3).astype(np.float32), odt)
+    want_w = np.zeros(K * N // 8, dtype=np.uint32)
+    want_sz = np.zeros((K // g) * N, dtype=np.uint32)
+    capi.w4a16_repack_host(capi.W4_AWQ_INT32_NPACK, orc.awq_pack(u), capi.ZERO_AWQ_INT32, orc.awq_pack(z), s, cdt, K, N, g,
+                           want_w, want_sz)
+    got_w, got_sz = np.zeros_like(want_w), np.zeros_like(want_sz)
+    n0 = 0
+    for w in widths:
+        wb, sb = capi.w4a16_repack_sizes(K, n0, g) if n0 else (0, 0)
+        capi.w4a16_repack_host(capi.W4_AWQ_INT32_NPACK, orc.awq_pack(np.ascontiguousarray(u[:, n0:n0 + w])),
+                               capi.ZERO_AWQ_INT32, orc.awq_pack(np.ascontiguousarray(z[:, n0:n0 + w])),
+                               np.ascontiguousarray(s[:, n0:n0 + w]), cdt, K, w, g, got_w[wb // 4:], got_sz[sb // 4:])
+        n0 += w
+    assert np.array_equal(got_w, want_w)
+    assert np.array_equal(got_sz, want_sz)
