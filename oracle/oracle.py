@@ -133,12 +133,14 @@ def awq_additive_zeros(scales_bits, dtype, z):
 
 
 # ---------------------------------------------------------------- dequantize-then-GEMM
-def dequant(u, scales_bits, sdtype, z, g):
+def dequant(u, scales_bits, sdtype, z, g, out=None):
+    """fp32 [K,N] = s * (u - z); ``out`` = a C-contiguous float32 [K,N] buffer to fill instead of a new array."""
     u = _c(u, np.uint8)
     scales_bits = _c(scales_bits)
     z = _c(z, np.uint8) if z is not None else None
     K, N = u.shape
-    w = np.empty((K, N), dtype=np.float32)
+    w = np.empty((K, N), dtype=np.float32) if out is None else out
+    assert w.shape == (K, N) and w.dtype == np.float32 and w.flags.c_contiguous
     lib().orc_dequant(_p(u), _p(scales_bits), sdtype, _p(z), _sz(K), _sz(N), _sz(g), _p(w))
     return w
 
