@@ -33,8 +33,14 @@ struct KstatArgs {
   Epilogue epi;
 };
 
-template <typename T, int GPT, int MT, int TPW, int NB, int NW>
+// PPI = 16-byte pieces of one activation row that one load instruction brings in (4, 8 or 16): a load covers 64 / PPI
+// rows, so with few rows (M <= 8, M <= 4) a k tile takes two or one instruction instead of four.  The memory pipeline
+// of a compute unit holds a limited number of instructions in flight, whatever their size or lane mask, and at the
+// start of this kernel that window is what every wave waits for.
+template <typename T, int GPT, int MT, int TPW, int NB, int NW, int PPI>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4))) void w4a16_kstat_kernel(KstatArgs p) {
+  static_assert(PPI == 4 || ((PPI == 8 || PPI == 16) && MT == 1), "wide activation loads: one row tile only");
+  constexpr int API = 16 / PPI;  // activation load instructions per k tile
   using O = Ops<T>;
   constexpr int DPG = 4 / GPT;
   constexpr int D = NB * TPW;  // ring depth = one batch
@@ -85,23 +91,23 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
     sz_off[r] = ok ? (unsigned)i * sz_stride + (unsigned)gq * 64u + (unsigned)c * 4u : 0x80000000u;
   }
 
-  // Activation fragments of this wave's k tiles: registers for the whole kernel.  They are loaded with lane l on
-  // row l / 4, 16-byte piece l % 4 of a 32-k step, so that every aligned group of four lanes reads 64 contiguous
-  // bytes (the memory pipeline then takes four lanes per clock instead of one), and moved to the MFMA operand layout
-  // (lane 16 j + c = row c, piece j) by a lane permutation further down.
+  // Activation fragments of this wave's k tiles: registers for the whole kernel.  Load instruction i of a k tile has
+  // lane l on row l / PPI, 16-byte piece i * PPI + l % PPI of the tile's 16, so that every aligned group of four lanes
+  // reads 64 contiguous bytes (the memory pipeline then takes four lanes per clock instead of one); the MFMA operand
+  // layout (lane 16 j + c = row c, piece 4 d + j for the 32-k step d) comes from a lane permutation further down.
   u32x4 af[MT][TPW][4];
   {
-    const int lr = lane >> 2, lp = lane & 3;
+    const int lr = lane / PPI, lp = lane % PPI;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int t = 0; t < TPW; ++t)
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
+        for (int i = 0; i < API; ++i) {
           const int row = 16 * mt + lr;
           const bool ok = row < p.M && kt0 + t < wg_end;
-          const unsigned ao = ok ? ((unsigned)row * p.K + (kt0 + t) * kTileK + 32 * d + 8 * lp) * 2u : 0x80000000u;
-          af[mt][t][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+          const unsigned ao = ok ? ((unsigned)row * p.K + (kt0 + t) * kTileK + 8 * (i * PPI + lp)) * 2u : 0x80000000u;
+          af[mt][t][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
         }
   }
 
@@ -136,17 +142,34 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  {  // lane 16 j + c takes what lane 4 c + j loaded
-    const int from = (4 * c + j) * 4;
+  {  // lane 16 j + c takes piece 4 d + j of row c: loaded by instruction (4 d + j) / PPI, lane c * PPI + (4 d + j) % PPI
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int t = 0; t < TPW; ++t)
+      for (int t = 0; t < TPW; ++t) {
+        u32x4 got[4];
 #pragma unroll
-        for (int d = 0; d < 4; ++d)
+        for (int d = 0; d < 4; ++d) {
+          const int piece = 4 * d + j;
+          const int from = (c * PPI + piece % PPI) * 4;
 #pragma unroll
-          for (int q = 0; q < 4; ++q)
-            af[mt][t][d][q] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)af[mt][t][d][q]);
+          for (int q = 0; q < 4; ++q) {
+            uint32_t v = 0;
+            if constexpr (PPI == 4) {
+              v = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)af[mt][t][d][q]);
+            } else if constexpr (PPI == 8) {  // instruction 0 for d < 2, instruction 1 for d >= 2
+              v = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)af[mt][t][d >> 1][q]);
+              v = c < 8 ? v : 0u;  // rows 8..15 were not loaded
+            } else {
+              v = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)af[mt][t][0][q]);
+              v = c < 4 ? v : 0u;
+            }
+            got[d][q] = v;
+          }
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) af[mt][t][d] = got[d];
+      }
   }
 
   uint16_t* out = static_cast<uint16_t*>(p.out);
@@ -250,8 +273,18 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 }
 
-#define KSQ_GO(MT, TPW, NB, NW) \
-  hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, MT, TPW, NB, NW>), grid, dim3(64 * NW), 0, s, a)
+#define KSQ_GO4(MT, TPW, NB, NW) \
+  hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, MT, TPW, NB, NW, 4>), grid, dim3(64 * NW), 0, s, a)
+// one row tile: the activation loads widen as the rows get fewer
+#define KSQ_GO(MT, TPW, NB, NW)                                                                                  \
+  do {                                                                                                           \
+    if (MT == 1 && a.M <= 4)                                                                                     \
+      hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, 1, TPW, NB, NW, 16>), grid, dim3(64 * NW), 0, s, a);         \
+    else if (MT == 1 && a.M <= 8)                                                                                \
+      hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, 1, TPW, NB, NW, 8>), grid, dim3(64 * NW), 0, s, a);          \
+    else                                                                                                         \
+      KSQ_GO4(MT, TPW, NB, NW);                                                                                  \
+  } while (0)
 template <typename T, int GPT>
 void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
   const int tpw = pl.tpw, nb = pl.nb;
@@ -272,23 +305,24 @@ void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
     }
   } else if (pl.mt == 2) {
     if (tpw <= 2) {
-      if (nb >= 2) KSQ_GO(2, 2, 2, 8);
-      else KSQ_GO(2, 2, 1, 8);
+      if (nb >= 2) KSQ_GO4(2, 2, 2, 8);
+      else KSQ_GO4(2, 2, 1, 8);
     } else {
-      if (nb >= 2) KSQ_GO(2, 4, 2, 8);
-      else KSQ_GO(2, 4, 1, 8);
+      if (nb >= 2) KSQ_GO4(2, 4, 2, 8);
+      else KSQ_GO4(2, 4, 1, 8);
     }
   } else {
     if (tpw <= 1) {
-      if (nb >= 2) KSQ_GO(4, 1, 2, 8);
-      else KSQ_GO(4, 1, 1, 8);
+      if (nb >= 2) KSQ_GO4(4, 1, 2, 8);
+      else KSQ_GO4(4, 1, 1, 8);
     } else {
-      if (nb >= 2) KSQ_GO(4, 2, 2, 8);
-      else KSQ_GO(4, 2, 1, 8);
+      if (nb >= 2) KSQ_GO4(4, 2, 2, 8);
+      else KSQ_GO4(4, 2, 1, 8);
     }
   }
 }
 #undef KSQ_GO
+#undef KSQ_GO4
 
 }  // namespace
 
