@@ -619,6 +619,15 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     const Fp8KstatPlan kp = fp8_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
     if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   }
+  // large m: the partial tiles of a split last round of 256 x 256 tiles; the plan depends on the number of 256-row
+  // blocks only
+  for (size_t mb = 1; mb <= (max_m + 255) / 256 && mb <= 64; ++mb) {
+    const size_t mm = mb * 256 < max_m ? mb * 256 : max_m;
+    if (mm > 128 && fp8_prefill_supported(mm, n, k)) {
+      const size_t need = fp8_prefill_workspace_bytes(mm, n, k, cus);
+      if (need > best) best = need;
+    }
+  }
   *bytes = best;
   return KSQ_OK;
 }
@@ -660,7 +669,7 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
   if (!di) return KSQ_ERR_HIP;
   if (fp8_prefill_supported(m, n, k) && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
     return fp8_launch_prefill(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
-                              static_cast<hipStream_t>(stream), epi);
+                              workspace, workspace ? workspace_bytes : 0, static_cast<hipStream_t>(stream), epi);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
   // split-K needs the stream's arrival counters; a stream that got none is planned as if it had no workspace
   if (workspace && !counter_slot_device_ptr(static_cast<hipStream_t>(stream))) workspace = nullptr;

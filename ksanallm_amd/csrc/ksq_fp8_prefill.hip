@@ -30,6 +30,11 @@ struct Fp8PrefillArgs {
   void* out;
   int M, N, K, KS /* 128-byte k stages */, mblocks, nblocks, super_n;
   int a_scale_per_row, w_scale_per_col;
+  // 256 x 256 kernel only: this launch covers the logical tile ids lid_begin .. of the whole grid; with ksplit > 1
+  // it is the launch for the tiles of a last, mostly empty round: K is split over grid.y and every split stores its
+  // raw fp32 tile to `partial` [split][tile - lid_begin][256][256] for fp8_tail_reduce_kernel
+  int lid_begin, ksplit, tail_tiles;
+  float* partial;
   Epilogue epi;
 };
 
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
 
   // super-tiles of 8 row blocks x 4 column blocks = the 32 workgroups resident on one XCD
   const int per_xcd = gridDim.x >> 3;
-  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int lid = p.lid_begin + (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   const int st = lid >> 5, rr0 = lid & 31;
   const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
   const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 4 + (rr0 >> 3);
@@ -312,14 +317,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
     }
   };
 
+  // k stages of this launch's split (all of them unless this is the tail launch)
+  const int s_begin = (int)(((long)p.KS * blockIdx.y) / p.ksplit), s_end = (int)(((long)p.KS * (blockIdx.y + 1)) / p.ksplit);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) load_item(lds_a0, lds_b0, 0, 0, i);
+  for (int i = 0; i < 4; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
 #pragma unroll
-  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b0, 0, 0, i);
+  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
 #pragma unroll
-  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b1, 0, 1, i);
-  int s = 0;
-  for (; s + 6 <= p.KS; s += 6) {
+  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b1, s_begin, s_begin + 1, i);
+  int s = s_begin;
+  for (; s + 6 <= s_end; s += 6) {
     step(lds_a0, lds_b0, lds_a1, lds_b2, s);
     step(lds_a1, lds_b1, lds_a0, lds_b0, s + 1);
     step(lds_a0, lds_b2, lds_a1, lds_b1, s + 2);
@@ -327,12 +334,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
     step(lds_a0, lds_b1, lds_a1, lds_b0, s + 4);
     step(lds_a1, lds_b2, lds_a0, lds_b1, s + 5);
   }
-  // the remaining zero to five stages, same rotation (their prefetches past K re-read the last stage)
-  if (s < p.KS) step(lds_a0, lds_b0, lds_a1, lds_b2, s);
-  if (s + 1 < p.KS) step(lds_a1, lds_b1, lds_a0, lds_b0, s + 1);
-  if (s + 2 < p.KS) step(lds_a0, lds_b2, lds_a1, lds_b1, s + 2);
-  if (s + 3 < p.KS) step(lds_a1, lds_b0, lds_a0, lds_b2, s + 3);
-  if (s + 4 < p.KS) step(lds_a0, lds_b1, lds_a1, lds_b0, s + 4);
+  // the remaining zero to five stages, same rotation (their prefetches past the end re-read a stage nobody uses)
+  if (s < s_end) step(lds_a0, lds_b0, lds_a1, lds_b2, s);
+  if (s + 1 < s_end) step(lds_a1, lds_b1, lds_a0, lds_b0, s + 1);
+  if (s + 2 < s_end) step(lds_a0, lds_b2, lds_a1, lds_b1, s + 2);
+  if (s + 3 < s_end) step(lds_a1, lds_b0, lds_a0, lds_b2, s + 3);
+  if (s + 4 < s_end) step(lds_a0, lds_b1, lds_a1, lds_b0, s + 4);
 
   // ---- epilogue: scales, then a transpose through LDS so that every lane stores 16 contiguous bytes
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
@@ -344,8 +351,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
   for (int t = 0; t < kNT; ++t) {
     const int col = nw + 16 * t + r;
-    ws[t] = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
+    ws[t] = p.ksplit > 1 ? 1.f : p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
   }
+  // split launch: the raw fp32 tile of this split, rows of 256 floats, for the reduction kernel
+  float* part = p.ksplit > 1 ? p.partial + ((size_t)blockIdx.y * p.tail_tiles + (lid - p.lid_begin)) * 65536 : nullptr;
 #pragma unroll
   for (int mt = 0; mt < kMT; ++mt) {
 #pragma unroll
@@ -358,6 +367,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
       const float* src = epi + rr * kEpiStride + cc;
       const int row = mw + 16 * mt + rr, col = nw + cc;
+      if (part) {
+        f32x4* dst = reinterpret_cast<f32x4*>(part + (128 * wm + 16 * mt + rr) * 256 + 64 * wn + cc);
+        dst[0] = f32x4{src[0], src[1], src[2], src[3]};
+        dst[1] = f32x4{src[4], src[5], src[6], src[7]};
+        continue;
+      }
       const float as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
       float vals[8];
 #pragma unroll
@@ -368,7 +383,72 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   }
 }
 
+// Second half of the split tail launch of the 256 x 256 kernel: one thread per eight consecutive columns of a tail
+// tile; adds the splits in order, applies the scales and the epilogue.
+template <typename T>
+__global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // [tail tile][256 rows][32 segments]
+  const int tile = (int)(idx >> 13), rr = (int)(idx >> 5) & 255, seg = (int)idx & 31;
+  if (tile >= p.tail_tiles) return;
+  const int lid = p.lid_begin + tile;
+  const int st = lid >> 5, rr0 = lid & 31;
+  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
+  const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 4 + (rr0 >> 3);
+  const int row = mb * 256 + rr, col = nb * 256 + seg * 8;
+  if (mb >= p.mblocks || nb >= p.nblocks || row >= p.M || col + 8 > p.N) return;
+  const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + (size_t)tile * 65536 + rr * 256 + seg * 8);
+  const size_t stride = (size_t)p.tail_tiles * 65536 / 4;
+  f32x4 lo = src[0], hi = src[1];
+  for (int sp = 1; sp < p.ksplit; ++sp) {
+    lo += src[sp * stride];
+    hi += src[sp * stride + 1];
+  }
+  const float as = p.a_scale[p.a_scale_per_row ? row : 0];
+  float vals[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const float w = p.w_scale[p.w_scale_per_col ? col + q : 0];
+    vals[q] = ((q < 4 ? lo[q] : hi[q - 4]) * w) * as;  // the order of the one-launch epilogue: column scale, then row scale
+  }
+  epi_store_row8<T>(p.epi, static_cast<uint16_t*>(p.out), vals, row, col, p.N);
+}
+
 }  // namespace
+
+// A grid of 256 x 256 tiles runs in rounds of one workgroup per CU.  When the last round is at most half full and K
+// is long, its tiles go out as a launch of their own with K split so that it fills the device: every split stores its
+// raw fp32 tile with plain stores and a reduction kernel finishes (the Qwen-72B qkv shape at M = 2048 is 320 tiles
+// on 256 CUs: a second round a quarter full).  Returns the split count (1 = no split) and the tiles in the tail.
+static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int* tail_super, size_t* need) {
+  *tail_super = 0;
+  *need = 0;
+  if (m <= 128) return 1;
+  const size_t mblocks = (m + 255) / 256, nblocks = (n + 255) / 256, super_n = (nblocks + 3) / 4;
+  const size_t supers = ((mblocks + 7) / 8) * super_n, per_round = (size_t)cus / 32;
+  if (per_round == 0 || supers <= per_round) return 1;  // a single round: nothing to even out
+  const size_t rem = supers % per_round;
+  // measured at the Qwen-72B shapes, M = 2048: qkv (one full round + a quarter) 194 -> 186 us; gate_up (seven rounds
+  // + a quarter) no gain, so grids of four rounds or more are left alone
+  if (rem == 0 || 2 * rem > per_round || k / 128 < 32 || supers >= 4 * per_round) return 1;
+  size_t ks = per_round / rem;
+  if (ks > 4) ks = 4;
+  if (const char* e = tuning_env("KSQ_FP8_TAIL_KSPLIT")) {  // tuning / test override (1 switches the split off)
+    const int v = atoi(e);
+    if (v >= 1 && v <= 8 && (size_t)v <= k / 128) ks = (size_t)v;
+  }
+  const size_t bytes = ks * rem * 32 * 65536 * 4;
+  if (ks <= 1 || bytes > workspace_bytes) return 1;
+  *tail_super = (int)rem;
+  *need = bytes;
+  return (int)ks;
+}
+
+size_t fp8_prefill_workspace_bytes(size_t m, size_t n, size_t k, int cus) {
+  int tail = 0;
+  size_t need = 0;
+  fp8_tail_split(m, n, k, cus, (size_t)-1, &tail, &need);
+  return need;
+}
 
 bool fp8_prefill_supported(size_t m, size_t n, size_t k) {
   return m >= 128 && n % 8 == 0 && k % 128 == 0 && m * k < 0x7FFFFF00ull && n * k < 0x7FFFFF00ull;
@@ -376,7 +456,7 @@ bool fp8_prefill_supported(size_t m, size_t n, size_t k) {
 
 int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                        const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
-                       hipStream_t s, const Epilogue& epi) {
+                       void* workspace, size_t workspace_bytes, hipStream_t s, const Epilogue& epi) {
   KSQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0, KSQ_ERR_INVALID_ARGUMENT, "output must be 16-byte aligned");
   Fp8PrefillArgs a{};
   a.epi = epi;
@@ -399,16 +479,42 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     const int v = atoi(e);
     if (v == 128 || v == 256) tile = v;
   }
+  a.lid_begin = 0;
+  a.ksplit = 1;
+  a.tail_tiles = 0;
+  a.partial = nullptr;
   if (tile == 256) {
     a.mblocks = (int)((m + 255) / 256);
     a.nblocks = (int)((n + 255) / 256);
     a.super_n = (a.nblocks + 3) / 4;
     const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 32;  // whole 8 x 4 super-tiles
     KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    const DeviceInfo* di = device_info();
+    KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
+    int tail_super = 0;
+    size_t need = 0;
+    const bool ws_ok = workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
+    const int ks = fp8_tail_split(m, n, k, di->cus, ws_ok ? workspace_bytes : 0, &tail_super, &need);
+    const size_t main_tiles = total - (size_t)tail_super * 32;
     if (out_dtype == KSQ_F16)
-      hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, dim3((unsigned)total), dim3(512), 0, s, a);
+      hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
     else
-      hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, dim3((unsigned)total), dim3(512), 0, s, a);
+      hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
+    if (ks > 1) {
+      Fp8PrefillArgs t = a;
+      t.lid_begin = (int)main_tiles;
+      t.ksplit = ks;
+      t.tail_tiles = tail_super * 32;
+      t.partial = static_cast<float*>(workspace);
+      const dim3 tgrid((unsigned)t.tail_tiles, (unsigned)ks), rgrid((unsigned)((size_t)t.tail_tiles * 8192 / 256));
+      if (out_dtype == KSQ_F16) {
+        hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, tgrid, dim3(512), 0, s, t);
+        hipLaunchKernelGGL(fp8_tail_reduce_kernel<_Float16>, rgrid, dim3(256), 0, s, t);
+      } else {
+        hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, tgrid, dim3(512), 0, s, t);
+        hipLaunchKernelGGL(fp8_tail_reduce_kernel<__bf16>, rgrid, dim3(256), 0, s, t);
+      }
+    }
   } else {
     a.mblocks = (int)((m + kBM - 1) / kBM);
     a.nblocks = (int)((n + kBN - 1) / kBN);

@@ -214,6 +214,34 @@ def test_gemm_large_m_both_tiles(gpu, tile, M, K, N):
     assert np.array_equal(got, got2)
 
 
+@pytest.mark.parametrize("ksplit", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,K,N", [(300, 4096, 9208), (2048, 4096, 9216)])
+def test_gemm_large_m_split_last_round(gpu, ksplit, M, K, N):
+    """Nine super-tiles of 256 x 256 tiles on a device whose round holds eight: the ninth goes out as a launch of its
+    own with K split (0 = the planner's own count, 1 = no split), partial tiles through the workspace, a reduction
+    kernel behind it.  Ragged M and N; twice, bit for bit; and without a workspace (no split)."""
+    import os
+
+    xq, xs, wq, ws = _fp8_case(450 + M, M, K, N)
+    old = os.environ.get("KSQ_FP8_TAIL_KSPLIT")
+    if ksplit:
+        os.environ["KSQ_FP8_TAIL_KSPLIT"] = str(ksplit)
+    try:
+        got = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+        got2 = _run_gemm(gpu, xq, xs, wq, ws, "bf16")
+    finally:
+        if old is None:
+            os.environ.pop("KSQ_FP8_TAIL_KSPLIT", None)
+        else:
+            os.environ["KSQ_FP8_TAIL_KSPLIT"] = old
+    rows = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(M).choice(M, size=40, replace=False)]))
+    want = orc.fp8_gemm(xq[rows], xs[rows], wq, ws)
+    orc.assert_parity(got[rows], want, f"fp8 tail split {ksplit} M={M} K={K} N={N}")
+    assert np.array_equal(got, got2)
+    got3 = _run_gemm(gpu, xq, xs, wq, ws, "bf16", use_workspace=False)
+    orc.assert_parity(got3[rows], want, f"fp8 no workspace M={M}")
+
+
 def test_gemm_large_m_small_integers_exact(gpu):
     rng = np.random.default_rng(420)
     M, K, N = 256, 384, 256
