@@ -266,6 +266,23 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
                     const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
                     int epilogue, const void* bias, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Per-token dynamic quantisation and the GEMM as one call: act is [m,k] T (not yet quantised), out is T,
+ *   scale[r] = max(absmax(act[r,:]) / 448, 1/(448*512)),  a_q = e4m3(clamp(act / scale[r], +-448)),
+ *   out[m,n] = T( (sum_k a_q[m,k] * w[n,k]) * w_scale[n or 0] * scale[m] ),
+ * i.e. ksq_fp8_quantize(KSQ_FP8_PER_TOKEN_DYNAMIC) followed by ksq_fp8_gemm_ex, which is what it runs for m > 1: one
+ * call for the reference's Fp8E4m3Quantize + Fp8QuantizedMatMul pair (KS/kernels/nvidia/kernel_wrapper.cpp:1015-1041,
+ * KS/layers/nvidia/fp8_matmul_layer.cpp:56-63).  A single token (k a multiple of 128, at most 8192) is one launch:
+ * every workgroup takes the row maximum and quantises the activations itself, with the same arithmetic, so the
+ * quantised bytes are those of ksq_fp8_quantize.  (Measured, that form only ties with the two launches at one row and
+ * loses from two rows on, since every workgroup repeats the quantisation; it can do up to eight rows.)  The workspace
+ * (ksq_fp8_gemm_dynamic_workspace_bytes, 256-byte aligned) holds the quantised activations and scales of the two-launch
+ * route and the split-K partial sums; without one only the single-launch case works, anything else fails with
+ * KSQ_ERR_WORKSPACE. */
+int ksq_fp8_gemm_dynamic_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
+int ksq_fp8_gemm_dynamic(int dtype, void* out, const void* act, const void* w_q, const float* w_scale,
+                         size_t w_scale_count, size_t m, size_t n, size_t k, int epilogue, const void* bias,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* out row 2i = in row i, out row 2i + 1 = in row rows/2 + i, for rows of row_bytes bytes (rows even, row_bytes a
  * multiple of 4; in and out must not overlap).  Load-time helper for the interleaved gate / up weight and its
  * per-channel scales (row_bytes = 4). */

@@ -29,7 +29,7 @@ EXPORTS = [
     "ksq_fp8_convert_weight_per_channel", "ksq_fp8_merge_qkv_scales", "ksq_fp8_workspace_bytes", "ksq_fp8_gemm",
     "ksq_w4a16_repack_ex", "ksq_w4a16_repack_ex_host", "ksq_gptq_act_order_perm", "ksq_permute_columns",
     "ksq_w4a16_workspace_bytes_ex", "ksq_w4a16_gemm_ex", "ksq_fp8_gemm_ex", "ksq_interleave_halves",
-    "ksq_w4a16_gemm_static_scratch",
+    "ksq_w4a16_gemm_static_scratch", "ksq_fp8_gemm_dynamic_workspace_bytes", "ksq_fp8_gemm_dynamic",
 ]
 STATIC_SCRATCH_BYTES = 64 << 20
 
@@ -76,6 +76,8 @@ def lib():
         L.ksq_fp8_gemm_ex.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
         L.ksq_interleave_halves.argtypes = [vp, vp, sz, sz, vp]
         L.ksq_w4a16_gemm_static_scratch.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp]
+        L.ksq_fp8_gemm_dynamic_workspace_bytes.argtypes = [sz, sz, sz, psz]
+        L.ksq_fp8_gemm_dynamic.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
         for name in EXPORTS:
             if name not in ("ksq_last_error_string",):
                 getattr(L, name).restype = ci
@@ -179,6 +181,18 @@ def w4a16_gemm(dtype, out, act, weight, sz, m, n, k, group_size, workspace=None,
 def w4a16_gemm_static_scratch(dtype, out, act, weight, sz, m, n, k, group_size, stream=None):
     _check(lib().ksq_w4a16_gemm_static_scratch(dtype, _addr(out), _addr(act), _addr(weight), _addr(sz), m, n, k,
                                                group_size, stream))
+
+
+def fp8_gemm_dynamic_workspace_bytes(max_m, n, k):
+    b = ctypes.c_size_t(0)
+    _check(lib().ksq_fp8_gemm_dynamic_workspace_bytes(max_m, n, k, ctypes.byref(b)))
+    return b.value
+
+
+def fp8_gemm_dynamic(dtype, out, act, w_q, w_scale, w_scale_count, m, n, k, epilogue=EPILOGUE_NONE, bias=None,
+                     workspace=None, workspace_bytes=0, stream=None):
+    _check(lib().ksq_fp8_gemm_dynamic(dtype, _addr(out), _addr(act), _addr(w_q), _addr(w_scale), w_scale_count, m, n, k,
+                                      epilogue, _addr(bias), _addr(workspace), workspace_bytes, stream))
 
 
 def fp8_quantize(dtype, act, m, k, mode, act_q, act_scale, stream=None):

@@ -2,17 +2,20 @@
 #include <cstdlib>
 
 #include "ksq_epilogue.h"
+#include "ksq_fp8_ops.h"
 #include "ksq_internal.h"
 
 namespace ksq {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-constexpr float kE4m3Max = 448.0f;
-constexpr float kMinScale = 1.0f / 448.0f / 512.0f;  // FP8_E4M3_MIN_SCALE of the reference
+using fp8ops::kE4m3Max;
+using fp8ops::kMinScale;
+using fp8ops::u32x2;
+using fp8ops::u32x4;
+using fp8ops::absmax8;
+using fp8ops::quantize8;
+using fp8ops::unpack8;
 
 template <typename T>
 __device__ inline float load_as_float(const uint16_t* p, size_t i);
@@ -103,38 +106,8 @@ __global__ __launch_bounds__(256) void quantize_per_token_kernel(const uint16_t*
   for (size_t i = threadIdx.x; i < k; i += 256) qr[i] = quantize_one(load_as_float<T>(xr, i), s);
 }
 
-// ---- vector forms (k a multiple of 8, 16-byte aligned rows): eight elements per lane and access
-template <typename T>
-__device__ inline void unpack8(u32x4 v, float (&f)[8]) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if constexpr (__is_same(T, _Float16)) {
-      f[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[i] & 0xFFFFu));
-      f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[i] >> 16));
-    } else {
-      f[2 * i] = __builtin_bit_cast(float, v[i] << 16);
-      f[2 * i + 1] = __builtin_bit_cast(float, v[i] & 0xFFFF0000u);
-    }
-  }
-}
-
-__device__ inline float absmax8(const float (&f)[8], float mx) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) mx = fmaxf(mx, fabsf(f[i]));
-  return mx;
-}
-
-__device__ inline u32x2 quantize8(const float (&f)[8], float scale) {
-  float c[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) c[i] = fminf(fmaxf(f[i] / scale, -kE4m3Max), kE4m3Max);
-  int lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
-  lo = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], lo, true);
-  int hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[4], c[5], 0, false);
-  hi = __builtin_amdgcn_cvt_pk_fp8_f32(c[6], c[7], hi, true);
-  return u32x2{(uint32_t)lo, (uint32_t)hi};
-}
-
+// ---- vector forms (k a multiple of 8, 16-byte aligned rows): eight elements per lane and access; unpack8, absmax8 and
+// quantize8 live in ksq_fp8_ops.h
 template <int THREADS>
 __device__ inline float block_max(float v, float* smem) {
 #pragma unroll
@@ -630,6 +603,70 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
   }
   *bytes = best;
   return KSQ_OK;
+}
+
+// front part of the workspace of ksq_fp8_gemm_dynamic: e4m3 activations and one scale per row, each rounded up to 256
+static size_t dynamic_front_bytes(size_t m, size_t k) { return (m * k + 255) / 256 * 256 + (m * 4 + 255) / 256 * 256; }
+
+int ksq_fp8_gemm_dynamic_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
+  int rc = ksq_fp8_workspace_bytes(max_m, n, k, bytes);
+  if (rc != KSQ_OK) return rc;
+  *bytes = (*bytes + 255) / 256 * 256 + dynamic_front_bytes(max_m, k);
+  return KSQ_OK;
+}
+
+int ksq_fp8_gemm_dynamic(int dtype, void* out, const void* act, const void* w_q, const float* w_scale,
+                         size_t w_scale_count, size_t m, size_t n, size_t k, int epilogue, const void* bias,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(out && act && w_q && w_scale, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
+              "bad epilogue %d", epilogue);
+  KSQ_REQUIRE(epilogue != KSQ_EPILOGUE_BIAS || (bias && (reinterpret_cast<uintptr_t>(bias) & 15) == 0),
+              KSQ_ERR_INVALID_ARGUMENT, "the bias epilogue needs a 16-byte aligned bias");
+  KSQ_REQUIRE(epilogue != KSQ_EPILOGUE_SILU_MUL || n % 16 == 0, KSQ_ERR_UNSUPPORTED,
+              "the SiLU-mul epilogue needs n %% 16 == 0 (got %zu)", n);
+  int rc = check_fp8_shape(n, k);
+  if (rc != KSQ_OK) return rc;
+  if (m == 0) return KSQ_OK;
+  KSQ_REQUIRE(w_scale_count == 1 || w_scale_count == n, KSQ_ERR_INVALID_ARGUMENT,
+              "w_scale_count must be 1 or n (got %zu)", w_scale_count);
+  KSQ_REQUIRE((reinterpret_cast<uintptr_t>(act) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_q) & 15) == 0,
+              KSQ_ERR_INVALID_ARGUMENT, "act and w_q must be 16-byte aligned");
+  const DeviceInfo* di = device_info();
+  if (!di) return KSQ_ERR_HIP;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) workspace = nullptr;
+  if (!workspace) workspace_bytes = 0;
+  const size_t front = dynamic_front_bytes(m, k);
+  char* gemm_ws = workspace_bytes > front ? static_cast<char*>(workspace) + front : nullptr;
+  size_t gemm_ws_bytes = gemm_ws ? workspace_bytes - front : 0;
+  // One launch instead of two: the kernel that takes the row maxima and quantises its share of the activations itself.
+  // Every one of its workgroups repeats that work, so it only ties with the two launches at a single row without a
+  // split of K (Qwen-72B qkv: 22.2 us against 3.0 + 19.3) and loses beyond (two rows 23.5 against 22.5, eight rows
+  // 29.9 against 23.6; K = 29568, split four ways: 65.9 against 59.3): it serves m = 1, and up to eight rows on request.
+  const char* sw = tuning_env("KSQ_FP8_FUSED_QUANT");  // tuning / test switch: 0 = never, 1 = up to eight rows
+  const size_t fused_rows = sw ? (atoi(sw) == 0 ? 0 : 8) : 1;
+  if (m <= fused_rows && k % 128 == 0 && m * k * 2 < 0x7FFFFF00ull) {
+    if (gemm_ws && !counter_slot_device_ptr(s)) gemm_ws = nullptr, gemm_ws_bytes = 0;
+    const Fp8KstatPlan kp = fp8_kstat_plan(m, n, k, di->cus, gemm_ws_bytes, true);
+    if (kp.ok && kp.nb <= 2 && kp.tpw <= 4 && (kp.ksplit == 1 || sw)) {
+      Epilogue epi;
+      epi.kind = epilogue;
+      epi.bias = bias;
+      return fp8_launch_kstat(dtype, kp, out, nullptr, nullptr, m, w_q, w_scale, w_scale_count, m, n, k, gemm_ws, s, epi,
+                              act);
+    }
+  }
+  // Otherwise: quantise into the front of the workspace, then the GEMM.
+  KSQ_REQUIRE(workspace_bytes >= front, KSQ_ERR_WORKSPACE,
+              "m=%zu k=%zu needs %zu bytes of 256-byte aligned workspace for the quantised activations", m, k, front);
+  void* act_q = workspace;
+  float* act_scale = reinterpret_cast<float*>(static_cast<char*>(workspace) + (m * k + 255) / 256 * 256);
+  rc = ksq_fp8_quantize(dtype, act, m, k, KSQ_FP8_PER_TOKEN_DYNAMIC, act_q, act_scale, stream);
+  if (rc != KSQ_OK) return rc;
+  return ksq_fp8_gemm_ex(dtype, out, act_q, act_scale, m, w_q, w_scale, w_scale_count, m, n, k, epilogue, bias, gemm_ws,
+                         gemm_ws_bytes, stream);
 }
 
 int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,

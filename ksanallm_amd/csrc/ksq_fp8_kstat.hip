@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "ksq_epilogue.h"
+#include "ksq_fp8_ops.h"
 #include "ksq_internal.h"
 
 namespace ksq {
@@ -23,6 +24,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 struct Fp8KstatArgs {
+  const uint16_t* a_src;  // fused quantisation: the activations [M][K] as T, M <= 8; aq and a_scale are then unused
   const uint8_t* aq;  // [M][K]
   const uint8_t* wq;  // [N][K]
   const float* a_scale;
@@ -53,11 +55,22 @@ __device__ inline i32x8 join(u32x4 lo, u32x4 hi) {
   return v;
 }
 
-template <typename T, int MT, int TPW, int NB, int NW>
+// FUSED: the kernel quantises its own activations (per token: one scale per row, Fp8E4m3Quantize of the reference
+// with num_channels = m) instead of reading e4m3 bytes and scales: every workgroup takes the row maxima over the
+// whole K, quantises the k range it works on into LDS -- the same arithmetic as the quantisation kernel, so the
+// bytes are the same -- and its waves read their operand fragments from there.  Up to eight rows.
+constexpr int kFusedRows = 8;
+constexpr int kFusedRowBytes = 64 * 128 + 16;  // 64 stages per workgroup at most; 16 bytes of padding spread the banks
+
+template <typename T, int MT, int TPW, int NB, int NW, bool FUSED>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4))) void fp8_kstat_kernel(Fp8KstatArgs p) {
   constexpr int D = NB * TPW;  // ring depth = one batch
   static_assert(NB * MT * NW <= 64 && NB * MT <= NW, "two reduction buffers of at most 64 KiB, one tile per wave");
+  static_assert(!FUSED || (MT == 1 && NB <= 2 && NW == 16 && TPW <= 4), "fused quantisation: one row tile, 64 KiB of LDS left");
   __shared__ f32x4 red[2 * NB * MT * NW * 64];
+  __shared__ __attribute__((aligned(16))) uint8_t aq_lds[FUSED ? kFusedRows * kFusedRowBytes : 16];
+  __shared__ float row_part[FUSED ? kFusedRows * NW : 1];
+  __shared__ float row_scale[FUSED ? kFusedRows : 1];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -115,19 +128,56 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
 
   // activation fragments of this wave's stages: registers for the whole kernel
   i32x8 af[MT][TPW];
+  if constexpr (!FUSED) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < TPW; ++t) {
-      const int row = 16 * mt + lr;
-      u32x4 piece[2];
+      for (int t = 0; t < TPW; ++t) {
+        const int row = 16 * mt + lr;
+        u32x4 piece[2];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const unsigned ao = (row < p.M && k_off[t][h] != 0x80000000u) ? (unsigned)row * p.K + k_off[t][h] : 0x80000000u;
-        piece[h] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+        for (int h = 0; h < 2; ++h) {
+          const unsigned ao = (row < p.M && k_off[t][h] != 0x80000000u) ? (unsigned)row * p.K + k_off[t][h] : 0x80000000u;
+          piece[h] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+        }
+        af[mt][t] = join(piece[0], piece[1]);
       }
-      af[mt][t] = join(piece[0], piece[1]);
+  }
+
+  // Fused quantisation, first half (before the weight stream starts, so that these loads are not queued behind
+  // it): row maxima over the whole K.  Every thread takes one 16-byte chunk of each row per round, all rows' loads
+  // of a round in flight together; rows past M cost no instruction.
+  constexpr int TH = 64 * NW;
+  const int tid = threadIdx.x;
+  const __amdgpu_buffer_rsrc_t rs_src = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(FUSED ? p.a_src : nullptr), 0, FUSED ? (int)((size_t)p.M * p.K * 2) : 0, 0x00020000);
+  const int chunks = p.K / 8;  // per row
+  u32x4 v[FUSED ? kFusedRows : 1];
+  float mx[FUSED ? kFusedRows : 1];
+  if constexpr (FUSED) {
+#pragma unroll
+    for (int row = 0; row < kFusedRows; ++row) {
+      mx[row] = 0.f;
+      v[row] = u32x4{0u, 0u, 0u, 0u};
     }
+    for (int base = 0; base < chunks; base += TH) {
+      const int ch = base + tid;
+#pragma unroll
+      for (int row = 0; row < kFusedRows; ++row)
+        if (row < p.M) {
+          const unsigned off = ch < chunks ? ((unsigned)row * p.K + (unsigned)ch * 8u) * 2u : 0x80000000u;
+          v[row] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_src, off, 0, 0));
+        }
+      if (base + TH < chunks) {  // more rounds follow: fold this one in now (the last round's chunks stay in v)
+#pragma unroll
+        for (int row = 0; row < kFusedRows; ++row) {
+          float f[8];
+          fp8ops::unpack8<T>(v[row], f);
+          mx[row] = fp8ops::absmax8(f, mx[row]);
+        }
+      }
+    }
+  }
 
   u32x4 wq[D][2];
   auto fetch = [&](int slot, int i /* column tile inside the workgroup */, int t) {
@@ -144,18 +194,71 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
     __builtin_amdgcn_sched_barrier(0);
   }
 
+  if constexpr (!FUSED) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) {
+        u32x4 lo, hi;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          lo[q] = (uint32_t)af[mt][t][q];
+          hi[q] = (uint32_t)af[mt][t][4 + q];
+        }
+        af[mt][t] = to_operand(lo, hi);
+      }
+  } else {
+    // ---- second half: the weight stream is under way.  Fold the last round of chunks in, reduce over the workgroup.
+#pragma unroll
+    for (int row = 0; row < kFusedRows; ++row) {
+      float f[8];
+      fp8ops::unpack8<T>(v[row], f);
+      mx[row] = fp8ops::absmax8(f, mx[row]);
+    }
+#pragma unroll
+    for (int row = 0; row < kFusedRows; ++row) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) mx[row] = fmaxf(mx[row], __shfl_xor(mx[row], off));
+      if (lane == 0) row_part[row * NW + wave] = mx[row];
+    }
+    __syncthreads();
+    if (tid < kFusedRows) {
+      float m = row_part[tid * NW];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) m = fmaxf(m, row_part[tid * NW + w]);
+      row_scale[tid] = fmaxf(m / fp8ops::kE4m3Max, fp8ops::kMinScale);
+    }
+    __syncthreads();
+    // ---- quantise the k range of this workgroup into LDS: one chunk per thread and row (at most 64 stages = 1024
+    // chunks).  With one split and a row of at most 1024 chunks the registers still hold exactly these chunks.
+    const int kw0 = wg_begin * 16, kwn = (wg_end - wg_begin) * 16;  // first chunk and chunk count of the range
+    if (!(p.ksplit == 1 && chunks <= TH)) {
+#pragma unroll
+      for (int row = 0; row < kFusedRows; ++row)
+        if (row < p.M) {
+          const unsigned off = tid < kwn ? ((unsigned)row * p.K + (unsigned)(kw0 + tid) * 8u) * 2u : 0x80000000u;
+          v[row] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_src, off, 0, 0));
+        }
+    }
+#pragma unroll
+    for (int row = 0; row < kFusedRows; ++row)
+      if (row < p.M) {  // uniform: rows past M cost nothing (the division is the expensive part)
+        float f[8];
+        fp8ops::unpack8<T>(v[row], f);
+        const fp8ops::u32x2 q = fp8ops::quantize8(f, row_scale[row]);
+        if (tid < kwn) *reinterpret_cast<fp8ops::u32x2*>(aq_lds + row * kFusedRowBytes + tid * 8) = q;
+      }
+    __syncthreads();
+    // ---- operand fragments straight from LDS: lane (r, j) takes bytes [16j, 16j+16) and [64+16j, ..) of row r
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
-      u32x4 lo, hi;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        lo[q] = (uint32_t)af[mt][t][q];
-        hi[q] = (uint32_t)af[mt][t][4 + q];
-      }
-      af[mt][t] = to_operand(lo, hi);
+      const bool ok = r < p.M && s0 + t < wg_end;
+      const uint8_t* src = aq_lds + (r & (kFusedRows - 1)) * kFusedRowBytes + (ok ? (s0 + t - wg_begin) * 128 : 0) + 16 * j;
+      u32x4 lo = *reinterpret_cast<const u32x4*>(src), hi = *reinterpret_cast<const u32x4*>(src + 64);
+      if (!ok) lo = hi = u32x4{0u, 0u, 0u, 0u};
+      af[0][t] = join(lo, hi);
     }
+  }
 
   uint16_t* out = static_cast<uint16_t*>(p.out);
   for (int b = 0; b < nbatches; ++b) {
@@ -220,7 +323,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int row = row0 + e;
-          sum[e] = sum[e] * ws * p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
+          float as;
+          if constexpr (FUSED) as = row_scale[row < p.M ? row : 0];
+          else as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
+          sum[e] = sum[e] * ws * as;
         }
         epi_store_acc<T>(p.epi, out, sum, row0, col, p.M, p.N, col < p.N);
       }
@@ -228,7 +334,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 }
 
-#define KSQ_GO(MT, TPW, NB, NW) hipLaunchKernelGGL((fp8_kstat_kernel<T, MT, TPW, NB, NW>), grid, dim3(64 * NW), 0, s, a)
+#define KSQ_GO(MT, TPW, NB, NW) hipLaunchKernelGGL((fp8_kstat_kernel<T, MT, TPW, NB, NW, false>), grid, dim3(64 * NW), 0, s, a)
+#define KSQ_GO_FUSED(TPW, NB) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, TPW, NB, 16, true>), grid, dim3(1024), 0, s, a)
+template <typename T>
+bool launch_fused(int tpw, int nb, const Fp8KstatArgs& a, dim3 grid, hipStream_t s) {
+  if (tpw == 4 && nb == 1) KSQ_GO_FUSED(4, 1);
+  else if (tpw == 4 && nb == 2) KSQ_GO_FUSED(4, 2);
+  else if (tpw == 2 && nb == 1) KSQ_GO_FUSED(2, 1);
+  else if (tpw == 2 && nb == 2) KSQ_GO_FUSED(2, 2);
+  else if (tpw == 1 && nb == 1) KSQ_GO_FUSED(1, 1);
+  else if (tpw == 1 && nb == 2) KSQ_GO_FUSED(1, 2);
+  else return false;
+  return true;
+}
+#undef KSQ_GO_FUSED
+
 template <typename T>
 void launch(int mt, int tpw, int nb, const Fp8KstatArgs& a, dim3 grid, hipStream_t s) {
   if (mt == 1 && tpw == 8) {
@@ -274,7 +394,7 @@ void launch(int mt, int tpw, int nb, const Fp8KstatArgs& a, dim3 grid, hipStream
 // Plan: row tiles (1, 2 or 4), waves per workgroup (8 with four row tiles or one row tile and a long K, else 16),
 // stages per wave (1, 2, 4 or 8; at most 2 with two row tiles: the activations of waves x TPW stages live in
 // registers), split count, column tiles per workgroup and per batch.
-Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, bool fused) {
   Fp8KstatPlan p{};
   const size_t ntiles = (n + 15) / 16, stages = (k + 127) / 128;
   p.ok = m >= 1 && m <= 64 && ntiles * 4 <= (size_t)kCountersPerSlot && m * k < 0x7FFFFF00ull;
@@ -285,6 +405,7 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
   // flight per CU (measured at K = 29568: 15 % faster; no gain for K <= 8192).
   bool wide = p.mt == 1 && stages > 64;
   if (const char* e = tuning_env("KSQ_FP8_WIDE")) wide = atoi(e) != 0 && p.mt == 1;  // tuning / test override
+  if (fused) wide = false;  // the kernel that quantises its own activations: 16 waves, LDS for two column tiles a batch
   const size_t nw = (p.mt == 4 || wide) ? 8 : 16;
   const size_t cap = nw * (wide ? 8u : (p.mt == 2 ? 2u : 4u));
   size_t ksplit = (stages + cap - 1) / cap;
@@ -320,17 +441,22 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
     if (v == 1 || v == 2 || (v == 4 && p.mt == 1 && p.tpw < 4)) p.nb = v;
     if (wide && p.nb > 2) p.nb = 2;
   }
+  if (fused && p.nb > 2) p.nb = 2;
   p.partial_bytes = need(ksplit);
   return p;
 }
 
 int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const void* act_q, const float* act_scale,
                      size_t act_scale_count, const void* w_q, const float* w_scale, size_t w_scale_count, size_t m,
-                     size_t n, size_t k, void* workspace, hipStream_t s, const Epilogue& epi) {
+                     size_t n, size_t k, void* workspace, hipStream_t s, const Epilogue& epi, const void* act_src) {
   KSQ_REQUIRE(((size_t)plan.nt_per_wg + 8) * 16 * k < 0x3FFFFF00ull, KSQ_ERR_UNSUPPORTED,
               "column range of one workgroup larger than 1 GiB");
+  KSQ_REQUIRE(act_src == nullptr || (m <= (size_t)kFusedRows && k % 128 == 0 && plan.mt == 1 && plan.nb <= 2 &&
+                                     plan.tpw <= 4 && m * k * 2 < 0x7FFFFF00ull),
+              KSQ_ERR_UNSUPPORTED, "fused activation quantisation: at most %d rows, k a multiple of 128", kFusedRows);
   Fp8KstatArgs a{};
   a.epi = epi;
+  a.a_src = static_cast<const uint16_t*>(act_src);
   a.aq = static_cast<const uint8_t*>(act_q);
   a.wq = static_cast<const uint8_t*>(w_q);
   a.a_scale = act_scale;
@@ -353,8 +479,16 @@ int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const v
     KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
-  if (out_dtype == KSQ_F16) launch<_Float16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
-  else launch<__bf16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
+  if (act_src != nullptr) {
+    const bool ok = out_dtype == KSQ_F16 ? launch_fused<_Float16>(plan.tpw, plan.nb, a, grid, s)
+                                         : launch_fused<__bf16>(plan.tpw, plan.nb, a, grid, s);
+    KSQ_REQUIRE(ok, KSQ_ERR_UNSUPPORTED, "no fused kernel for %d stages per wave, %d column tiles per batch", plan.tpw,
+                plan.nb);
+  } else if (out_dtype == KSQ_F16) {
+    launch<_Float16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
+  } else {
+    launch<__bf16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
+  }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

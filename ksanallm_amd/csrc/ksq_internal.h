@@ -174,10 +174,14 @@ struct Fp8KstatPlan {
   int nb;         // column tiles per batch
   size_t partial_bytes;
 };
-Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+// `fused`: plan for the kernel that quantises its own activations (m <= 8)
+Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, bool fused = false);
+// act_src != nullptr: the activations as 16-bit elements of the output type, quantised per token inside the kernel
+// (act_q / act_scale unused); needs a plan made with `fused`
 int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const void* act_q, const float* act_scale,
                      size_t act_scale_count, const void* w_q, const float* w_scale, size_t w_scale_count, size_t m,
-                     size_t n, size_t k, void* workspace, hipStream_t s, const Epilogue& epi = Epilogue());
+                     size_t n, size_t k, void* workspace, hipStream_t s, const Epilogue& epi = Epilogue(),
+                     const void* act_src = nullptr);
 
 struct Fp8Plan {
   int MT;

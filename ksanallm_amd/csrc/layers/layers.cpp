@@ -255,7 +255,7 @@ size_t Fp8MatMulLayer<T>::GetWorkSpaceSize(const int m, const int k) {
   size_t input_size = (size_t)m * k * GetTypeSize(TYPE_FP8_E4M3);
   input_size = (input_size + 15) / 16 * 16;
   size_t scale_size = (size_t)m * GetTypeSize(TYPE_FP32);
-  return input_size + scale_size + kFp8GemmWorkspaceBytes;
+  return input_size + scale_size + kFp8GemmWorkspaceBytes + 512;  // + the slack of two 256-byte roundings
 }
 
 template <typename T>
@@ -297,9 +297,16 @@ Status Fp8MatMulLayer<T>::Forward(const std::vector<Tensor>& input_tensors, std:
     input_scale = input_tensors[1].input_scales->GetPtr<float>();
     ThrowOnKsqError(ksq_fp8_quantize(KsqDtype<T>(), input, m, k, KSQ_FP8_PER_TENSOR_STATIC, input_quant, input_scale,
                                      stream), "ksq_fp8_quantize");
+  } else if (weight_scale_count > 1) {
+    // per-channel weight scales go with per-token activation scales: quantisation and GEMM as one call (a single
+    // launch for decode batches of up to eight tokens); the call carves the same buffer up itself
+    ThrowOnKsqError(ksq_fp8_gemm_dynamic(KsqDtype<T>(), output, input, weight_quant, weight_scale, weight_scale_count, m,
+                                         n, k, epilogue_, bias_ ? bias_->GetPtr<void>() : nullptr, gemm_workspace,
+                                         workspace_buffer_->GetTotalBytes(), stream), "ksq_fp8_gemm_dynamic");
+    return Status();
   } else {
     input_scale = reinterpret_cast<float*>(input_quant + quant_bytes);
-    const bool per_token = weight_scale_count > 1;
+    const bool per_token = false;
     input_scale_count = per_token ? m : 1;
     ThrowOnKsqError(ksq_fp8_quantize(KsqDtype<T>(), input, m, k,
                                      per_token ? KSQ_FP8_PER_TOKEN_DYNAMIC : KSQ_FP8_PER_TENSOR_DYNAMIC, input_quant,

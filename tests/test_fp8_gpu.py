@@ -355,3 +355,127 @@ def test_merge_qkv_scales(gpu):
         part = _run_gemm(gpu, xq, xs, np.ascontiguousarray(wq[row:row + rows]), sc, "f16")
         assert np.array_equal(fused[:, row:row + rows], part)
         row += rows
+
+
+def _run_dynamic(gpu, x_bits, wq, w_scale, dtype, use_workspace=True, epilogue=0, bias_bits=None):
+    """ksq_fp8_gemm_dynamic on activations given as 16-bit patterns of `dtype`."""
+    import torch
+
+    from ksanallm_amd import capi
+
+    M, K = x_bits.shape
+    N = wq.shape[0]
+    dx = _upload_bits(x_bits, dtype, gpu)
+    dw, dws = torch.from_numpy(wq).to(gpu), torch.from_numpy(w_scale).to(gpu)
+    cols = N // 2 if epilogue == capi.EPILOGUE_SILU_MUL else N
+    out = torch.full((M, cols), float("nan"), dtype=torch_dtype(dtype), device=gpu)
+    wsb = capi.fp8_gemm_dynamic_workspace_bytes(M, N, K) if use_workspace else 0
+    ws = torch.empty(max(wsb, 256), dtype=torch.uint8, device=gpu)
+    bias = _upload_bits(bias_bits, dtype, gpu) if bias_bits is not None else None
+    capi.fp8_gemm_dynamic(capi_dtype(dtype), out, dx, dw, dws, w_scale.size, M, N, K, epilogue, bias,
+                          ws if use_workspace else None, wsb)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8, 9, 40])
+@pytest.mark.parametrize("K,N", [(1024, 272), (8192, 528), (9600, 1040), (4096, 4112)])
+def test_gemm_dynamic_quantises_inside(gpu, dtype, M, K, N):
+    """Per-token quantisation folded into the GEMM (one launch up to eight rows, two beyond): parity against the
+    oracle's quantise-then-GEMM, agreement with the library's own two calls, twice bit for bit; K = 9600 is split over
+    workgroups, N = 4112 gives a workgroup several batches."""
+    import os
+
+    rng = np.random.default_rng(460 + M + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    ws = orc.fp8_compute_scale(w, orc.F32, N, K)
+    wq = orc.fp8_quantize(w, orc.F32, ws, N, K)
+    xv = rng.standard_normal((M, K)).astype(np.float32) * np.exp2(rng.integers(-6, 7, size=(M, 1))).astype(np.float32)
+    x = orc.to_bits(xv, ORC_DT[dtype])
+    os.environ["KSQ_FP8_FUSED_QUANT"] = "1"  # the single-launch form for every m <= 8 (by default it serves m = 1 only)
+    try:
+        got = _run_dynamic(gpu, x, wq, ws, dtype)
+        got2 = _run_dynamic(gpu, x, wq, ws, dtype)
+        got3 = _run_dynamic(gpu, x, wq, ws, dtype, use_workspace=False) if M <= 8 and K <= 8192 else None
+    finally:
+        os.environ.pop("KSQ_FP8_FUSED_QUANT", None)
+    xs = orc.fp8_compute_scale(x, ORC_DT[dtype], M, K)
+    xq = orc.fp8_quantize(x, ORC_DT[dtype], xs, M, K)
+    want = orc.fp8_gemm(xq, xs, wq, ws)
+    orc.assert_parity(got.float().cpu().numpy(), want, f"fp8 dynamic M={M} K={K} N={N} {dtype}")
+    assert np.array_equal(bits_of(got), bits_of(got2))
+    two = _run_gemm(gpu, xq, xs, wq, ws, dtype).astype(np.float64)
+    diff = np.abs(got.float().cpu().numpy().astype(np.float64) - two)
+    assert np.all(diff <= 2.0 ** -7 * np.maximum(np.abs(two), 1e-6)), "differs from quantise + GEMM by more than an output ulp"
+    if got3 is not None:  # no workspace: still one launch (a longer K is split over workgroups and needs one)
+        orc.assert_parity(got3.float().cpu().numpy(), want, f"fp8 dynamic, no workspace M={M}")
+    dflt = _run_dynamic(gpu, x, wq, ws, dtype)  # the default route choice
+    orc.assert_parity(dflt.float().cpu().numpy(), want, f"fp8 dynamic default route M={M}")
+    os.environ["KSQ_FP8_FUSED_QUANT"] = "0"
+    try:
+        got4 = _run_dynamic(gpu, x, wq, ws, dtype)
+    finally:
+        os.environ.pop("KSQ_FP8_FUSED_QUANT", None)
+    assert np.array_equal(got4.float().cpu().numpy().astype(np.float64), two), "two-launch route must equal the two calls"
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("M", [1, 4, 8])
+def test_gemm_dynamic_quantiser_is_the_quantise_kernels(gpu, dtype, M):
+    """An identity weight (e4m3 1.0 on the diagonal, scale 1) turns the GEMM into out[m, k] = T(float(q[m, k]) * scale[m]):
+    the quantised bytes and scales inside the fused kernel, compared exactly with the oracle's."""
+    K = N = 1024
+    rng = np.random.default_rng(470 + M)
+    xv = rng.standard_normal((M, K)).astype(np.float32) * np.exp2(rng.integers(-10, 11, size=(M, 1))).astype(np.float32)
+    xv[0, :5] = [0.0, -0.0, 1e-30, -3.0e4 if dtype == "f16" else -3.0e30, 7.5]
+    x = orc.to_bits(xv, ORC_DT[dtype])
+    wq = np.zeros((N, K), dtype=np.uint8)
+    wq[np.arange(N), np.arange(N)] = orc.e4m3_encode(np.array([1.0], dtype=np.float32))[0]
+    import os
+
+    os.environ["KSQ_FP8_FUSED_QUANT"] = "1"
+    try:
+        got = _run_dynamic(gpu, x, wq, np.ones(1, dtype=np.float32), dtype)
+    finally:
+        os.environ.pop("KSQ_FP8_FUSED_QUANT", None)
+    xs = orc.fp8_compute_scale(x, ORC_DT[dtype], M, K)
+    xq = orc.fp8_quantize(x, ORC_DT[dtype], xs, M, K)
+    want = orc.e4m3_decode(xq) * xs[:, None]
+    gb, wb = bits_of(got), orc.to_bits(want.astype(np.float32), ORC_DT[dtype])
+    same = (gb == wb) | (((gb & 0x7FFF) == 0) & ((wb & 0x7FFF) == 0))  # the sign of zero is not significant
+    assert np.all(same)
+
+
+def test_gemm_dynamic_epilogues_and_errors(gpu):
+    import torch
+
+    from ksanallm_amd import capi
+
+    rng = np.random.default_rng(480)
+    M, K, N = 4, 1024, 256
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    ws = orc.fp8_compute_scale(w, orc.F32, N, K)
+    wq = orc.fp8_quantize(w, orc.F32, ws, N, K)
+    x = orc.to_bits(rng.standard_normal((M, K)).astype(np.float32), orc.BF16)
+    xs = orc.fp8_compute_scale(x, orc.BF16, M, K)
+    xq = orc.fp8_quantize(x, orc.BF16, xs, M, K)
+    acc = orc.fp8_gemm(xq, xs, wq, ws)
+    bias = orc.to_bits(rng.standard_normal(N).astype(np.float32), orc.BF16)
+    import os
+
+    os.environ["KSQ_FP8_FUSED_QUANT"] = "1"
+    got = _run_dynamic(gpu, x, wq, ws, "bf16", epilogue=capi.EPILOGUE_BIAS, bias_bits=bias)
+    orc.assert_parity(got.float().cpu().numpy(), acc + orc.from_bits(bias, orc.BF16)[None, :], "fp8 dynamic + bias")
+    # rows [gate ; up] interleaved gate / up (what ksq_interleave_halves builds): row 2i = gate i, row 2i + 1 = up i
+    il = np.empty_like(wq)
+    il[0::2], il[1::2] = wq[: N // 2], wq[N // 2:]
+    ils = np.empty_like(ws)
+    ils[0::2], ils[1::2] = ws[: N // 2], ws[N // 2:]
+    got = _run_dynamic(gpu, x, il, ils, "bf16", epilogue=capi.EPILOGUE_SILU_MUL)
+    orc.assert_parity(got.float().cpu().numpy(), orc.silu_mul(acc), "fp8 dynamic + SiLU-mul")
+    os.environ.pop("KSQ_FP8_FUSED_QUANT", None)
+    big = orc.to_bits(rng.standard_normal((12, K)).astype(np.float32), orc.BF16)
+    with pytest.raises(capi.KsqError) as e:
+        _run_dynamic(gpu, big, wq, ws, "bf16", use_workspace=False)
+    assert e.value.code == capi.ERR_WORKSPACE
