@@ -122,9 +122,10 @@ int ksq_device_compute_units(void);
  * (KS/models/quant/quant_weight.cpp:331-346, 577-579; LK/asymmetric_gemm/cutlass_preprocessors.cpp:466-508)
  * and the scale / zero binding of ConvertGroupTensor (quant_weight.cpp:530-536, 632-636).
  *
- * Output "fragment order" (K % 128 == 0, N % 16 == 0, g in {64,128}; the reference's kernels take K % 64 == 0,
- * LK/asymmetric_gemm/fpA_intB_gemm/fpA_intB_gemm_template.h:168-171: a K that is an odd multiple of 64 is refused
- * here with KSQ_ERR_UNSUPPORTED):
+ * Output "fragment order" (N % 16 == 0, g in {64,128}, K a whole number of groups -- with g = 64 that includes the odd
+ * multiples of 64 that the reference's kernels take, LK/asymmetric_gemm/fpA_intB_gemm/fpA_intB_gemm_template.h:168-171;
+ * such a K is padded to whole 128-row tiles here: the rows past K hold u = z = 8 under a zero scale, the sizes below
+ * count them, and the GEMM pads the activation rows to match in its workspace, so such a K needs a workspace):
  *   weight : K*N/2 bytes = tiles [N/16][K/128] of 1024 B.  Tile (nt,kt) is 64 lanes x 16 B; lane l = 16*j + c
  *            owns column n = 16*nt + c; 32-bit word d (0..3) of the lane covers k = 128*kt + 32*d + 8*j + e,
  *            e = 0..7, with element e in nibble e/2 when e is even and nibble 4 + e/2 when e is odd; nibbles are

@@ -206,7 +206,7 @@ static int check_w4_shape(size_t k, size_t n, size_t g) {
   // the reference kernels accept group sizes 64 and 128 only (LK/asymmetric_gemm/fpA_intB_gemm/
   // fpA_intB_gemm_template.h:130) and k % 64 == 0 (:168-171); the fragment order needs whole 128 x 16 tiles
   KSQ_REQUIRE(g == 64 || g == 128, KSQ_ERR_UNSUPPORTED, "group size %zu not supported (64 or 128)", g);
-  KSQ_REQUIRE(k % kTileK == 0, KSQ_ERR_UNSUPPORTED, "k=%zu must be a multiple of %d", k, kTileK);
+  KSQ_REQUIRE(k % g == 0, KSQ_ERR_UNSUPPORTED, "k=%zu must be a multiple of the group size %zu", k, g);
   KSQ_REQUIRE(n % kTileN == 0, KSQ_ERR_UNSUPPORTED, "n=%zu must be a multiple of %d", n, kTileN);
   KSQ_REQUIRE(k < (1u << 30) && n < (1u << 30), KSQ_ERR_UNSUPPORTED, "k or n too large");
   return KSQ_OK;
@@ -216,14 +216,25 @@ int ksq_w4a16_repack_sizes(size_t k, size_t n, size_t g, size_t* weight_bytes, s
   int rc = check_w4_shape(k, n, g);
   if (rc != KSQ_OK) return rc;
   KSQ_REQUIRE(weight_bytes && sz_bytes, KSQ_ERR_INVALID_ARGUMENT, "null output pointer");
-  *weight_bytes = k * n / 2;
-  *sz_bytes = (k / g) * n * 4;
+  const size_t kp = (k + kTileK - 1) / kTileK * kTileK;  // an odd multiple of 64 (g = 64) is padded to whole k tiles
+  *weight_bytes = kp * n / 2;
+  *sz_bytes = (kp / g) * n * 4;
   return KSQ_OK;
+}
+
+// the copy of the activations with rows padded to whole k tiles, in front of the workspace, when k % 128 == 64
+static size_t padded_act_bytes(size_t m, size_t k) {
+  return k % kTileK == 0 ? 0 : (m * (k + 64) * 2 + 255) / 256 * 256;
 }
 
 int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
   KSQ_REQUIRE(bytes, KSQ_ERR_INVALID_ARGUMENT, "null output pointer");
   KSQ_REQUIRE(max_m > 0, KSQ_ERR_INVALID_ARGUMENT, "max_m must be positive");
+  if (k % kTileK == 64) {  // group size 64: planned on the padded K, plus the padded copy of the activations
+    int rcp = ksq_w4a16_workspace_bytes(max_m, n, k + 64, bytes);
+    if (rcp == KSQ_OK) *bytes += padded_act_bytes(max_m, k);
+    return rcp;
+  }
   int rc = check_w4_shape(k, n, 128);
   if (rc != KSQ_OK) return rc;
   const DeviceInfo* di = device_info();
@@ -286,6 +297,22 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) workspace = nullptr;
   if (!workspace) workspace_bytes = 0;
+  if (k % kTileK != 0) {
+    // K an odd multiple of 64 (group size 64): the repacked weight has a last k tile whose upper half is padding; the
+    // activations get rows of k + 64 elements with zeros behind the data, in front of the workspace
+    KSQ_REQUIRE(act_perm == nullptr, KSQ_ERR_UNSUPPORTED, "act_perm needs k %% 128 == 0 (got %zu)", k);
+    const size_t need = padded_act_bytes(m, k);
+    KSQ_REQUIRE(workspace_bytes >= need, KSQ_ERR_WORKSPACE,
+                "k=%zu is not a multiple of 128: %zu bytes of 256-byte aligned workspace are needed for the padded "
+                "activations", k, need);
+    rc = pad_rows(workspace, act, m, k, k + 64, s);
+    if (rc != KSQ_OK) return rc;
+    act = workspace;
+    workspace = static_cast<char*>(workspace) + need;
+    workspace_bytes -= need;
+    if (workspace_bytes == 0) workspace = nullptr;
+    k += 64;
+  }
   if (act_perm) {
     const size_t need = (m * k * 2 + 255) / 256 * 256;
     KSQ_REQUIRE(workspace_bytes >= need, KSQ_ERR_WORKSPACE,

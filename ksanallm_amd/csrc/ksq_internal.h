@@ -95,6 +95,9 @@ __device__ inline ksq_f32x4 load_agent(const ksq_f32x4* p) {
 }
 #endif
 
+// out [m][k_out] = in [m][k_in] followed by zeros, 16-bit elements, k_in and k_out multiples of 8 (ksq_repack.hip)
+int pad_rows(void* out, const void* in, size_t m, size_t k_in, size_t k_out, hipStream_t s);
+
 struct DeviceInfo {
   int cus;
 };

@@ -13,7 +13,9 @@ struct RepackArgs {
   const void* scales;
   uint32_t* dst_weight;
   uint32_t* dst_sz;
-  size_t K, N, g;
+  size_t K, N, g;  // K = rows of the source tensors
+  size_t Kp;       // rows of the destination: K rounded up to whole 128-row tiles (the rows past K hold u = z = 8
+                   // under a zero scale, and the GEMM gives them zero activations)
   int layout, zero_kind, scale_dtype;
   const int32_t* row_perm;  // destination row i holds source row row_perm[i]; null = identity
   int column_order;
@@ -131,9 +133,10 @@ __host__ __device__ inline uint32_t source_nibble(const RepackArgs& a, size_t k,
 
 __host__ __device__ inline uint32_t build_weight_word(const RepackArgs& a, size_t word) {
   size_t k0, n;
-  frag_word_origin(word, a.K, &k0, &n);
+  frag_word_origin(word, a.Kp, &k0, &n);
   n = source_column(a, n);
   uint32_t out = 0;
+  if (k0 >= a.K) return 0x88888888u;  // padding rows (eight rows at a time: K is a multiple of 64)
   if (a.row_perm) {
     for (int e = 0; e < 8; ++e) {
       size_t kr = (size_t)(uint32_t)a.row_perm[k0 + e];
@@ -153,11 +156,13 @@ __host__ __device__ inline uint32_t build_weight_word(const RepackArgs& a, size_
 }
 
 __host__ __device__ inline uint32_t build_sz_word(const RepackArgs& a, size_t idx) {
-  // idx enumerates [N/16][G][16]
-  const size_t G = a.K / a.g;
+  // idx enumerates [N/16][G][16], G counted over the padded rows
+  const size_t G = a.Kp / a.g;
   size_t c = idx & 15, rest = idx >> 4;
   size_t gi = rest % G, nt = rest / G;
   size_t n = source_column(a, nt * kTileN + c);
+  const bool padding = gi >= a.K / a.g;
+  if (padding) gi = 0;  // the padding group: zero scale, z = 8, the column's exponent field like every other word
   // Marlin keeps scales (and zero points) permuted inside blocks of 64 columns, or of 32 when there is a single
   // group (MarlinPermuteScales, KS/models/quant/quant_weight.cpp:350-375): entry p of a block is column
   // p / 8 + 8 * (p % 8), resp. 2 * (p / 8) + {0,1,8,9,16,17,24,25}[p % 8]
@@ -173,6 +178,7 @@ __host__ __device__ inline uint32_t build_sz_word(const RepackArgs& a, size_t id
   }
   uint16_t sbits = static_cast<const uint16_t*>(a.scales)[gi * a.N + ns];
   uint32_t z = 8;
+  if (padding) return (8u << 16) | ((uint32_t)(uint8_t)(int8_t)column_exponent(a, ns) << 24);
   switch (a.zero_kind) {
     case KSQ_ZERO_AWQ_INT32: {
       uint32_t w = static_cast<const uint32_t*>(a.zeros)[gi * (a.N >> 3) + (n >> 3)];
@@ -254,6 +260,7 @@ RepackArgs make_args(int layout, const void* qweight, int zero_kind, const void*
   a.dst_weight = static_cast<uint32_t*>(dst_weight);
   a.dst_sz = static_cast<uint32_t*>(dst_sz);
   a.K = k;
+  a.Kp = (k + kTileK - 1) / kTileK * kTileK;
   a.N = n;
   a.g = g;
   a.layout = layout;
@@ -262,6 +269,22 @@ RepackArgs make_args(int layout, const void* qweight, int zero_kind, const void*
   a.row_perm = row_perm;
   a.column_order = column_order;
   return a;
+}
+
+// out [m][k_out] = in [m][k_in] then zeros: one thread per eight destination elements
+__global__ __launch_bounds__(256) void pad_rows_kernel(uint32_t* out, const uint32_t* in, size_t m, size_t k_in,
+                                                       size_t k_out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t per_row = k_out / 8;
+  if (i >= m * per_row) return;
+  const size_t row = i / per_row, c = i - row * per_row;
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (c * 8 < k_in) {
+    const uint32_t* src = in + (row * k_in + c * 8) / 2;
+    for (int q = 0; q < 4; ++q) w[q] = src[q];
+  }
+  uint32_t* dst = out + (row * k_out + c * 8) / 2;
+  for (int q = 0; q < 4; ++q) dst[q] = w[q];
 }
 
 // out[m, i] = in[m, perm[i]]: one thread per eight destination elements (16 bytes stored)
@@ -309,10 +332,19 @@ extern "C" int ksq_w4a16_repack_ex(int layout, const void* qweight, int zero_kin
   RepackArgs a = make_args(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, row_perm, column_order,
                            dst_weight, dst_sz);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const size_t words = k * n / 8, count = (k / g) * n;
+  const size_t words = a.Kp * n / 8, count = (a.Kp / g) * n;
   KSQ_REQUIRE((words + 255) / 256 < (1ull << 31), KSQ_ERR_UNSUPPORTED, "tensor too large for one launch");
   hipLaunchKernelGGL(repack_weight_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, s, a, words);
   hipLaunchKernelGGL(repack_sz_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, a, count);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+int ksq::pad_rows(void* out, const void* in, size_t m, size_t k_in, size_t k_out, hipStream_t s) {
+  const size_t threads = m * (k_out / 8);
+  KSQ_REQUIRE((threads + 255) / 256 < (1ull << 31), KSQ_ERR_UNSUPPORTED, "tensor too large for one launch");
+  hipLaunchKernelGGL(pad_rows_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                     static_cast<uint32_t*>(out), static_cast<const uint32_t*>(in), m, k_in, k_out);
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }
@@ -335,7 +367,7 @@ extern "C" int ksq_w4a16_repack_ex_host(int layout, const void* qweight, int zer
                   "row_perm[%zu] = %d is outside [0, %zu)", i, row_perm[i], k);
   RepackArgs a = make_args(layout, qweight, zero_kind, zeros, scales, scale_dtype, k, n, g, row_perm, column_order,
                            dst_weight, dst_sz);
-  const size_t words = k * n / 8, count = (k / g) * n;
+  const size_t words = a.Kp * n / 8, count = (a.Kp / g) * n;
   std::vector<int8_t> col_exp;
   if (scale_dtype == KSQ_BF16) {
     col_exp.resize(n);

@@ -80,6 +80,8 @@ template <typename T, DataType WT>
 size_t GroupMatMulLayer<T, WT>::GetWorkSpaceSize() {
   if constexpr (WT == TYPE_I4_GROUP) {
     size_t bytes = 0;
+    // the kernels take whole groups (and the reference k % 64 == 0: fpA_intB_gemm_template.h:168-171)
+    if (groupsize_ == 0 || max_k_ % groupsize_ != 0) KLLM_THROW("GroupMatMulLayer: k is not a multiple of the group size.");
     ThrowOnKsqError(ksq_w4a16_workspace_bytes_ex(max_m_, max_n_, max_k_, is_gptq_desc_ ? 1 : 0, &bytes),
                     "ksq_w4a16_workspace_bytes_ex");
     return bytes;

@@ -293,7 +293,7 @@ static int RunErrors() {
     std::vector<Tensor> outs = {o};
     l->Forward({a, w}, outs);
   });
-  Expect("k not a multiple of 128 is refused", true, [&] {
+  Expect("k not a whole number of groups is refused", true, [&] {
     std::vector<std::any> p = good;
     p[6] = size_t(192);
     factory.Make(TYPE_I4_GROUP, TYPE_FP16, p);

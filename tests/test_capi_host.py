@@ -127,9 +127,10 @@ def test_sizes_and_argument_validation():
     with pytest.raises(capi.KsqError) as ei:  # the reference kernels also refuse other group sizes
         capi.w4a16_gemm(capi.F16, buf, buf, buf, buf, 1, 16, 128, 32)
     assert ei.value.code == capi.ERR_UNSUPPORTED
-    with pytest.raises(capi.KsqError) as ei:  # k not a multiple of the tile
-        capi.w4a16_gemm(capi.F16, buf, buf, buf, buf, 1, 16, 192, 64)
-    assert ei.value.code == capi.ERR_UNSUPPORTED
+    for k, g in ((192, 128), (160, 64)):  # k not a whole number of groups
+        with pytest.raises(capi.KsqError) as ei:
+            capi.w4a16_gemm(capi.F16, buf, buf, buf, buf, 1, 16, k, g)
+        assert ei.value.code == capi.ERR_UNSUPPORTED
     with pytest.raises(capi.KsqError) as ei:  # bad dtype
         capi.w4a16_gemm(7, buf, buf, buf, buf, 1, 16, 128, 128)
     assert ei.value.code == capi.ERR_INVALID_ARGUMENT
@@ -164,3 +165,27 @@ def test_workspace_sizes_are_monotone_and_bounded():
         # per compute unit (64 x 256 fp32 each)
         assert w4096 <= max(w64, 4096 * k * 2 + 4096 * 4 + 512 + 2 * 256 * 64 * 256 * 4)
     assert capi.fp8_workspace_bytes(64, 8192, 8192) <= 8192 * 8192
+
+
+def test_host_repack_pads_a_k_that_is_an_odd_multiple_of_64():
+    """Group size 64 admits K = 64 * odd (the reference's k % 64 == 0): the destination has whole 128-row tiles, the
+    rows past K hold nibble 8 and their group's words a zero scale with z = 8, everything else is the ordinary repack."""
+    rng = np.random.default_rng(33)
+    K, N, g = 192, 32, 64
+    Kp = 256
+    u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8)
+    s = orc.to_bits(np.abs(rng.standard_normal((K // g, N))) * 0.02 + 1e-3, orc.F16)
+    assert capi.w4a16_repack_sizes(K, N, g) == (Kp * N // 2, (Kp // g) * N * 4)
+    dw = np.zeros(Kp * N // 8, dtype=np.uint32)
+    dsz = np.zeros((Kp // g) * N, dtype=np.uint32)
+    capi.w4a16_repack_host(capi.W4_AWQ_INT32_NPACK, orc.awq_pack(u), capi.ZERO_AWQ_INT32, orc.awq_pack(z), s, capi.F16,
+                           K, N, g, dw, dsz)
+    upad = np.concatenate([u, np.full((Kp - K, N), 8, dtype=np.uint8)])
+    assert np.array_equal(dw, _expected_words(upad))
+    szw = dsz.reshape(N // 16, Kp // g, 16).transpose(1, 0, 2).reshape(Kp // g, N)
+    assert np.array_equal((szw[: K // g] & 0xFFFF).astype(np.uint16), s)
+    assert np.array_equal(((szw[: K // g] >> 16) & 0xFF).astype(np.uint8), z)
+    assert np.all(szw[K // g:] == (8 << 16))
+    with pytest.raises(capi.KsqError):
+        capi.w4a16_repack_sizes(192, N, 128)   # group size 128 needs whole groups

@@ -312,6 +312,27 @@ def test_bf16_scales_far_outside_the_fp16_range(gpu, M):
         orc.assert_parity(got[:, cols], want[:, cols], f"M={M} column block {b} (scale ~ {base[0, b * N // 8]:g})")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("kind", ["awq", "gptq"])
+@pytest.mark.parametrize("M,K,N", [(1, 192, 272), (16, 1088, 528), (40, 448, 1040), (100, 1088, 272), (600, 704, 512)])
+def test_k_odd_multiple_of_64(gpu, dtype, kind, M, K, N):
+    """Group size 64 with K = 64 * odd, which the reference's kernels accept (k % 64 == 0): the repack pads the last
+    k tile, the GEMM pads the activation rows in its workspace; every kernel family by M; without a workspace the
+    call must refuse."""
+    from ksanallm_amd import capi
+
+    case = W4Case(1500 + M + K, M, K, N, g=64, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    assert dev.workspace_bytes >= M * (K + 64) * 2
+    got1 = dev.gemm_f32()
+    got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"K={K} g=64 {kind} {dtype} M={M}")
+    assert np.array_equal(got1, got2)
+    with pytest.raises(capi.KsqError) as e:
+        dev.gemm(use_workspace=False)
+    assert e.value.code == capi.ERR_WORKSPACE
+
+
 def test_no_workspace_still_correct(gpu):
     case = W4Case(1300, 16, 4096, 512, kind="gptq", dtype="f16")
     dev = W4Device(case, gpu)
