@@ -96,11 +96,15 @@ def e4m3_encode(x, table):
     return code | np.where(np.signbit(x), 0x80, 0).astype(np.uint8)
 
 
-def w4a16_case(seed, M, K, N, g, awq, bf16):
+def w4a16_case(seed, M, K, N, g, awq, bf16, column_exponents=0):
+    """column_exponents = e > 0 multiplies every column's scales by 2^j, j drawn per column from [-e, e]: bf16 scales
+    that no fp16 holds, with the spread inside a column (about 2^6) left as it is."""
     rng = np.random.default_rng(seed)
     u = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
     z = rng.integers(0, 16, size=(K // g, N), dtype=np.uint8) if awq else np.full((K // g, N), 8, dtype=np.uint8)
     s = np.abs(rng.standard_normal((K // g, N))).astype(np.float32) * 0.02 + 1e-3
+    if column_exponents:
+        s = s * np.exp2(rng.integers(-column_exponents, column_exponents + 1, size=N)).astype(np.float32)[None, :]
     a = rng.standard_normal((M, K)).astype(np.float32)
     to_bits, to_val = (bf16_bits, bf16_value) if bf16 else (f16_bits, f16_value)
     sb, ab = to_bits(s), to_bits(a)
@@ -211,6 +215,11 @@ def main():
     np.savez_compressed(os.path.join(HERE, "w4a16_awq_f16_5x256x64_g64.npz"), **w4a16_case(2, 5, 256, 64, 64, True, False))
     np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_16x384x128.npz"), **w4a16_case(3, 16, 384, 128, 128, True, True))
     np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_130x256x272.npz"), **w4a16_case(4, 130, 256, 272, 128, True, True))
+
+    # K an odd multiple of 64 (group size 64), and bf16 scales spread over 2^-40 .. 2^40 from column to column
+    np.savez_compressed(os.path.join(HERE, "w4a16_gptq_f16_7x192x64_g64.npz"), **w4a16_case(6, 7, 192, 64, 64, False, False))
+    np.savez_compressed(os.path.join(HERE, "w4a16_awq_bf16_9x256x64_wide.npz"),
+                        **w4a16_case(7, 9, 256, 64, 128, True, True, column_exponents=40))
 
     np.savez_compressed(os.path.join(HERE, "w4a16_next_f16_12x256x128.npz"), **next_case(5, 12, 256, 128, 128))
 

@@ -167,6 +167,18 @@ def test_workspace_sizes_are_monotone_and_bounded():
     assert capi.fp8_workspace_bytes(64, 8192, 8192) <= 8192 * 8192
 
 
+def test_workspace_sizes_of_padded_k_and_split_last_round():
+    """What the planners add to the workspace, computed on the host alone (256 compute units when no device is there):
+    the padded copy of the activation rows when K is an odd multiple of 64, and the fp32 partial tiles of a large-M FP8
+    GEMM whose last round of 256 x 256 tiles is at most half full (Qwen-72B qkv at M = 2048: 40 + 40 + ... = 320 tiles
+    on 256 units, so 64 tiles x 4 splits x 256 KiB); the self-quantising entry point adds the FP8 rows and scales."""
+    assert capi.w4a16_workspace_bytes(16, 64, 192) == capi.w4a16_workspace_bytes(16, 64, 256) + 16 * 256 * 2
+    assert capi.fp8_workspace_bytes(2048, 10240, 8192) == 64 * 4 * 256 * 256 * 4
+    assert capi.fp8_workspace_bytes(2048, 8192, 8192) < 64 * 4 * 256 * 256 * 4      # 256 tiles: one full round
+    front = capi.fp8_gemm_dynamic_workspace_bytes(2048, 10240, 8192) - capi.fp8_workspace_bytes(2048, 10240, 8192)
+    assert 2048 * 8192 + 2048 * 4 <= front <= 2048 * 8192 + 2048 * 4 + 1024
+
+
 def test_host_repack_pads_a_k_that_is_an_odd_multiple_of_64():
     """Group size 64 admits K = 64 * odd (the reference's k % 64 == 0): the destination has whole 128-row tiles, the
     rows past K hold nibble 8 and their group's words a zero scale with z = 8, everything else is the ordinary repack."""

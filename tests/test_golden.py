@@ -9,7 +9,7 @@ from oracle import oracle as orc
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 W4_CASES = ["w4a16_gptq_f16_16x256x128", "w4a16_awq_f16_5x256x64_g64", "w4a16_awq_bf16_16x384x128",
-            "w4a16_awq_bf16_130x256x272"]
+            "w4a16_awq_bf16_130x256x272", "w4a16_gptq_f16_7x192x64_g64", "w4a16_awq_bf16_9x256x64_wide"]
 
 
 def load(name):

@@ -44,6 +44,8 @@ def test_w4a16_golden(gpu, name):
     wsb = capi.w4a16_workspace_bytes(M, N, K)
     ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=gpu)
     for use_ws in (True, False):
+        if not use_ws and K % 128:
+            continue  # the padded copy of the activation rows lives in the workspace
         out = torch.full((M, N), float("nan"), dtype=tdt, device=gpu)
         capi.w4a16_gemm(cdt, out, act, weight, sz, M, N, K, g, ws if use_ws else None, wsb if use_ws else 0)
         torch.cuda.synchronize()
