@@ -382,13 +382,8 @@ __global__ __launch_bounds__(256) void fp8_stream_kernel(Fp8Args p) {
   };
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) store_agent(p.partial + pidx(split, mt), acc[mt]);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores are acknowledged
   unsigned* ctr = p.counters + (size_t)mblock * p.ntiles + nt;
-  unsigned arrived = 0;
-  if (lane == 0) arrived = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  arrived = __builtin_amdgcn_readfirstlane(arrived);
-  if (arrived != (unsigned)(p.ksplit - 1)) return;
-  asm volatile("" ::: "memory");
+  if (!splitk_arrive_last(ctr, lane, p.ksplit)) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};

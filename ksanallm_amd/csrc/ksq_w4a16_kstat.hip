@@ -255,14 +255,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
         const size_t stride = (size_t)p.ntiles * MT * 64;
         const size_t tile = ((size_t)nt * MT + mt) * 64 + lane;
         store_agent(p.partial + (size_t)split * stride + tile, sum);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         unsigned* counter = p.counters + nt * MT + mt;
-        unsigned arrived = 0;
-        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        arrived = __builtin_amdgcn_readfirstlane(arrived);
-        store = arrived == (unsigned)(p.ksplit - 1);
+        store = splitk_arrive_last(counter, lane, p.ksplit);
         if (store) {
-          asm volatile("" ::: "memory");
           sum = f32x4{0.f, 0.f, 0.f, 0.f};
           for (int sp = 0; sp < p.ksplit; ++sp) sum += load_agent(p.partial + (size_t)sp * stride + tile);
           if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

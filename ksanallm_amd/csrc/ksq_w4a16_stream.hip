@@ -304,13 +304,8 @@ w4a16_stream_kernel(StreamArgs p) {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
       if (tile_ok[t]) store_agent(p.partial + pidx(split, mt, t), acc[mt][t]);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores are acknowledged
   unsigned* ctr = p.counters + (size_t)mblock * p.ngroups + grp;
-  unsigned arrived = 0;
-  if (lane == 0) arrived = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  arrived = __builtin_amdgcn_readfirstlane(arrived);
-  if (arrived != (unsigned)(p.ksplit - 1)) return;
-  asm volatile("" ::: "memory");
+  if (!splitk_arrive_last(ctr, lane, p.ksplit)) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
