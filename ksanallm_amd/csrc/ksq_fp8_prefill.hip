@@ -28,7 +28,7 @@ struct Fp8PrefillArgs {
   const float* a_scale;
   const float* w_scale;
   void* out;
-  int M, N, K, KS /* 128-byte k stages */, mblocks, nblocks, super_n;
+  int M, N, K, KS /* 128-byte k stages */, mblocks, nblocks;
   int a_scale_per_row, w_scale_per_col;
   // 256 x 256 kernel only: this launch covers the logical tile ids lid_begin .. of the whole grid; with ksplit > 1
   // it is the launch for the tiles of a last, mostly empty round: K is split over grid.y and every split stores its
@@ -72,14 +72,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, j = lane >> 4;
 
-  // Hardware hands consecutive workgroup ids to the 8 XCDs in turn; every XCD (own L2) gets a contiguous run of
-  // logical ids, which walk 8 x 8 super-tiles of (row block, column block) pairs.
-  const int per_xcd = gridDim.x >> 3;
-  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int st = lid >> 6, rr0 = lid & 63;
-  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
-  const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 8 + (rr0 >> 3);
-  if (mb >= p.mblocks || nb >= p.nblocks) return;
+  int mb, nb;
+  if (!tile_of(tile_logical_id(blockIdx.x, gridDim.x), p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
   const int m0 = mb * kBM, n0 = nb * kBN + wave * (kNT * 16);
 
   const __amdgpu_buffer_rsrc_t rs_a =
@@ -229,13 +223,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   const int wm = wave >> 2, wn = wave & 3;
   const int r = lane & 15, j = lane >> 4;
 
-  // super-tiles of 8 row blocks x 4 column blocks = the 32 workgroups resident on one XCD
-  const int per_xcd = gridDim.x >> 3;
-  const int lid = p.lid_begin + (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int st = lid >> 5, rr0 = lid & 31;
-  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
-  const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 4 + (rr0 >> 3);
-  if (mb >= p.mblocks || nb >= p.nblocks) return;
+  // this launch covers the logical tile ids lid_begin .. lid_begin + gridDim.x - 1 of the whole grid
+  const int lid = p.lid_begin + tile_logical_id(blockIdx.x, gridDim.x);
+  int mb, nb;
+  if (!tile_of(lid, p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
   const int m0 = mb * 256, n0 = nb * 256;
 
   const __amdgpu_buffer_rsrc_t rs_a =
@@ -390,12 +381,10 @@ __global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) 
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;  // [tail tile][256 rows][32 segments]
   const int tile = (int)(idx >> 13), rr = (int)(idx >> 5) & 255, seg = (int)idx & 31;
   if (tile >= p.tail_tiles) return;
-  const int lid = p.lid_begin + tile;
-  const int st = lid >> 5, rr0 = lid & 31;
-  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
-  const int mb = st_m * 8 + (rr0 & 7), nb = st_n * 4 + (rr0 >> 3);
+  int mb, nb;
+  if (!tile_of(p.lid_begin + tile, p.mblocks, p.nblocks, &mb, &nb)) return;
   const int row = mb * 256 + rr, col = nb * 256 + seg * 8;
-  if (mb >= p.mblocks || nb >= p.nblocks || row >= p.M || col + 8 > p.N) return;
+  if (row >= p.M || col + 8 > p.N) return;
   const f32x4* src = reinterpret_cast<const f32x4*>(p.partial + (size_t)tile * 65536 + rr * 256 + seg * 8);
   const size_t stride = (size_t)p.tail_tiles * 65536 / 4;
   f32x4 lo = src[0], hi = src[1];
@@ -419,26 +408,25 @@ __global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) 
 // is long, its tiles go out as a launch of their own with K split so that it fills the device: every split stores its
 // raw fp32 tile with plain stores and a reduction kernel finishes (the Qwen-72B qkv shape at M = 2048 is 320 tiles
 // on 256 CUs: a second round a quarter full).  Returns the split count (1 = no split) and the tiles in the tail.
-static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int* tail_super, size_t* need) {
-  *tail_super = 0;
+static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int* tail_tiles, size_t* need) {
+  *tail_tiles = 0;
   *need = 0;
-  if (m <= 128) return 1;
-  const size_t mblocks = (m + 255) / 256, nblocks = (n + 255) / 256, super_n = (nblocks + 3) / 4;
-  const size_t supers = ((mblocks + 7) / 8) * super_n, per_round = (size_t)cus / 32;
-  if (per_round == 0 || supers <= per_round) return 1;  // a single round: nothing to even out
-  const size_t rem = supers % per_round;
+  if (m <= 128 || cus <= 0 || cus % 8 != 0) return 1;  // the main launch's tile count has to stay a multiple of eight
+  const size_t total = ((m + 255) / 256) * ((n + 255) / 256), per_round = (size_t)cus;
+  if (total <= per_round) return 1;  // a single round: nothing to even out
+  const size_t rem = total % per_round;
   // measured at the Qwen-72B shapes, M = 2048: qkv (one full round + a quarter) 194 -> 186 us; gate_up (seven rounds
   // + a quarter) no gain, so grids of four rounds or more are left alone
-  if (rem == 0 || 2 * rem > per_round || k / 128 < 32 || supers >= 4 * per_round) return 1;
+  if (rem == 0 || 2 * rem > per_round || k / 128 < 32 || total >= 4 * per_round) return 1;
   size_t ks = per_round / rem;
   if (ks > 4) ks = 4;
   if (const char* e = tuning_env("KSQ_FP8_TAIL_KSPLIT")) {  // tuning / test override (1 switches the split off)
     const int v = atoi(e);
     if (v >= 1 && v <= 8 && (size_t)v <= k / 128) ks = (size_t)v;
   }
-  const size_t bytes = ks * rem * 32 * 65536 * 4;
+  const size_t bytes = ks * rem * 65536 * 4;
   if (ks <= 1 || bytes > workspace_bytes) return 1;
-  *tail_super = (int)rem;
+  *tail_tiles = (int)rem;
   *need = bytes;
   return (int)ks;
 }
@@ -486,16 +474,17 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
   if (tile == 256) {
     a.mblocks = (int)((m + 255) / 256);
     a.nblocks = (int)((n + 255) / 256);
-    a.super_n = (a.nblocks + 3) / 4;
-    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 32;  // whole 8 x 4 super-tiles
-    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    const size_t total = (size_t)a.mblocks * a.nblocks;
+    KSQ_REQUIRE(total < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
     const DeviceInfo* di = device_info();
     KSQ_REQUIRE(di != nullptr, KSQ_ERR_HIP, "no device");
-    int tail_super = 0;
+    int tail_tiles = 0;
     size_t need = 0;
     const bool ws_ok = workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
-    const int ks = fp8_tail_split(m, n, k, di->cus, ws_ok ? workspace_bytes : 0, &tail_super, &need);
-    const size_t main_tiles = total - (size_t)tail_super * 32;
+    const int ks = fp8_tail_split(m, n, k, di->cus, ws_ok ? workspace_bytes : 0, &tail_tiles, &need);
+    // without a tail launch the one launch covers everything, rounded up to a multiple of eight; with one, the main
+    // launch covers whole rounds (a multiple of eight by itself)
+    const size_t main_tiles = ks > 1 ? total - (size_t)tail_tiles : tile_grid(a.mblocks, a.nblocks);
     if (out_dtype == KSQ_F16)
       hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
     else
@@ -504,9 +493,9 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
       Fp8PrefillArgs t = a;
       t.lid_begin = (int)main_tiles;
       t.ksplit = ks;
-      t.tail_tiles = tail_super * 32;
+      t.tail_tiles = tail_tiles;
       t.partial = static_cast<float*>(workspace);
-      const dim3 tgrid((unsigned)t.tail_tiles, (unsigned)ks), rgrid((unsigned)((size_t)t.tail_tiles * 8192 / 256));
+      const dim3 tgrid((unsigned)((tail_tiles + 7) / 8 * 8), (unsigned)ks), rgrid((unsigned)((size_t)tail_tiles * 8192 / 256));
       if (out_dtype == KSQ_F16) {
         hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, tgrid, dim3(512), 0, s, t);
         hipLaunchKernelGGL(fp8_tail_reduce_kernel<_Float16>, rgrid, dim3(256), 0, s, t);
@@ -518,13 +507,12 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
   } else {
     a.mblocks = (int)((m + kBM - 1) / kBM);
     a.nblocks = (int)((n + kBN - 1) / kBN);
-    a.super_n = (a.nblocks + 7) / 8;
-    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
-    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
+    KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
+    const dim3 grid(tile_grid(a.mblocks, a.nblocks));
     if (out_dtype == KSQ_F16)
-      hipLaunchKernelGGL(fp8_prefill_kernel<_Float16>, dim3((unsigned)total), dim3(256), 0, s, a);
+      hipLaunchKernelGGL(fp8_prefill_kernel<_Float16>, grid, dim3(256), 0, s, a);
     else
-      hipLaunchKernelGGL(fp8_prefill_kernel<__bf16>, dim3((unsigned)total), dim3(256), 0, s, a);
+      hipLaunchKernelGGL(fp8_prefill_kernel<__bf16>, grid, dim3(256), 0, s, a);
   }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;

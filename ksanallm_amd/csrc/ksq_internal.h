@@ -113,6 +113,29 @@ __device__ inline bool splitk_arrive_last(unsigned* counter, int lane, int kspli
 }
 #endif
 
+// ---- workgroup id -> output tile, for the kernels that tile the whole [M, N] output ------------------------------
+// A grid of mblocks x nblocks tiles is launched as exactly that many workgroups, rounded up to a multiple of eight:
+// no workgroup is launched only to find that it has no tile (a regular pattern of such workgroups -- seven of eight
+// with one row block padded to a band of eight -- was measured to leave seven of eight compute units without work,
+// because consecutive workgroups go to consecutive compute units).  Hardware hands consecutive workgroup ids to the
+// 8 XCDs in turn; every XCD (own L2) gets a contiguous run of logical ids.  Logical ids walk bands of eight row
+// blocks, column block by column block and down the band's row blocks first (the last band is as high as what is
+// left), so the workgroups resident on an XCD at one time share at most eight activation row blocks and a few
+// neighbouring column blocks of the weights.
+inline unsigned tile_grid(size_t mblocks, size_t nblocks) { return (unsigned)((mblocks * nblocks + 7) / 8 * 8); }
+#if defined(__HIPCC__)
+__device__ inline int tile_logical_id(int block, int grid) { return (block & 7) * (grid >> 3) + (block >> 3); }
+#endif
+__host__ __device__ inline bool tile_of(int lid, int mblocks, int nblocks, int* mb, int* nb) {
+  if (lid >= mblocks * nblocks) return false;
+  const int band = lid / (8 * nblocks);
+  const int left = mblocks - 8 * band, h = left < 8 ? left : 8;
+  const int idx = lid - band * 8 * nblocks;
+  *nb = idx / h;
+  *mb = 8 * band + (idx - *nb * h);
+  return true;
+}
+
 // out [m][k_out] = in [m][k_in] followed by zeros, 16-bit elements, k_in and k_out multiples of 8 (ksq_repack.hip)
 int pad_rows(void* out, const void* in, size_t m, size_t k_in, size_t k_out, hipStream_t s);
 

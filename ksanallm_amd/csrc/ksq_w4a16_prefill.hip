@@ -38,7 +38,7 @@ struct PrefillArgs {
   const void* act;
   void* out;
   const float* row_scale;  // bf16 route: 2^e per row of the re-encoded activations
-  int M, N, K, KT, G, ntiles, mblocks, nblocks, super_n;
+  int M, N, K, KT, G, ntiles, mblocks, nblocks;
   int ksplit;          // 64-row kernel only: grid.y
   float* partial;      // [ksplit][mblocks * 64][N] fp32, ksplit > 1 only
   Epilogue epi;
@@ -132,7 +132,6 @@ template <typename T, int GPT, int NW>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
   static_assert(NW == 4 || NW == 8, "four or eight waves side by side");
   constexpr int kFPW = 32 / NW;  // activation fragments of a stage that one wave brings in
-  constexpr int kSN = 32 / NW;   // column blocks per super-tile
   using O = Ops<_Float16>;  // the matrix cores run in fp16 for both element types
   using DQ = Dequant<T>;
   constexpr bool kBF16 = sizeof(T) == 2 && !__is_same(T, _Float16);
@@ -146,16 +145,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
 
-  // Workgroup numbering.  Hardware hands consecutive workgroup ids to the 8 XCDs in turn; every XCD (own L2) gets a
-  // contiguous run of logical ids, and logical ids walk super-tiles of 8 row blocks x kSN column blocks, so the
-  // workgroups resident on an XCD at one time (two per CU with four waves, one with eight) share 8 activation row
-  // blocks and 2048 weight columns.
-  const int per_xcd = gridDim.x >> 3;
-  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int st = lid / (8 * kSN), r = lid - st * (8 * kSN);
-  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
-  const int mb = st_m * 8 + (r & 7), nb = st_n * kSN + (r >> 3);
-  if (mb >= p.mblocks || nb >= p.nblocks) return;  // padding of partial super-tiles
+  int mb, nb;
+  if (!tile_of(tile_logical_id(blockIdx.x, gridDim.x), p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
   const int m0 = mb * kBM;
   const int nt0 = (nb * NW + wave) * kNT;
 
@@ -355,12 +346,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
 
-  const int per_xcd = gridDim.x >> 3;
-  const int lid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  const int st = lid >> 6, r = lid & 63;
-  const int st_m = st / p.super_n, st_n = st - st_m * p.super_n;
-  const int mb = st_m * 8 + (r & 7), nb = st_n * 8 + (r >> 3);
-  if (mb >= p.mblocks || nb >= p.nblocks) return;
+  int mb, nb;
+  if (!tile_of(tile_logical_id(blockIdx.x, gridDim.x), p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
   const int m0 = mb * (16 * kRows);
   const int nt0 = (nb * 4 + wave) * KNT;
 
@@ -709,19 +696,15 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     const int knt = plan.knt;
     nw = -knt;
     a.nblocks = (a.ntiles + 4 * knt - 1) / (4 * knt);
-    a.super_n = (a.nblocks + 7) / 8;
-    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * 64;  // whole 8 x 8 super-tiles
-    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
-    grid = dim3((unsigned)total, (unsigned)plan.ksplit);
+    KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
+    grid = dim3(tile_grid(a.mblocks, a.nblocks), (unsigned)plan.ksplit);
   } else {
     a.mblocks = (int)((m + kBM - 1) / kBM);
     nw = plan.nw;
-    const int bnt = nw * kNT, sn = 32 / nw;
+    const int bnt = nw * kNT;
     a.nblocks = (a.ntiles + bnt - 1) / bnt;
-    a.super_n = (a.nblocks + sn - 1) / sn;
-    const size_t total = (size_t)((a.mblocks + 7) / 8) * a.super_n * (8 * sn);  // whole super-tiles
-    KSQ_REQUIRE(total < (1ull << 31), KSQ_ERR_UNSUPPORTED, "grid too large");
-    grid = dim3((unsigned)total);
+    KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
+    grid = dim3(tile_grid(a.mblocks, a.nblocks));
     block = dim3(64 * nw);
   }
   const int gpt = (int)(kTileK / g);
