@@ -253,11 +253,11 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
       if (ap.partial_bytes > best) best = ap.partial_bytes;
     }
   }
-  if (max_m >= 65) {
+  if (max_m >= 49) {  // the large-M kernels serve 49 rows and more where the shape suits them
     // the element type is not known here: size for the bf16 route of the prefill kernel, plus the largest set of
     // split-K partial tiles any m up to max_m asks for (the plan depends on the number of 64-row blocks only)
     size_t partial = 0;
-    for (size_t mb = 2; mb <= (max_m + 63) / 64 && mb <= 2 * (size_t)cus; ++mb) {
+    for (size_t mb = 1; mb <= (max_m + 63) / 64 && mb <= 2 * (size_t)cus; ++mb) {
       const PrefillPlan pp = w4a16_prefill_plan(mb * 64, n, k, cus, (size_t)-1);
       if (pp.partial_bytes > partial) partial = pp.partial_bytes;
     }
@@ -327,7 +327,7 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   Epilogue epi;
   epi.kind = epilogue;
   epi.bias = bias;
-  if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g) &&
+  if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g, di->cus) &&
       workspace_bytes >= w4a16_prefill_workspace_bytes(dtype, m, k))
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, workspace_bytes, s, epi);
   // The kernels below split K across workgroups through arrival counters owned per stream; a stream that got none

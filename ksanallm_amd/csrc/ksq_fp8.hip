@@ -587,11 +587,11 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     const Fp8KstatPlan kp = fp8_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
     if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
   }
-  // large m: the partial tiles of a split last round of 256 x 256 tiles; the plan depends on the number of 256-row
+  // large m: the partial tiles of a split (last) round of 256 x 256 tiles; the plan depends on the number of 256-row
   // blocks only
   for (size_t mb = 1; mb <= (max_m + 255) / 256 && mb <= 64; ++mb) {
     const size_t mm = mb * 256 < max_m ? mb * 256 : max_m;
-    if (mm > 128 && fp8_prefill_supported(mm, n, k)) {
+    if (fp8_prefill_supported(mm, n, k)) {
       const size_t need = fp8_prefill_workspace_bytes(mm, n, k, cus);
       if (need > best) best = need;
     }

@@ -411,9 +411,24 @@ __global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) 
 static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int* tail_tiles, size_t* need) {
   *tail_tiles = 0;
   *need = 0;
-  if (m <= 128 || cus <= 0 || cus % 8 != 0) return 1;  // the main launch's tile count has to stay a multiple of eight
+  if (cus <= 0 || cus % 8 != 0) return 1;  // the main launch's tile count has to stay a multiple of eight
   const size_t total = ((m + 255) / 256) * ((n + 255) / 256), per_round = (size_t)cus;
-  if (total <= per_round) return 1;  // a single round: nothing to even out
+  if (total <= per_round) {
+    // A single round.  With at most half the CUs holding a tile and K long, the whole grid is the "tail": K split
+    // so that the splits fill the device, 16 k stages each at least (Qwen-72B qkv at M = 256: 40 tiles, 86 us unsplit).
+    size_t ks = per_round / total;
+    if (ks > 8) ks = 8;
+    if (ks > k / 128 / 16) ks = k / 128 / 16;
+    if (const char* e = tuning_env("KSQ_FP8_TAIL_KSPLIT")) {  // tuning / test override (1 switches the split off)
+      const int v = atoi(e);
+      if (v >= 1 && v <= 8 && (size_t)v <= k / 128) ks = (size_t)v;
+    }
+    const size_t bytes = ks * total * 65536 * 4;
+    if (ks <= 1 || bytes > workspace_bytes) return 1;
+    *tail_tiles = (int)total;
+    *need = bytes;
+    return (int)ks;
+  }
   const size_t rem = total % per_round;
   // measured at the Qwen-72B shapes, M = 2048: qkv (one full round + a quarter) 194 -> 186 us; gate_up (seven rounds
   // + a quarter) no gain, so grids of four rounds or more are left alone
@@ -459,10 +474,11 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
   a.KS = (int)(k / 128);
   a.a_scale_per_row = act_scale_count > 1;
   a.w_scale_per_col = w_scale_count > 1;
-  // 256 x 256 tiles (one workgroup of eight waves per CU) whenever there is more than one 128-row block: measured
-  // on the Qwen-72B shapes that kernel sustains 1.7 times the rate of the 128 x 256 one and is up to twice as fast
-  // even where its workgroups cover a third of the CUs; never more than 13 % slower.
-  int tile = m > 128 ? 256 : 128;
+  // 256 x 256 tiles (one workgroup of eight waves per CU): measured on the Qwen-72B shapes that kernel sustains 1.7
+  // times the rate of the 128 x 256 one and is the faster one from M = 128 on (at M = 128, where half of every tile
+  // is padding, by 8 to 18 %; it also has the K split that partly empty grids need).  The 128 x 256 kernel stays
+  // reachable through the override, which the parity tests use.
+  int tile = 256;
   if (const char* e = tuning_env("KSQ_FP8_PREFILL_TILE")) {  // tuning / test override
     const int v = atoi(e);
     if (v == 128 || v == 256) tile = v;
@@ -485,10 +501,13 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     // without a tail launch the one launch covers everything, rounded up to a multiple of eight; with one, the main
     // launch covers whole rounds (a multiple of eight by itself)
     const size_t main_tiles = ks > 1 ? total - (size_t)tail_tiles : tile_grid(a.mblocks, a.nblocks);
-    if (out_dtype == KSQ_F16)
+    if (main_tiles == 0) {
+      // every tile is in the split launch
+    } else if (out_dtype == KSQ_F16) {
       hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
-    else
+    } else {
       hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
+    }
     if (ks > 1) {
       Fp8PrefillArgs t = a;
       t.lid_begin = (int)main_tiles;

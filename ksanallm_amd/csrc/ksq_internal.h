@@ -177,7 +177,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
                          size_t n, size_t k, size_t g, void* workspace, size_t workspace_bytes, hipStream_t s,
                          const Epilogue& epi = Epilogue());
 size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k);
-bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g);
+bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g, int cus);
 int w4a16_stream_max_slices(int mt, int nt);
 
 struct KstatPlan {

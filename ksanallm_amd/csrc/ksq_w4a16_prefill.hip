@@ -582,10 +582,15 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, 
 
 }  // namespace
 
-bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g) {
+bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g, int cus) {
   (void)g;
   (void)dtype;
-  size_t min_m = 65;
+  // From 65 rows on.  49 to 64 rows as well where the columns alone fill the device several times over, or fill it
+  // with a K long enough to split: there one 64-row block with the activations shared through LDS beats the decode
+  // kernels, whose workgroups each pull all activations through their own loads (measured at M = 64: Llama-3-70B
+  // gate_up 108 -> 86..102 us, down 53 -> 48, Llama-2-7B gate_up 30.2 -> 27.9; narrower shapes lose 10 to 60 %).
+  const size_t ntiles = n / kTileN, kt = k / kTileK;
+  size_t min_m = (ntiles >= 4 * (size_t)cus || (ntiles >= 2 * (size_t)cus && kt >= 128)) ? 49 : 65;
   if (const char* e = tuning_env("KSQ_W4_PREFILL_MIN_M")) {  // tuning / test override
     const int v = atoi(e);
     if (v >= 1) min_m = (size_t)v;
@@ -603,10 +608,25 @@ size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k) {
 PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   PrefillPlan p{};
   const size_t ntiles = n / kTileN, kt = k / kTileK, mb128 = (m + 127) / 128;
-  // Row tile of the workgroup: 128 rows when such tiles (128 x 256) give every CU a workgroup and every weight tile
-  // is shared by four row blocks or more (that kernel prefetches weights one k tile ahead only, which covers an L2
-  // hit but not a trip to HBM); else 64 rows with deeper prefetch.
-  p.rows = (mb128 * ((ntiles + 15) / 16) >= (size_t)cus && mb128 >= 4) ? 128 : 64;
+  // Row tile of the workgroup and, for 128 rows, the waves per workgroup, by a cost model of how the tiles fall on the
+  // compute units, in units of the time two 128 x 256 workgroups take side by side on one CU: workgroups run in
+  // rounds of two per CU (one for the eight-wave 128 x 512 tiles); a last round that puts at most one workgroup on a
+  // CU costs a little over half a round.  A 128 x 512 tile costs 1.85 of a 128 x 256 one, a 64 x 256 one 0.62 (the
+  // dequantisation is shared by half the rows).  Measured on the Llama-2-7B and Llama-3-70B shapes at M = 96 .. 2048:
+  // the choice is the fastest of the three or within 5 % of it wherever K is short enough not to ask for a K split,
+  // which only the 64-row kernel has (long K with few column blocks: o / down projections).
+  const size_t nb16 = (ntiles + 15) / 16, nb32 = (ntiles + 31) / 32, mb64 = (m + 63) / 64;
+  auto rounds_of_two = [&](size_t wgs, double tile) {  // two workgroups per CU
+    const size_t full = wgs / (2 * (size_t)cus), rem = wgs % (2 * (size_t)cus);
+    return 2.0 * tile * (double)full + (rem == 0 ? 0.0 : rem <= (size_t)cus ? 1.1 * tile : 2.0 * tile);
+  };
+  const double cost128w4 = rounds_of_two(mb128 * nb16, 1.0);
+  const double cost128w8 = 1.85 * (double)((mb128 * nb32 + (size_t)cus - 1) / (size_t)cus);
+  const double cost64 = rounds_of_two(mb64 * nb16, 0.62);
+  // a K that the 64-row kernel would split (64 k tiles or more, fewer workgroups than CUs) stays with it
+  const bool long_k_few_tiles = kt >= 64 && mb64 * nb16 < (size_t)cus;
+  const double cost128 = cost128w8 < cost128w4 ? cost128w8 : cost128w4;
+  p.rows = (!long_k_few_tiles && cost128 < 0.97 * cost64) ? 128 : 64;
   if (const char* e = tuning_env("KSQ_W4_PREFILL_ROWS")) {  // tuning / test override
     const int v = atoi(e);
     if (v == 64 || v == 128) p.rows = v;
@@ -630,7 +650,10 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     if (kt >= 64 && wgs(4) < (size_t)cus) {
       ks = 2 * (size_t)cus / wgs(4);
       if (ks > 8) ks = 8;
-      if (ks > kt / 12) ks = kt / 12;
+      if (ks > kt / 12) {  // too short for two workgroups per CU: one per CU if that fits, else what fits
+        const size_t one = (size_t)cus / wgs(4);
+        ks = one <= kt / 12 ? one : kt / 12;
+      }
       auto traffic_us = [&](size_t c) { return 2.0 * (double)c * (double)(mb * 64) * (double)n * 4.0 / 4e6; };
       while (ks > 1 && traffic_us(ks) > 0.4 * 0.7 * (double)kt) --ks;
       if (ks < 1) ks = 1;
@@ -650,11 +673,7 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     p.ksplit = (int)ks;
     p.partial_bytes = need(ks);
   } else {
-    // Eight waves (128 x 512 per workgroup, one workgroup per CU) halve the activation traffic per flop; measured at
-    // M = 4096 they win up to N = 8192 (fewer, fatter workgroups), four waves (128 x 256, two per CU) beyond.
-    // (and up to N = 12288 when they fill every CU at least twice: qkv of Llama-2-7B at M = 4096, +5 %)
-    const size_t wgs8 = mb128 * ((ntiles + 31) / 32);
-    p.nw = ((wgs8 >= (size_t)cus && ntiles <= 512) || (wgs8 >= 2 * (size_t)cus && ntiles <= 768)) ? 8 : 4;
+    p.nw = cost128w8 < cost128w4 ? 8 : 4;
     if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 4 || v == 8) p.nw = v;

@@ -171,10 +171,13 @@ def test_workspace_sizes_of_padded_k_and_split_last_round():
     """What the planners add to the workspace, computed on the host alone (256 compute units when no device is there):
     the padded copy of the activation rows when K is an odd multiple of 64, and the fp32 partial tiles of a large-M FP8
     GEMM whose last round of 256 x 256 tiles is at most half full (Qwen-72B qkv at M = 2048: 40 + 40 + ... = 320 tiles
-    on 256 units, so 64 tiles x 4 splits x 256 KiB); the self-quantising entry point adds the FP8 rows and scales."""
+    on 256 units, so 64 tiles x 4 splits x 256 KiB) or that is a single round leaving most units empty; the
+    self-quantising entry point adds the FP8 rows and scales."""
     assert capi.w4a16_workspace_bytes(16, 64, 192) == capi.w4a16_workspace_bytes(16, 64, 256) + 16 * 256 * 2
     assert capi.fp8_workspace_bytes(2048, 10240, 8192) == 64 * 4 * 256 * 256 * 4
-    assert capi.fp8_workspace_bytes(2048, 8192, 8192) < 64 * 4 * 256 * 256 * 4      # 256 tiles: one full round
+    # a single round that leaves most units empty is split as a whole: 40 tiles, 64 k stages = 4 splits of 16
+    assert capi.fp8_workspace_bytes(256, 10240, 8192) == 40 * 4 * 256 * 256 * 4
+    assert capi.fp8_workspace_bytes(64, 10240, 8192) < 40 * 4 * 256 * 256 * 4       # decode kernels only
     front = capi.fp8_gemm_dynamic_workspace_bytes(2048, 10240, 8192) - capi.fp8_workspace_bytes(2048, 10240, 8192)
     assert 2048 * 8192 + 2048 * 4 <= front <= 2048 * 8192 + 2048 * 4 + 1024
 
