@@ -591,7 +591,7 @@ int ksq_fp8_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
   // blocks only
   for (size_t mb = 1; mb <= (max_m + 255) / 256 && mb <= 64; ++mb) {
     const size_t mm = mb * 256 < max_m ? mb * 256 : max_m;
-    if (fp8_prefill_supported(mm, n, k)) {
+    if (fp8_prefill_supported(mm, n, k, cus)) {
       const size_t need = fp8_prefill_workspace_bytes(mm, n, k, cus);
       if (need > best) best = need;
     }
@@ -699,7 +699,7 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
               KSQ_ERR_INVALID_ARGUMENT, "act_q and w_q must be 16-byte aligned");
   const DeviceInfo* di = device_info();
   if (!di) return KSQ_ERR_HIP;
-  if (fp8_prefill_supported(m, n, k) && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
+  if (fp8_prefill_supported(m, n, k, di->cus) && (reinterpret_cast<uintptr_t>(out) & 15) == 0)
     return fp8_launch_prefill(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k,
                               workspace, workspace ? workspace_bytes : 0, static_cast<hipStream_t>(stream), epi);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;

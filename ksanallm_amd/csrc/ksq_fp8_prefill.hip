@@ -453,8 +453,18 @@ size_t fp8_prefill_workspace_bytes(size_t m, size_t n, size_t k, int cus) {
   return need;
 }
 
-bool fp8_prefill_supported(size_t m, size_t n, size_t k) {
-  return m >= 128 && n % 8 == 0 && k % 128 == 0 && m * k < 0x7FFFFF00ull && n * k < 0x7FFFFF00ull;
+bool fp8_prefill_supported(size_t m, size_t n, size_t k, int cus) {
+  // From 65 rows on (the decode kernels end at 64; the streaming fallback is several times slower than a padded
+  // 256-row tile with K split over the grid).  From 33 rows on shapes whose columns fill the device several times
+  // over, or fill it with a K long enough to split (measured at M = 48 and 64 on the Qwen-72B shapes: gate_up 134 ->
+  // 120 and 139 -> 117 us, down 86 -> 78 and 89 -> 79 us; qkv and o lose 30 %).
+  const size_t ntiles = n / 16, ks = k / 128;
+  size_t min_m = (ntiles >= 4 * (size_t)cus || (ntiles >= 2 * (size_t)cus && ks >= 128)) ? 33 : 65;
+  if (const char* e = tuning_env("KSQ_FP8_PREFILL_MIN_M")) {  // tuning / test override
+    const int v = atoi(e);
+    if (v >= 1) min_m = (size_t)v;
+  }
+  return m >= min_m && n % 8 == 0 && k % 128 == 0 && m * k < 0x7FFFFF00ull && n * k < 0x7FFFFF00ull;
 }
 
 int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,

@@ -235,7 +235,7 @@ struct Fp8Plan {
   bool prefill;
 };
 Fp8Plan fp8_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
-bool fp8_prefill_supported(size_t m, size_t n, size_t k);
+bool fp8_prefill_supported(size_t m, size_t n, size_t k, int cus);
 size_t fp8_prefill_workspace_bytes(size_t m, size_t n, size_t k, int cus);  // partial tiles of a split last round
 int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                        const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,

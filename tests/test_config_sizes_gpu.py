@@ -150,6 +150,21 @@ def test_64_row_kernel_more_than_eight_row_blocks(gpu):
         w.check(M, what=f"64-row M={M}")
 
 
+@pytest.mark.parametrize("kind,dtype,K,N", [("awq", "bf16", 4096, 22016), ("awq", "f16", 4096, 22016),
+                                            ("gptq", "f16", 28672, 8192)])
+def test_wide_shapes_49_to_64_rows(gpu, kind, dtype, K, N):
+    """49 to 64 rows on shapes whose columns fill the device several times over (or fill it, with a K long enough to
+    split) go through the 64-row kernel of the large-M path, 48 rows and fewer through the decode kernels: both sides
+    of that boundary, ragged row counts, bf16 (re-encoded activations) and fp16, and the K split."""
+    import torch
+
+    w = BigW4(torch, gpu, 2300 + K + N, K, N, kind, dtype)
+    for M in (48, 49, 57, 64):
+        w.check(M, what=f"wide {kind} {dtype} K={K} N={N} M={M}")
+    del w
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("name,K,N", SHAPES_70B)
 def test_config3_gptq_70b_all_shapes(gpu, name, K, N):
     """configs[3]: GPTQ symmetric int4, fp16, M = 1, 32 and 256 at the four Llama-3-70B shapes."""
@@ -179,7 +194,8 @@ def test_config1_awq_decode_device_built(gpu, name, K, N):
 def test_config4_fp8_all_shapes(gpu, name, K, N):
     """configs[4]: e4m3 weights [N, K] with per-channel scales (N(0,1) x 0.02 quantised per output channel by the
     library's own load-time conversion, which has its own bit-exact test), bf16 activations N(0,1) quantised per token,
-    M = 1, 64 and 2048, bf16 out.  The activation quantisation of the chosen rows is checked bit for bit against the
+    M = 1, 64 and 2048, bf16 out; and M = 40 and 100, which the wide shapes (40) and all shapes (100) give to the
+    256-row tile kernel with K split over a grid that one round does not fill.  The activation quantisation of the chosen rows is checked bit for bit against the
     oracle, the GEMM to the parity bar."""
     import torch
 
@@ -196,7 +212,7 @@ def test_config4_fp8_all_shapes(gpu, name, K, N):
         capi.fp8_convert_weight_per_channel(capi.BF16, src, K, n1 - n0, wq[n0:n1], wscale[n0:n1])
         torch.cuda.synchronize()
         del src
-    for M in (1, 64, 2048):
+    for M in (1, 40, 64, 100, 2048):
         what = f"cfg4 {name} M={M}"
         act = torch.randn((M, K), device=gpu, generator=gen).to(torch.bfloat16)
         aq = torch.empty((M, K), dtype=torch.uint8, device=gpu)
