@@ -287,15 +287,16 @@ def fp8_case(torch, capi, dev, stream, gen, ws, wscale, k, n, M, reps):
 def fp8_sweep(torch, capi, dev, stream):
     """configs[4]: FP8 e4m3 GEMM at the Qwen-72B shapes, per-channel weight scales x per-token activation scales,
     bf16 in / out.  M = 1 and 64 against the HBM peak (algorithmic bytes K*N + 4N + M*K + 4M + 2*M*N), M = 2048 against
-    the dense FP8 MFMA peak; the activation quantisation is timed on its own."""
+    the dense FP8 MFMA peak (and M = 256, a batch between the configs' own, where the tile grid leaves most compute
+    units without a tile of their own); the activation quantisation is timed on its own."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(3)
     table = {}
     for name, k, n in SHAPES_72B:
         ws, wscale = fp8_weights(torch, dev, gen, k, n)
         row = {"copies": len(ws)}
-        for M in (1, 64, 2048):
-            uq, ug, ud = fp8_case(torch, capi, dev, stream, gen, ws, wscale, k, n, M, 32 if M <= 64 else 4)
+        for M in (1, 64, 256, 2048):
+            uq, ug, ud = fp8_case(torch, capi, dev, stream, gen, ws, wscale, k, n, M, 32 if M <= 64 else (16 if M < 2048 else 4))
             if M <= 64:
                 b = fp8_bytes(M, k, n)
                 row[f"m{M}"] = {"quant_us": round(uq, 1), "gemm_us": round(ug, 1), "GBps": round(b / ug / 1e3, 1),
@@ -314,14 +315,14 @@ def fp8_sweep(torch, capi, dev, stream):
 
 def gptq_70b_sweep(torch, capi, dev, stream):
     """configs[3]: symmetric GPTQ int4 g=128, fp16, the Llama-3-70B shapes at M = 1, 32 (HBM-bound: GB/s against the
-    HBM peak) and 256 (TFLOP/s against the dense MFMA peak)."""
+    HBM peak) and 256 (TFLOP/s against the dense MFMA peak), and 128 as a batch between the two."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(5)
     table = {}
     for name, k, n in SHAPES_70B:
         w, sz = gptq_weight(torch, capi, dev, gen, k, n)
         row = {"copies": ncopies_for(w.numel())}
-        for M in (1, 32, 256):
+        for M in (1, 32, 128, 256):
             us = w4_decode_shape(torch, capi, stream, name, k, n, w, sz, M, capi.F16, gen, count=max(16, ncopies_for(w.numel())))
             if M <= 32:
                 b = w4a16_bytes(M, k, n, awq=False)
@@ -602,6 +603,7 @@ def main():
         extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], stream, gen, "f16")
         extra["prefill_m2048"] = prefill(torch, capi, layers[0], stream, gen, M=2048)
         extra["prefill_m512"] = prefill(torch, capi, layers[0], stream, gen, M=512)
+        extra["prefill_m128"] = prefill(torch, capi, layers[0], stream, gen, M=128)  # between configs[1] and [2]
         del layers[1:]
         torch.cuda.empty_cache()
         extra["fp8_cfg4"] = fp8_sweep(torch, capi, dev, stream)
