@@ -316,17 +316,19 @@ def _fp8_case(seed, M, K, N, per_channel):
 
 @pytest.mark.parametrize("out_dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("per_channel", [False, True])
-@pytest.mark.parametrize("M,kstat", [(1, 1), (16, 1), (16, 0), (40, 1), (64, 1), (100, 1), (256, 1)])
+@pytest.mark.parametrize("M,kstat,K", [(1, 1, 1024), (16, 1, 1024), (16, 0, 1024), (40, 1, 1024), (64, 1, 1024),
+                                       (100, 1, 1024), (256, 1, 1024), (100, 1, 4096), (300, 1, 4096)])
 @pytest.mark.parametrize("epilogue", ["bias", "silu_mul"])
-def test_fp8_epilogues(gpu, out_dtype, per_channel, M, kstat, epilogue):
-    """The same two epilogues on the FP8 GEMM (k-stationary, streaming and large-M kernels).  For SiLU-mul the weight
+def test_fp8_epilogues(gpu, out_dtype, per_channel, M, kstat, K, epilogue):
+    """The same two epilogues on the FP8 GEMM (k-stationary, streaming and large-M kernels; with K = 4096 the large-M
+    kernel splits K over its few tiles and the reduction kernel applies the epilogue).  For SiLU-mul the weight
     rows [gate ; up] and their scales are interleaved with ksq_interleave_halves."""
     import torch
 
     from ksanallm_amd import capi
 
-    K, N = 1024, 544
-    aq, a_s, wq, w_s = _fp8_case(2300 + M, M, K, N, per_channel)
+    N = 544
+    aq, a_s, wq, w_s = _fp8_case(2300 + M + K, M, K, N, per_channel)
     acc = orc.fp8_gemm(aq, a_s, wq, w_s)
     d_wq, d_ws = _dev(wq, gpu), _dev(w_s, gpu)
     bias = None
