@@ -359,9 +359,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       const float* src = epi + rr * kEpiStride + cc;
       const int row = mw + 16 * mt + rr, col = nw + cc;
       if (part) {
-        f32x4* dst = reinterpret_cast<f32x4*>(part + (128 * wm + 16 * mt + rr) * 256 + 64 * wn + cc);
-        dst[0] = f32x4{src[0], src[1], src[2], src[3]};
-        dst[1] = f32x4{src[4], src[5], src[6], src[7]};
+        if (row < p.M) {  // the reduction kernel reads no row past M either
+          f32x4* dst = reinterpret_cast<f32x4*>(part + (128 * wm + 16 * mt + rr) * 256 + 64 * wn + cc);
+          dst[0] = f32x4{src[0], src[1], src[2], src[3]};
+          dst[1] = f32x4{src[4], src[5], src[6], src[7]};
+        }
         continue;
       }
       const float as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
