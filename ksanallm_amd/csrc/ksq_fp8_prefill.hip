@@ -265,14 +265,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
     for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Rows past M: the activation rows 32 * wave .. 32 * wave + 31 that this wave stages are not loaded when all of them
+  // lie past M (what the LDS then holds feeds only output rows that are never stored), and a wave whose 128 output
+  // rows all lie past M issues its share of the loads and no matrix instruction.  Both are uniform over the wave; a
+  // step's `vmcnt(4)` keeps its meaning, since the loads that may stay in flight are the step's weight loads.
+  const bool a_live = m0 + 32 * wave < p.M, rows_live = m0 + 128 * wm < p.M;
   // item i < 8 of a step's loads: i < 4 activations of stage sa, else weights of stage sb
   auto load_item = [&](u32x4* abuf, u32x4* bbuf, int sa, int sb, int i) {
     const int f = i & 3;
     // the scalar offset is not range-checked: past K, the last stage again (nobody uses it)
     const int sac = sa < p.KS ? sa : p.KS - 1, sbc = sb < p.KS ? sb : p.KS - 1;
-    if (i < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sac * 128, 0, 0);
-    else
+    if (i < 4) {
+      if (a_live)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sac * 128, 0, 0);
+    } else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], sbc * 128, 0, 0);
   };
   auto read_frag = [&](const u32x4* buf, int tile) {
@@ -287,6 +293,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
     __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
     __builtin_amdgcn_s_barrier();        // ... everyone's share has landed, and everyone is done with the stage before
     __builtin_amdgcn_sched_barrier(0);
+    if (!rows_live) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) load_item(anxt, bnxt2, s + 1, s + 2, i);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
     i32x8 bf[kNT];
 #pragma unroll
     for (int t = 0; t < kNT; ++t) bf[t] = read_frag(bcur, 4 * wn + t);
