@@ -168,7 +168,8 @@ int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* ac
 struct PrefillPlan {
   int rows;    // rows per workgroup tile: 64 or 128
   int knt;     // 64-row kernel: column tiles per wave (1, 2 or 4)
-  int nw;      // 128-row kernel: waves per workgroup (4 or 8)
+  int nw;      // 128-row kernel: waves side by side (4 or 8)
+  int kg;      // 128-row kernel with four waves side by side: k groups of such waves (1 or 2)
   int ksplit;  // 64-row kernel: grid.y
   size_t partial_bytes;
 };

@@ -128,9 +128,13 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_long_kernel(const uint16
   }
 }
 
-template <typename T, int GPT, int NW>
+template <typename T, int GPT, int NW, int KG = 1>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
   static_assert(NW == 4 || NW == 8, "four or eight waves side by side");
+  // KG = 2: two groups of four waves on the same 128 x 256 tile, the first on the even k tiles, the second on the
+  // odd ones, each with its own pair of activation stages; the second group's accumulators reach the first through
+  // LDS at the end.  For grids that put one workgroup on a CU: two waves per SIMD instead of one.
+  static_assert(KG == 1 || (KG == 2 && NW == 4), "two k groups of four waves");
   constexpr int kFPW = 32 / NW;  // activation fragments of a stage that one wave brings in
   using O = Ops<_Float16>;  // the matrix cores run in fp16 for both element types
   using DQ = Dequant<T>;
@@ -140,9 +144,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   // two activation stages as two separate objects: loads into one are then known not to alias reads of the other
   __shared__ u32x4 lds_a0[kStage];
   __shared__ u32x4 lds_a1[kStage];
+  __shared__ u32x4 lds_a2[KG == 2 ? kStage : 1];
+  __shared__ u32x4 lds_a3[KG == 2 ? kStage : 1];
 
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kg = KG == 2 ? wave_all >> 2 : 0;           // k group of this wave
+  const int wave = KG == 2 ? wave_all & 3 : wave_all;  // its place among the waves side by side
   const int c = lane & 15, j = lane >> 4;
 
   int mb, nb;
@@ -243,7 +251,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   };
   // One k tile.  On entry everything in flight (this tile's activations and weights) has landed and is visible to
   // the whole workgroup, and every wave is done with the other buffer.
-  auto step = [&](const u32x4* cur, u32x4* nxt, const BTile& bt, BTile& bn, int kt) {
+  auto step = [&](const u32x4* cur, u32x4* nxt, const BTile& bt, BTile& bn, int kt) __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -262,7 +270,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         mfma_row(a0[i], b, i);
-        if (ks < 2) load_item(nxt, bn, kt + 1, 2 * ks, i);
+        if (ks < 2) load_item(nxt, bn, kt + KG, 2 * ks, i);
         __builtin_amdgcn_sched_barrier(0);
       }
       if (ks < 3) read_half(a0, cur, ks + 1, 0);
@@ -270,25 +278,60 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         mfma_row(a1[i], b, 4 + i);
-        if (ks < 2) load_item(nxt, bn, kt + 1, 2 * ks + 1, i);
+        if (ks < 2) load_item(nxt, bn, kt + KG, 2 * ks + 1, i);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
 
+  // The k loop of one k group over its pair of stages: k tiles kg, kg + KG, ...  Both groups make the same number of
+  // steps (a step is one barrier); with an odd number of k tiles the second group's last step has no tile.
+  // (everything here has to be inlined: a call would put the accumulators, captured by reference, into memory)
+  auto k_loop = [&](u32x4* s0, u32x4* s1) __attribute__((always_inline)) {
+    auto run = [&](const u32x4* cur, u32x4* nxt, const BTile& bt, BTile& bn, int kt) __attribute__((always_inline)) {
+      if (KG == 1 || kt < p.KT) {
+        step(cur, nxt, bt, bn, kt);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();
+      }
+    };
 #pragma unroll
-  for (int q = 0; q < 4; ++q) load_part(lds_a0, b0, 0, q);
-  int kt = 0;
-  for (; kt + 2 <= p.KT; kt += 2) {
-    step(lds_a0, lds_a1, b0, b1, kt);
-    step(lds_a1, lds_a0, b1, b0, kt + 1);
-  }
-  if (kt < p.KT) step(lds_a0, lds_a1, b0, b1, kt);
+    for (int q = 0; q < 4; ++q) load_part(s0, b0, kg, q);
+    const int nsteps = (p.KT + KG - 1) / KG;
+    int st = 0;
+    for (; st + 2 <= nsteps; st += 2) {
+      run(s0, s1, b0, b1, kg + st * KG);
+      run(s1, s0, b1, b0, kg + (st + 1) * KG);
+    }
+    if (st < nsteps) run(s0, s1, b0, b1, kg + st * KG);
+  };
+  if (KG == 1 || kg == 0) k_loop(lds_a0, lds_a1);
+  else k_loop(lds_a2, lds_a3);
 
   // ---- epilogue: transpose each 16-row slab through LDS so that every lane stores 16 contiguous bytes
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
   __syncthreads();
   float* epi = reinterpret_cast<float*>(wave < 4 ? lds_a0 : lds_a1) + (wave & 3) * (16 * kEpiStride);  // 4352 B
+  if constexpr (KG == 2) {
+    // wave w of the second group parks its accumulators in stage w; wave w of the first group, which owns the same
+    // output tiles, adds them to its own and then uses that stage, and no other, for its transposes
+    f32x4* park = reinterpret_cast<f32x4*>(wave == 0 ? lds_a0 : wave == 1 ? lds_a1 : wave == 2 ? lds_a2 : lds_a3);
+    if (kg == 1) {
+#pragma unroll
+      for (int mt = 0; mt < kMT; ++mt)
+#pragma unroll
+        for (int t = 0; t < kNT; ++t) park[(mt * kNT + t) * 64 + lane] = acc[mt][t];
+    }
+    __syncthreads();
+    if (kg == 1) return;
+#pragma unroll
+    for (int mt = 0; mt < kMT; ++mt)
+#pragma unroll
+      for (int t = 0; t < kNT; ++t) acc[mt][t] += park[(mt * kNT + t) * 64 + lane];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): all of them read before the transposes overwrite the stage
+    epi = reinterpret_cast<float*>(park);
+  }
   uint16_t* out = static_cast<uint16_t*>(p.out);
   const int ncol0 = nt0 * 16;
   float cf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // bf16 scales: 2^E of this lane's eight columns
@@ -560,7 +603,7 @@ __global__ __launch_bounds__(256) void w4a16_splitk_reduce_kernel(const float* _
 }
 
 template <typename T>
-void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, hipStream_t s) {
+void launch_typed(const PrefillArgs& a, int gpt, int nw, int kg, dim3 grid, dim3 block, hipStream_t s) {
   if (nw <= 0) {  // 64-row tiles; -nw = 16-column tiles per wave
     const int knt = -nw;
     if (gpt == 1) {
@@ -572,6 +615,11 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, dim3 grid, dim3 block, 
       else if (knt == 2) hipLaunchKernelGGL((w4a16_mid_kernel<T, 2, 2>), grid, block, 0, s, a);
       else hipLaunchKernelGGL((w4a16_mid_kernel<T, 2, 1>), grid, block, 0, s, a);
     }
+    return;
+  }
+  if (nw == 4 && kg == 2) {
+    if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 4, 2>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 4, 2>), grid, block, 0, s, a);
     return;
   }
   if (gpt == 1 && nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 4>), grid, block, 0, s, a);
@@ -607,6 +655,7 @@ size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k) {
 // Tile shapes and the K split of the 64-row kernel; `workspace_bytes` is what remains behind the bf16 front part.
 PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   PrefillPlan p{};
+  p.kg = 1;
   const size_t ntiles = n / kTileN, kt = k / kTileK, mb128 = (m + 127) / 128;
   // Row tile of the workgroup and, for 128 rows, the waves per workgroup, by a cost model of how the tiles fall on the
   // compute units, in units of the time two 128 x 256 workgroups take side by side on one CU: workgroups run in
@@ -620,7 +669,8 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     const size_t full = wgs / (2 * (size_t)cus), rem = wgs % (2 * (size_t)cus);
     return 2.0 * tile * (double)full + (rem == 0 ? 0.0 : rem <= (size_t)cus ? 1.1 * tile : 2.0 * tile);
   };
-  const double cost128w4 = rounds_of_two(mb128 * nb16, 1.0);
+  // (a grid of at most one 128 x 256 workgroup per CU runs as two k groups of four waves: the price of a full tile)
+  const double cost128w4 = (mb128 * nb16 <= (size_t)cus && kt >= 4) ? 1.0 : rounds_of_two(mb128 * nb16, 1.0);
   const double cost128w8 = 1.85 * (double)((mb128 * nb32 + (size_t)cus - 1) / (size_t)cus);
   const double cost64 = rounds_of_two(mb64 * nb16, 0.62);
   // a K that the 64-row kernel would split (64 k tiles or more, fewer workgroups than CUs) stays with it
@@ -674,10 +724,17 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     p.partial_bytes = need(ks);
   } else {
     p.nw = cost128w8 < cost128w4 ? 8 : 4;
+    // one workgroup per CU at most: two k groups of four waves each
+    p.kg = (p.nw == 4 && mb128 * nb16 <= (size_t)cus && kt >= 4) ? 2 : 1;
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_KG")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 1 || (v == 2 && kt >= 2)) p.kg = v;
+    }
     if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 4 || v == 8) p.nw = v;
     }
+    if (p.nw == 8) p.kg = 1;
   }
   return p;
 }
@@ -724,11 +781,11 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     a.nblocks = (a.ntiles + bnt - 1) / bnt;
     KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
     grid = dim3(tile_grid(a.mblocks, a.nblocks));
-    block = dim3(64 * nw);
+    block = dim3(64 * nw * plan.kg);
   }
   const int gpt = (int)(kTileK / g);
   if (dtype == KSQ_F16) {
-    launch_typed<_Float16>(a, gpt, nw, grid, block, s);
+    launch_typed<_Float16>(a, gpt, nw, plan.kg, grid, block, s);
   } else {
     uint16_t* a16 = static_cast<uint16_t*>(workspace);
     float* row_scale = reinterpret_cast<float*>(static_cast<char*>(workspace) + (m * k * 2 + 255) / 256 * 256);
@@ -741,7 +798,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     else hipLaunchKernelGGL(bf16_rows_to_f16_long_kernel, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     a.act = a16;
     a.row_scale = row_scale;
-    launch_typed<__bf16>(a, gpt, nw, grid, block, s);
+    launch_typed<__bf16>(a, gpt, nw, plan.kg, grid, block, s);
   }
   if (plan.ksplit > 1) {  // add the splits up and store
     const size_t stride = (size_t)a.mblocks * 64 * n;

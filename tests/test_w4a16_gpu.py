@@ -174,6 +174,26 @@ def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("kg", [1, 2])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 65, 640, 528),      # five k tiles: the second k group's last step has no tile
+    ("bf16", "awq", 128, 200, 1024, 272),   # eight k tiles, two row blocks, ragged rows and columns
+    ("f16", "gptq", 64, 130, 384, 512),     # three k tiles, two groups per tile
+    ("bf16", "gptq", 64, 300, 256, 256),    # two k tiles: one step per k group
+])
+def test_prefill_128_rows_k_groups(gpu, kg, dtype, kind, g, M, K, N):
+    """The 128-row kernel with four waves side by side, as one group or as two groups that take the even and the odd
+    k tiles and add their accumulators through LDS at the end (what the planner picks for grids of at most one
+    workgroup per compute unit); twice, bit for bit."""
+    case = W4Case(1270 + kg + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    with _env(KSQ_W4_PREFILL_ROWS=128, KSQ_W4_PREFILL_WAVES=4, KSQ_W4_PREFILL_KG=kg):
+        got1 = dev.gemm_f32()
+        got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"prefill 128 rows kg={kg} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+
+
 @pytest.mark.parametrize("ksplit", [2, 3, 8])
 @pytest.mark.parametrize("nt", [1, 4])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
