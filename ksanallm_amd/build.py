@@ -85,6 +85,13 @@ def build_layer_driver():
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if p.returncode != 0:
         raise RuntimeError("layer driver build failed:\n" + p.stdout)
+    # host-only check of the workgroup -> tile map shared by the tile kernels (run by tests/test_capi_host.py)
+    tm = os.path.join(HERE, "tile_map_test")
+    cmd = [cc, "--offload-arch=gfx950", "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+           os.path.join(ROOT, "tests", "cpp", "tile_map_test.hip"), "-o", tm]
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("tile map test build failed:\n" + p.stdout)
     return out
 
 

@@ -204,3 +204,16 @@ def test_host_repack_pads_a_k_that_is_an_odd_multiple_of_64():
     assert np.all(szw[K // g:] == (8 << 16))
     with pytest.raises(capi.KsqError):
         capi.w4a16_repack_sizes(192, N, 128)   # group size 128 needs whole groups
+
+
+def test_workgroup_to_tile_map_is_a_bijection():
+    """tile_of / tile_grid (csrc/ksq_internal.h), the map from workgroup ids to output tiles that the large-M kernels
+    share: every tile exactly once for 40 x 31 grid sizes, ids past the last tile refused, bands of eight row blocks
+    walked column by column.  The checker is a host program built next to the library."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(capi.LIB_PATH), "tile_map_test")
+    if not os.path.exists(exe):
+        pytest.skip("tile_map_test has not been built (python -m ksanallm_amd.build)")
+    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert p.returncode == 0 and p.stdout.startswith("OK"), p.stdout
