@@ -62,9 +62,15 @@ __device__ inline i32x8 join(u32x4 lo, u32x4 hi) {
 constexpr int kFusedRows = 8;
 constexpr int kFusedRowBytes = 64 * 128 + 16;  // 64 stages per workgroup at most; 16 bytes of padding spread the banks
 
-template <typename T, int MT, int TPW, int NB, int NW, bool FUSED>
+// AR = activation rows that one load instruction covers: 16 (lane l on row l / 4), or 4 for M <= 4 (lane l on row
+// l / 4 % 4 of 64-byte chunk l / 16: four half stages per instruction instead of one; every vector memory instruction
+// costs the compute unit the same whatever its lanes carry, and at one token the activation loads were a quarter of
+// all loads of a workgroup).
+template <typename T, int MT, int TPW, int NB, int NW, bool FUSED, int AR = 16>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4))) void fp8_kstat_kernel(Fp8KstatArgs p) {
+  static_assert(AR == 16 || (AR == 4 && MT == 1 && !FUSED), "narrow activation loads: one row tile, at most four rows");
   constexpr int D = NB * TPW;  // ring depth = one batch
+  constexpr int NL = (2 * TPW + 3) / 4;  // AR = 4: load instructions for the 2 * TPW half stages of a wave
   static_assert(NB * MT * NW <= 64 && NB * MT <= NW, "two reduction buffers of at most 64 KiB, one tile per wave");
   static_assert(!FUSED || (MT == 1 && NB <= 2 && NW == 16 && TPW <= 4), "fused quantisation: one row tile, 64 KiB of LDS left");
   __shared__ f32x4 red[2 * NB * MT * NW * 64];
@@ -128,7 +134,17 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
 
   // activation fragments of this wave's stages: registers for the whole kernel
   i32x8 af[MT][TPW];
-  if constexpr (!FUSED) {
+  u32x4 araw[AR == 4 ? NL : 1];
+  if constexpr (AR == 4) {
+#pragma unroll
+    for (int u = 0; u < NL; ++u) {
+      const int hs = 4 * u + (lane >> 4), t = hs >> 1, h = hs & 1, row = (lane >> 2) & 3;
+      const unsigned kb = (unsigned)(s0 + t) * 128u + 64u * h + 16u * lp;
+      const bool ok = hs < 2 * TPW && s0 + t < wg_end && kb + 16u <= (unsigned)p.K && row < p.M;
+      araw[u] = __builtin_bit_cast(
+          u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ok ? (unsigned)row * p.K + kb : 0x80000000u, 0, 0));
+    }
+  } else if constexpr (!FUSED) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -194,7 +210,25 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  if constexpr (!FUSED) {
+  if constexpr (AR == 4) {
+    // operand lane 16 j + r takes piece j of row r from the lane that loaded it: row r < 4 of half stage hs sits in
+    // lane 16 * (hs % 4) + 4 r + j of load hs / 4; rows 4 .. 15 are zero
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+      i32x8 v;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int hs = 2 * t + h;
+        const int src = (16 * (hs & 3) + 4 * (r & 3) + j) * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int x = __builtin_amdgcn_ds_bpermute(src, (int)araw[hs >> 2][q]);
+          v[4 * h + q] = r < 4 ? x : 0;
+        }
+      }
+      af[0][t] = v;
+    }
+  } else if constexpr (!FUSED) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -329,7 +363,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 }
 
-#define KSQ_GO(MT, TPW, NB, NW) hipLaunchKernelGGL((fp8_kstat_kernel<T, MT, TPW, NB, NW, false>), grid, dim3(64 * NW), 0, s, a)
+// one row tile and at most four rows: the narrow activation loads
+#define KSQ_GO(MT, TPW, NB, NW)                                                                                   \
+  do {                                                                                                            \
+    if (MT == 1 && a.M <= 4)                                                                                      \
+      hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, TPW, NB, NW, false, 4>), grid, dim3(64 * NW), 0, s, a);          \
+    else                                                                                                          \
+      hipLaunchKernelGGL((fp8_kstat_kernel<T, MT, TPW, NB, NW, false>), grid, dim3(64 * NW), 0, s, a);            \
+  } while (0)
 #define KSQ_GO_FUSED(TPW, NB) hipLaunchKernelGGL((fp8_kstat_kernel<T, 1, TPW, NB, 16, true>), grid, dim3(1024), 0, s, a)
 template <typename T>
 bool launch_fused(int tpw, int nb, const Fp8KstatArgs& a, dim3 grid, hipStream_t s) {
