@@ -469,11 +469,12 @@ size_t fp8_prefill_workspace_bytes(size_t m, size_t n, size_t k, int cus) {
 
 bool fp8_prefill_supported(size_t m, size_t n, size_t k, int cus) {
   // From 65 rows on (the decode kernels end at 64; the streaming fallback is several times slower than a padded
-  // 256-row tile with K split over the grid).  From 33 rows on shapes whose columns fill the device several times
-  // over, or fill it with a K long enough to split (measured at M = 48 and 64 on the Qwen-72B shapes: gate_up 134 ->
-  // 120 and 139 -> 117 us, down 86 -> 78 and 89 -> 79 us; qkv and o lose 30 %).
+  // 256-row tile with K split over the grid).  From 17 rows on shapes whose columns fill the device several times
+  // over, or fill it with a K long enough to split (measured on the Qwen-72B shapes against the decode kernel:
+  // gate_up 111 -> 99 us at M = 17 .. 32 and 139 -> 101 .. 117 at M = 64, down 73 -> 56 and 89 -> 59; qkv and o lose
+  // 10 to 50 %, and so do the wide shapes at 16 rows and fewer).
   const size_t ntiles = n / 16, ks = k / 128;
-  size_t min_m = (ntiles >= 4 * (size_t)cus || (ntiles >= 2 * (size_t)cus && ks >= 128)) ? 33 : 65;
+  size_t min_m = (ntiles >= 4 * (size_t)cus || (ntiles >= 2 * (size_t)cus && ks >= 128)) ? 17 : 65;
   if (const char* e = tuning_env("KSQ_FP8_PREFILL_MIN_M")) {  // tuning / test override
     const int v = atoi(e);
     if (v >= 1) min_m = (size_t)v;
