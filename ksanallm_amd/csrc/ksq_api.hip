@@ -253,7 +253,7 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
       if (ap.partial_bytes > best) best = ap.partial_bytes;
     }
   }
-  if (max_m >= 49) {  // the large-M kernels serve 49 rows and more where the shape suits them
+  if (max_m >= 33) {  // the large-M kernels serve 33 rows and more where the shape suits them
     // the element type is not known here: size for the bf16 route of the prefill kernel, plus the largest set of
     // split-K partial tiles any m up to max_m asks for (the plan depends on the number of 64-row blocks only)
     size_t partial = 0;

@@ -401,6 +401,7 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   if (const char* e = tuning_env("KSQ_W4_KSTAT_NB")) {  // tuning override, within what is instantiated
     const int v = atoi(e);
     if (p.mt == 1 && (v == 1 || v == 2 || (v == 4 && p.tpw <= 2)) && !(p.tpw >= 4 && v > 1) && v <= p.nt_per_wg) p.nb = v;
+    if (p.mt >= 2 && (v == 1 || v == 2) && v <= p.nt_per_wg) p.nb = v;
   }
   p.partial_bytes = need(ksplit);
   return p;

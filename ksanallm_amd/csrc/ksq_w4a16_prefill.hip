@@ -633,12 +633,13 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, int kg, dim3 grid, dim3
 bool w4a16_prefill_supported(int dtype, size_t m, size_t n, size_t k, size_t g, int cus) {
   (void)g;
   (void)dtype;
-  // From 65 rows on.  49 to 64 rows as well where the columns alone fill the device several times over, or fill it
+  // From 65 rows on.  33 to 64 rows as well where the columns alone fill the device several times over, or fill it
   // with a K long enough to split: there one 64-row block with the activations shared through LDS beats the decode
-  // kernels, whose workgroups each pull all activations through their own loads (measured at M = 64: Llama-3-70B
-  // gate_up 108 -> 86..102 us, down 53 -> 48, Llama-2-7B gate_up 30.2 -> 27.9; narrower shapes lose 10 to 60 %).
+  // kernels, whose workgroups each pull all activations through their own loads (measured at M = 40 / 64: Llama-3-70B
+  // gate_up 96 -> 77 / 109 -> 81..88 us, down 47 -> 44.5 / 53 -> 48, Llama-2-7B gate_up 27.5 -> 25.9 / 30.3 -> 28;
+  // narrower shapes lose 10 to 60 %, and at 32 rows the decode kernel is 5 % ahead on the wide ones too).
   const size_t ntiles = n / kTileN, kt = k / kTileK;
-  size_t min_m = (ntiles >= 4 * (size_t)cus || (ntiles >= 2 * (size_t)cus && kt >= 128)) ? 49 : 65;
+  size_t min_m = (ntiles >= 4 * (size_t)cus || (ntiles >= 2 * (size_t)cus && kt >= 128)) ? 33 : 65;
   if (const char* e = tuning_env("KSQ_W4_PREFILL_MIN_M")) {  // tuning / test override
     const int v = atoi(e);
     if (v >= 1) min_m = (size_t)v;

@@ -152,14 +152,14 @@ def test_64_row_kernel_more_than_eight_row_blocks(gpu):
 
 @pytest.mark.parametrize("kind,dtype,K,N", [("awq", "bf16", 4096, 22016), ("awq", "f16", 4096, 22016),
                                             ("gptq", "f16", 28672, 8192)])
-def test_wide_shapes_49_to_64_rows(gpu, kind, dtype, K, N):
-    """49 to 64 rows on shapes whose columns fill the device several times over (or fill it, with a K long enough to
-    split) go through the 64-row kernel of the large-M path, 48 rows and fewer through the decode kernels: both sides
+def test_wide_shapes_33_to_64_rows(gpu, kind, dtype, K, N):
+    """33 to 64 rows on shapes whose columns fill the device several times over (or fill it, with a K long enough to
+    split) go through the 64-row kernel of the large-M path, 32 rows and fewer through the decode kernels: both sides
     of that boundary, ragged row counts, bf16 (re-encoded activations) and fp16, and the K split."""
     import torch
 
     w = BigW4(torch, gpu, 2300 + K + N, K, N, kind, dtype)
-    for M in (48, 49, 57, 64):
+    for M in (32, 33, 49, 57, 64):
         w.check(M, what=f"wide {kind} {dtype} K={K} N={N} M={M}")
     del w
     torch.cuda.empty_cache()
