@@ -371,7 +371,11 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   // One row tile: whole batches of four column tiles.  Fewer, fatter workgroups than CUs still win (measured at the
   // Llama-2-7B shapes: 3 -> 4 and 6 -> 8 column tiles per workgroup): every workgroup reads its whole k range of the
   // activations from the L2, and a short last batch costs a barrier and a reduction like a full one.
-  if (p.mt == 1 && p.nt_per_wg >= 3 && env_round4()) p.nt_per_wg = (p.nt_per_wg + 3) & ~3;
+  // (beyond four with at most two k tiles per wave, where the batches are two tiles each, whole batches of two: six
+  // tiles stay six -- at gate_up of Llama-2-7B 11.6 .. 11.9 us against 12.3 .. 13.0 with eight at M = 1, level at
+  // M = 16; with four k tiles per wave, Llama-3-70B gate_up, sixteen tiles beat fourteen by 2 %)
+  if (p.mt == 1 && p.nt_per_wg >= 3 && env_round4())
+    p.nt_per_wg = (p.nt_per_wg <= 4 || p.tpw >= 3) ? (p.nt_per_wg + 3) & ~3 : (p.nt_per_wg + 1) & ~1;
   if (const char* e = tuning_env("KSQ_W4_KSTAT_NT_PER_WG")) {  // tuning / test override: "v" or "ntiles:v,ntiles:v"
     for (const char* q = e; q && *q;) {
       const long a = strtol(q, const_cast<char**>(&q), 10);
