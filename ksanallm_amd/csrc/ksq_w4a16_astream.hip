@@ -520,6 +520,11 @@ void launch(int mt, int cnt, bool lds, const AstreamArgs& a, dim3 grid, hipStrea
     else if (cnt == 2) KSQ_GO(2, 2);
     else if (cnt == 3) KSQ_GO(2, 3);
     else KSQ_GO(2, 4);
+  } else if (mt == 3) {
+    if (cnt == 1) KSQ_GO(3, 1);
+    else if (cnt == 2) KSQ_GO(3, 2);
+    else if (cnt == 3) KSQ_GO(3, 3);
+    else KSQ_GO(3, 4);
   } else {
     if (cnt == 1) KSQ_GO(4, 1);
     else if (cnt == 2) KSQ_GO(4, 2);
@@ -569,9 +574,13 @@ bool w4a16_astream_supported(size_t m, size_t n, size_t k) {
 // never better than two).  The element type plays no part, so the workspace can be sized without it.
 AstreamPlan w4a16_astream_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   AstreamPlan p{};
-  p.mt = m <= 32 ? 2 : 4;
+  p.mt = m <= 32 ? 2 : (m <= 48 ? 3 : 4);  // row tiles past M cost their activation loads and matrix instructions
+  if (const char* e = tuning_env("KSQ_W4_ASTREAM_MT")) {  // tuning / test override: never fewer than the rows need
+    const int v = atoi(e);
+    if (v >= 2 && v <= 4 && (size_t)v * 16 >= m) p.mt = v;
+  }
   const size_t ntiles = n / kTileN, kt = k / kTileK;
-  size_t ks = (ntiles <= 2 * (size_t)cus && kt >= 16 && (p.mt == 4 || kt >= 80)) ? 2 : 1;
+  size_t ks = (ntiles <= 2 * (size_t)cus && kt >= 16 && (p.mt >= 3 || kt >= 80)) ? 2 : 1;
   if (const char* e = tuning_env("KSQ_W4_ASTREAM_KSPLIT")) {  // tuning / test override
     const size_t v = (size_t)atoi(e);
     if (v >= 1 && v <= 8 && v <= kt) ks = v;

@@ -98,18 +98,25 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_kernel(const uint16_t* _
   }
 }
 
-// the same for rows longer than 16384 elements: two passes over global memory
+// the same for rows longer than 32768 elements: two passes over global memory, eight elements per load
 __global__ __launch_bounds__(256) void bf16_rows_to_f16_long_kernel(const uint16_t* __restrict__ src,
                                                                     uint16_t* __restrict__ dst,
                                                                     float* __restrict__ row_scale, int K) {
   __shared__ float smem[4];
   const size_t row = blockIdx.x;
-  const uint16_t* s = src + row * K;
-  uint16_t* d = dst + row * K;
+  const u32x4* s = reinterpret_cast<const u32x4*>(src + row * K);
+  u32x4* d = reinterpret_cast<u32x4*>(dst + row * K);
+  const int nchunks = K / 8;
   float mx = 0.f;
-  for (int i = threadIdx.x; i < K; i += 256) {
-    const float v = __builtin_fabsf(__builtin_bit_cast(float, (uint32_t)s[i] << 16));
-    mx = (v == v && v < __builtin_inff()) ? __builtin_fmaxf(mx, v) : mx;
+  for (int ch = threadIdx.x; ch < nchunks; ch += 256) {
+    const u32x4 v = s[ch];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float lo = __builtin_fabsf(__builtin_bit_cast(float, v[q] << 16));
+      const float hi = __builtin_fabsf(__builtin_bit_cast(float, v[q] & 0xFFFF0000u));
+      mx = (lo == lo && lo < __builtin_inff()) ? __builtin_fmaxf(mx, lo) : mx;
+      mx = (hi == hi && hi < __builtin_inff()) ? __builtin_fmaxf(mx, hi) : mx;
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off));
@@ -122,9 +129,17 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_long_kernel(const uint16
   const float down = __builtin_bit_cast(float, (uint32_t)(127 - e) << 23);
   const float up = __builtin_bit_cast(float, (uint32_t)(127 + e) << 23);
   if (threadIdx.x == 0) row_scale[row] = up;
-  for (int i = threadIdx.x; i < K; i += 256) {
-    const float v = __builtin_bit_cast(float, (uint32_t)s[i] << 16) * down;
-    d[i] = __builtin_bit_cast(uint16_t, (_Float16)v);
+  for (int ch = threadIdx.x; ch < nchunks; ch += 256) {
+    const u32x4 v = s[ch];
+    u32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float lo = __builtin_bit_cast(float, v[q] << 16) * down;
+      const float hi = __builtin_bit_cast(float, v[q] & 0xFFFF0000u) * down;
+      o[q] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) |
+             ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+    }
+    d[ch] = o;
   }
 }
 
@@ -796,6 +811,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     else if (k <= 4096) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<2>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     else if (k <= 8192) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<4>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     else if (k <= 16384) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<8>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
+    else if (k <= 32768) hipLaunchKernelGGL(bf16_rows_to_f16_kernel<16>, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     else hipLaunchKernelGGL(bf16_rows_to_f16_long_kernel, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     a.act = a16;
     a.row_scale = row_scale;

@@ -155,6 +155,23 @@ def test_prefill_kernel_widths(gpu, waves, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("K", [8192, 17408, 28672, 33792])
+def test_prefill_bf16_long_rows(gpu, K):
+    """bf16 activations on the large-M route are re-encoded row by row as fp16 x 2^e: rows of up to 16384 and up to
+    32768 elements stay in registers between the row maximum and the conversion, longer ones are read twice.  Rows
+    with very different magnitudes, so that the per-row exponent matters."""
+    M, N = 70, 64
+    case = W4Case(1250 + K // 128, M, K, N, g=128, kind="gptq", dtype="bf16")
+    act = orc.from_bits(case.act, orc.BF16)
+    act *= np.exp2(np.random.default_rng(K).integers(-20, 21, size=(M, 1))).astype(np.float32)
+    case.act = orc.to_bits(act, orc.BF16)
+    dev = W4Device(case, gpu)
+    got1 = dev.gemm_f32()
+    got2 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"prefill bf16 rows of {K}")
+    assert np.array_equal(got1, got2)
+
+
 @pytest.mark.parametrize("rows,nt", [(64, 1), (64, 2), (64, 4), (128, 4)])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "awq", 128, 65, 640, 528),     # five k tiles: the four-deep ring wraps with a remainder
