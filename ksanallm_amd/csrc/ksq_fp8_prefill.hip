@@ -208,26 +208,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 // stages of activations, three of weights = all 160 KiB), so
 // each byte crosses the CU's vector memory path once per workgroup: 128 x 256 tiles need 46 B/clk per CU at the
 // matrix cores' FP8 rate, this one 32.  One workgroup per CU.
-template <typename T>
+// WN = 4: the whole tile, waves as 2 x 4.  WN = 1: a quarter of it, 256 rows x 64 columns, waves as 8 x 1 (every wave 32
+// rows x 64 columns), four workgroups to a tile: for the tiles of a last round that is mostly empty, which then fill
+// the device without a K split (no partial tiles through memory).  Its weight stage is 8 KiB, one block per wave.
+template <typename T, int WN = 4>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void fp8_prefill256_kernel(Fp8PrefillArgs p) {
-  constexpr int kHalf = 16 * 2 * 64;  // 16-byte elements of one operand of one stage (32 KiB)
+  static_assert(WN == 4 || WN == 1, "whole tiles or column quarters");
+  constexpr int kMTW = WN == 4 ? 8 : 2;      // row tiles per wave
+  constexpr int kHalf = 16 * 2 * 64;         // 16-byte elements of an activation stage (32 KiB)
+  constexpr int kHalfB = 4 * WN * 2 * 64;    // ... of a weight stage (32 or 8 KiB)
   constexpr int kEpiStride = 68;
   __shared__ u32x4 lds_a0[kHalf];
   __shared__ u32x4 lds_a1[kHalf];
-  __shared__ u32x4 lds_b0[kHalf];
-  __shared__ u32x4 lds_b1[kHalf];
-  __shared__ u32x4 lds_b2[kHalf];
+  __shared__ u32x4 lds_b0[kHalfB];
+  __shared__ u32x4 lds_b1[kHalfB];
+  __shared__ u32x4 lds_b2[kHalfB];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = WN == 4 ? wave >> 2 : wave, wn = WN == 4 ? wave & 3 : 0;
   const int r = lane & 15, j = lane >> 4;
 
-  // this launch covers the logical tile ids lid_begin .. lid_begin + gridDim.x - 1 of the whole grid
-  const int lid = p.lid_begin + tile_logical_id(blockIdx.x, gridDim.x);
+  // this launch covers the logical tile ids lid_begin .. of the whole grid (with WN = 1: four workgroups to a tile)
+  const int unit = tile_logical_id(blockIdx.x, gridDim.x);
+  const int lid = p.lid_begin + (WN == 4 ? unit : unit >> 2);
   int mb, nb;
   if (!tile_of(lid, p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
-  const int m0 = mb * 256, n0 = nb * 256;
+  const int m0 = mb * 256, n0 = nb * 256 + (WN == 4 ? 0 : 64 * (unit & 3));
 
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
@@ -250,27 +257,31 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       int row = m0 + 16 * (2 * wave + (i >> 1)) + 8 * q + rr;
       row = row < p.M ? row : p.M - 1;
       a_off[i] = (unsigned)row * p.K + kb;
-      int col = n0 + 16 * (2 * wave + (i >> 1)) + 8 * q + rr;
+      // weight blocks: four per wave of the 32, or (WN = 1) block `wave` of the 8: tile wave / 2, rows 8 (wave % 2) ..
+      const int wq8 = WN == 4 ? q : (wave & 1), wx = (rr >> 2) | (wq8 << 1);
+      const unsigned wkb = 64u * hh + 16u * ((lane & 3) ^ wx);
+      int col = WN == 4 ? n0 + 16 * (2 * wave + (i >> 1)) + 8 * q + rr : n0 + 16 * (wave >> 1) + 8 * (wave & 1) + rr;
       col = col < p.N ? col : p.N - 1;
-      w_off[i] = (unsigned)col * p.K + kb;
+      w_off[i] = (unsigned)col * p.K + wkb;
     }
   }
   // where lane (r, j) finds piece j of half 0 of row r of a tile inside the stage, apart from tile * 128 and
   // half * 32 (in 16-byte units)
   const int f_lane = (r >> 3) * 64 + (r & 7) * 4 + (j ^ (((r & 7) >> 2) | ((r >> 3) << 1)));
 
-  f32x4 acc[kMT][kNT];
+  f32x4 acc[kMTW][kNT];
 #pragma unroll
-  for (int mt = 0; mt < kMT; ++mt)
+  for (int mt = 0; mt < kMTW; ++mt)
 #pragma unroll
     for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // Rows past M: the activation rows 32 * wave .. 32 * wave + 31 that this wave stages are not loaded when all of them
   // lie past M (what the LDS then holds feeds only output rows that are never stored), and a wave whose 128 output
   // rows all lie past M issues its share of the loads and no matrix instruction.  Both are uniform over the wave; a
-  // step's `vmcnt(4)` keeps its meaning, since the loads that may stay in flight are the step's weight loads.
-  const bool a_live = m0 + 32 * wave < p.M, rows_live = m0 + 128 * wm < p.M;
-  // item i < 8 of a step's loads: i < 4 activations of stage sa, else weights of stage sb
+  // step's `vmcnt` keeps its meaning, since the loads that may stay in flight are the step's weight loads.
+  const bool a_live = m0 + 32 * wave < p.M, rows_live = m0 + 16 * kMTW * wm < p.M;
+  // item i of a step's loads: i < 4 activations of stage sa, else weights of stage sb (four, or one with WN = 1)
+  constexpr int kItems = 4 + WN;
   auto load_item = [&](u32x4* abuf, u32x4* bbuf, int sa, int sb, int i) {
     const int f = i & 3;
     // the scalar offset is not range-checked: past K, the last stage again (nobody uses it)
@@ -278,8 +289,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
     if (i < 4) {
       if (a_live)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sac * 128, 0, 0);
-    } else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (4 * wave + f) * 64), 16, w_off[f], sbc * 128, 0, 0);
+    } else if (i < kItems) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (WN * wave + f) * 64), 16, w_off[f], sbc * 128, 0, 0);
+    }
   };
   auto read_frag = [&](const u32x4* buf, int tile) {
     return join(buf[tile * 128 + f_lane], buf[tile * 128 + 32 + f_lane]);
@@ -290,27 +302,37 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   // retire in order and a step issues its activation loads before its weight loads, so on entry everything but the
   // four weight loads of the previous step (stage s + 1) has to have landed.
   auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt2, int s) {
-    __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+    if constexpr (WN == 4) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4): the four weight loads of the step before
+    else __builtin_amdgcn_s_waitcnt(0x0F71);                     // vmcnt(1)
     __builtin_amdgcn_s_barrier();        // ... everyone's share has landed, and everyone is done with the stage before
     __builtin_amdgcn_sched_barrier(0);
     if (!rows_live) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) load_item(anxt, bnxt2, s + 1, s + 2, i);
+      for (int i = 0; i < kItems; ++i) load_item(anxt, bnxt2, s + 1, s + 2, i);
       __builtin_amdgcn_sched_barrier(0);
       return;
     }
     i32x8 bf[kNT];
 #pragma unroll
     for (int t = 0; t < kNT; ++t) bf[t] = read_frag(bcur, 4 * wn + t);
-    i32x8 a_cur = read_frag(acur, 8 * wm + 0), a_nxt = read_frag(acur, 8 * wm + 1);
+    i32x8 a_cur = read_frag(acur, kMTW * wm + 0), a_nxt = read_frag(acur, kMTW * wm + 1);
 #pragma unroll
-    for (int mt = 0; mt < kMT; ++mt) {
+    for (int mt = 0; mt < kMTW; ++mt) {
       const i32x8 af = a_cur;
       a_cur = a_nxt;
-      if (mt + 2 < kMT) a_nxt = read_frag(acur, 8 * wm + mt + 2);
-      if (mt < 4) {  // the loads go out in the first half: activations first, then weights
-        load_item(anxt, bnxt2, s + 1, s + 2, mt < 2 ? 2 * mt : 4 + 2 * (mt - 2));
-        load_item(anxt, bnxt2, s + 1, s + 2, mt < 2 ? 2 * mt + 1 : 4 + 2 * (mt - 2) + 1);
+      if (mt + 2 < kMTW) a_nxt = read_frag(acur, kMTW * wm + mt + 2);
+      if constexpr (WN == 4) {
+        if (mt < 4) {  // the loads go out in the first half: activations first, then weights
+          load_item(anxt, bnxt2, s + 1, s + 2, mt < 2 ? 2 * mt : 4 + 2 * (mt - 2));
+          load_item(anxt, bnxt2, s + 1, s + 2, mt < 2 ? 2 * mt + 1 : 4 + 2 * (mt - 2) + 1);
+        }
+      } else {  // two row tiles: the four activation loads with the first, the weight load with the second
+        if (mt == 0) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) load_item(anxt, bnxt2, s + 1, s + 2, i);
+        } else {
+          load_item(anxt, bnxt2, s + 1, s + 2, 4);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -325,9 +347,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
   for (int i = 0; i < 4; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
 #pragma unroll
-  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
+  for (int i = 4; i < kItems; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
 #pragma unroll
-  for (int i = 4; i < 8; ++i) load_item(lds_a0, lds_b1, s_begin, s_begin + 1, i);
+  for (int i = 4; i < kItems; ++i) load_item(lds_a0, lds_b1, s_begin, s_begin + 1, i);
   int s = s_begin;
   for (; s + 6 <= s_end; s += 6) {
     step(lds_a0, lds_b0, lds_a1, lds_b2, s);
@@ -347,9 +369,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   // ---- epilogue: scales, then a transpose through LDS so that every lane stores 16 contiguous bytes
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
   __syncthreads();
-  float* epi = reinterpret_cast<float*>(wm == 0 ? lds_a0 : lds_a1) + wn * (16 * kEpiStride);
+  float* epi = reinterpret_cast<float*>(wave < 4 ? lds_a0 : lds_a1) + (wave & 3) * (16 * kEpiStride);
   uint16_t* out = static_cast<uint16_t*>(p.out);
-  const int mw = m0 + 128 * wm, nw = n0 + 64 * wn;
+  const int mw = m0 + 16 * kMTW * wm, nw = n0 + 64 * wn;
   float ws[kNT];
 #pragma unroll
   for (int t = 0; t < kNT; ++t) {
@@ -359,7 +381,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   // split launch: the raw fp32 tile of this split, rows of 256 floats, for the reduction kernel
   float* part = p.ksplit > 1 ? p.partial + ((size_t)blockIdx.y * p.tail_tiles + (lid - p.lid_begin)) * 65536 : nullptr;
 #pragma unroll
-  for (int mt = 0; mt < kMT; ++mt) {
+  for (int mt = 0; mt < kMTW; ++mt) {
 #pragma unroll
     for (int t = 0; t < kNT; ++t)
 #pragma unroll
@@ -371,8 +393,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       const float* src = epi + rr * kEpiStride + cc;
       const int row = mw + 16 * mt + rr, col = nw + cc;
       if (part) {
-        if (row < p.M) {  // the reduction kernel reads no row past M either
-          f32x4* dst = reinterpret_cast<f32x4*>(part + (128 * wm + 16 * mt + rr) * 256 + 64 * wn + cc);
+        if (row < p.M) {  // the reduction kernel reads no row past M either (whole tiles only: WN = 4)
+          f32x4* dst = reinterpret_cast<f32x4*>(part + (16 * kMTW * wm + 16 * mt + rr) * 256 + 64 * wn + cc);
           dst[0] = f32x4{src[0], src[1], src[2], src[3]};
           dst[1] = f32x4{src[4], src[5], src[6], src[7]};
         }
@@ -422,9 +444,11 @@ __global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) 
 // is long, its tiles go out as a launch of their own with K split so that it fills the device: every split stores its
 // raw fp32 tile with plain stores and a reduction kernel finishes (the Qwen-72B qkv shape at M = 2048 is 320 tiles
 // on 256 CUs: a second round a quarter full).  Returns the split count (1 = no split) and the tiles in the tail.
-static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int* tail_tiles, size_t* need) {
+static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int* tail_tiles, size_t* need,
+                          bool* quarters) {
   *tail_tiles = 0;
   *need = 0;
+  *quarters = false;
   if (cus <= 0 || cus % 8 != 0) return 1;  // the main launch's tile count has to stay a multiple of eight
   const size_t total = ((m + 255) / 256) * ((n + 255) / 256), per_round = (size_t)cus;
   if (total <= per_round) {
@@ -444,6 +468,15 @@ static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspac
     return (int)ks;
   }
   const size_t rem = total % per_round;
+  // A last round that covers at most a quarter of the CUs goes out as column quarters of its tiles (256 x 64, four
+  // workgroups to a tile, no K split and nothing through memory)
+  bool use_quarters = rem != 0 && 4 * rem <= per_round;
+  if (const char* e = tuning_env("KSQ_FP8_TAIL_QUARTERS")) use_quarters = use_quarters && atoi(e) != 0;  // tuning switch
+  if (use_quarters) {
+    *tail_tiles = (int)rem;
+    *quarters = true;
+    return 1;
+  }
   // measured at the Qwen-72B shapes, M = 2048: qkv (one full round + a quarter) 194 -> 186 us; gate_up (seven rounds
   // + a quarter) no gain, so grids of four rounds or more are left alone
   if (rem == 0 || 2 * rem > per_round || k / 128 < 32 || total >= 4 * per_round) return 1;
@@ -463,7 +496,8 @@ static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspac
 size_t fp8_prefill_workspace_bytes(size_t m, size_t n, size_t k, int cus) {
   int tail = 0;
   size_t need = 0;
-  fp8_tail_split(m, n, k, cus, (size_t)-1, &tail, &need);
+  bool quarters = false;
+  fp8_tail_split(m, n, k, cus, (size_t)-1, &tail, &need, &quarters);
   return need;
 }
 
@@ -522,10 +556,11 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     int tail_tiles = 0;
     size_t need = 0;
     const bool ws_ok = workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0;
-    const int ks = fp8_tail_split(m, n, k, di->cus, ws_ok ? workspace_bytes : 0, &tail_tiles, &need);
+    bool quarters = false;
+    const int ks = fp8_tail_split(m, n, k, di->cus, ws_ok ? workspace_bytes : 0, &tail_tiles, &need, &quarters);
     // without a tail launch the one launch covers everything, rounded up to a multiple of eight; with one, the main
     // launch covers whole rounds (a multiple of eight by itself)
-    const size_t main_tiles = ks > 1 ? total - (size_t)tail_tiles : tile_grid(a.mblocks, a.nblocks);
+    const size_t main_tiles = (ks > 1 || quarters) ? total - (size_t)tail_tiles : tile_grid(a.mblocks, a.nblocks);
     if (main_tiles == 0) {
       // every tile is in the split launch
     } else if (out_dtype == KSQ_F16) {
@@ -533,7 +568,15 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     } else {
       hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
     }
-    if (ks > 1) {
+    if (quarters) {
+      Fp8PrefillArgs t = a;
+      t.lid_begin = (int)main_tiles;
+      const dim3 qgrid((unsigned)((4 * (size_t)tail_tiles + 7) / 8 * 8));
+      if (out_dtype == KSQ_F16)
+        hipLaunchKernelGGL((fp8_prefill256_kernel<_Float16, 1>), qgrid, dim3(512), 0, s, t);
+      else
+        hipLaunchKernelGGL((fp8_prefill256_kernel<__bf16, 1>), qgrid, dim3(512), 0, s, t);
+    } else if (ks > 1) {
       Fp8PrefillArgs t = a;
       t.lid_begin = (int)main_tiles;
       t.ksplit = ks;

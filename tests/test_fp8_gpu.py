@@ -215,13 +215,14 @@ def test_gemm_large_m_both_tiles(gpu, tile, M, K, N):
 
 
 @pytest.mark.parametrize("ksplit", [0, 1, 2, 3])
-@pytest.mark.parametrize("M,K,N", [(300, 4096, 9208), (300, 4096, 2600), (2048, 4096, 9216)])
+@pytest.mark.parametrize("M,K,N", [(300, 4096, 9208), (300, 4096, 2600), (2048, 4096, 9216), (2040, 4096, 11256)])
 def test_gemm_large_m_split_last_round(gpu, ksplit, M, K, N):
-    """256 x 256 tiles that do not fill whole rounds of one tile per compute unit.  288 tiles on 256 units: the last
-    32 go out as a launch of their own with K split (0 = the planner's own count, 1 = no split), partial tiles through
-    the workspace, a reduction kernel behind it.  72 and 22 tiles (the latter not a multiple of eight: the grid is
-    rounded up): a single round that leaves most units empty, so the whole grid is that split launch.  Ragged M and
-    N; twice, bit for bit; and without a workspace (no split)."""
+    """256 x 256 tiles that do not fill whole rounds of one tile per compute unit.  352 tiles on 256 units: the last
+    96 go out as a launch of their own with K split (0 = the planner's own count, 1 = no split), partial tiles through
+    the workspace, a reduction kernel behind it.  288 tiles: the last 32 cover at most a quarter of the units and go
+    out as column quarters (256 x 64, four workgroups to a tile) instead.  72 and 22 tiles (the latter not a multiple
+    of eight: the grid is rounded up): a single round that leaves most units empty, so the whole grid is the split
+    launch.  Ragged M and N; twice, bit for bit; and without a workspace (no K split)."""
     import os
 
     xq, xs, wq, ws = _fp8_case(450 + M, M, K, N)
