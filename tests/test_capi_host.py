@@ -170,11 +170,15 @@ def test_workspace_sizes_are_monotone_and_bounded():
 def test_workspace_sizes_of_padded_k_and_split_last_round():
     """What the planners add to the workspace, computed on the host alone (256 compute units when no device is there):
     the padded copy of the activation rows when K is an odd multiple of 64, and the fp32 partial tiles of a large-M FP8
-    GEMM whose last round of 256 x 256 tiles is at most half full (Qwen-72B qkv at M = 2048: 40 + 40 + ... = 320 tiles
-    on 256 units, so 64 tiles x 4 splits x 256 KiB) or that is a single round leaving most units empty; the
+    GEMM whose last round of 256 x 256 tiles is between a quarter and half full, or that is a single round leaving most
+    units empty; the
     self-quantising entry point adds the FP8 rows and scales."""
     assert capi.w4a16_workspace_bytes(16, 64, 192) == capi.w4a16_workspace_bytes(16, 64, 256) + 16 * 256 * 2
-    assert capi.fp8_workspace_bytes(2048, 10240, 8192) == 64 * 4 * 256 * 256 * 4
+    # 8 x 44 = 352 tiles: the last 96 (more than a quarter, at most half of the units) with K split in two
+    assert capi.fp8_workspace_bytes(2048, 11264, 8192) == 96 * 2 * 256 * 256 * 4
+    # 8 x 40 = 320 tiles: the last 64 go out as column quarters and need nothing; what is left is the largest need of
+    # a smaller batch (M = 512: 80 tiles in one round, K split in three)
+    assert capi.fp8_workspace_bytes(2048, 10240, 8192) == 80 * 3 * 256 * 256 * 4
     # a single round that leaves most units empty is split as a whole: 40 tiles, 64 k stages = 4 splits of 16
     assert capi.fp8_workspace_bytes(256, 10240, 8192) == 40 * 4 * 256 * 256 * 4
     assert capi.fp8_workspace_bytes(64, 10240, 8192) < 40 * 4 * 256 * 256 * 4       # decode kernels only
