@@ -51,6 +51,25 @@ __device__ inline uint16_t out_bits<__bf16>(float v) {
   return __builtin_bit_cast(uint16_t, (__bf16)v);
 }
 
+// A global -> LDS load of 16 bytes per lane (lane l lands at lds + 16 l) written as an assembly statement, so that the
+// compiler does not know it to be one: it would otherwise wait for *every* outstanding vector memory load before an
+// LDS read that follows (it cannot always tell which LDS bytes a pending load writes), which empties a ring of stages
+// that are deliberately left in flight.  The statement sets M0 (LDS address of lane 0) itself; the kernel that uses it
+// has no other user of M0.  Ordering against the LDS reads is the kernel's business (s_waitcnt vmcnt + s_barrier).
+__device__ inline u32x4 raw_rsrc(const void* base, size_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  return u32x4{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
+}
+__device__ inline uint32_t lds_addr(const void* p) {
+  return (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p);
+}
+__device__ inline void load_lds_opaque(u32x4 rsrc, uint32_t lds, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
 __device__ inline i32x8 join(u32x4 lo, u32x4 hi) {
   i32x8 v;
   v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
@@ -236,10 +255,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   if (!tile_of(lid, p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
   const int m0 = mb * 256, n0 = nb * 256 + (WN == 4 ? 0 : 64 * (unit & 3));
 
-  const __amdgpu_buffer_rsrc_t rs_a =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rs_w =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.wq), 0, (int)((size_t)p.N * p.K), 0x00020000);
+  const u32x4 rs_a = raw_rsrc(p.aq, (size_t)p.M * p.K), rs_w = raw_rsrc(p.wq, (size_t)p.N * p.K);
   // Operand stage in LDS: 32 blocks of 1 KiB per operand, block (tile, q) = rows 8q .. 8q+7 of a 16-row tile, all
   // 128 bytes of the stage.  A block is one global -> LDS load instruction (lane l lands at l * 16) with lane l on
   // row l/4 % 8, half l / 32 of the 128 bytes and 16-byte piece (l % 4) ^ x(row, q): every aligned group of four
@@ -282,18 +298,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   const bool a_live = m0 + 32 * wave < p.M, rows_live = m0 + 16 * kMTW * wm < p.M;
   // item i of a step's loads: i < 4 activations of stage sa, else weights of stage sb (four, or one with WN = 1)
   constexpr int kItems = 4 + WN;
-  auto load_item = [&](u32x4* abuf, u32x4* bbuf, int sa, int sb, int i) {
+  auto load_item = [&](u32x4* abuf, u32x4* bbuf, int sa, int sb, int i) __attribute__((always_inline)) {
     const int f = i & 3;
     // the scalar offset is not range-checked: past K, the last stage again (nobody uses it)
     const int sac = sa < p.KS ? sa : p.KS - 1, sbc = sb < p.KS ? sb : p.KS - 1;
     if (i < 4) {
-      if (a_live)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(abuf + (4 * wave + f) * 64), 16, a_off[f], sac * 128, 0, 0);
+      if (a_live) load_lds_opaque(rs_a, lds_addr(abuf + (4 * wave + f) * 64), a_off[f], sac * 128);
     } else if (i < kItems) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lds_ptr)(bbuf + (WN * wave + f) * 64), 16, w_off[f], sbc * 128, 0, 0);
+      load_lds_opaque(rs_w, lds_addr(bbuf + (WN * wave + f) * 64), w_off[f], sbc * 128);
     }
   };
-  auto read_frag = [&](const u32x4* buf, int tile) {
+  auto read_frag = [&](const u32x4* buf, int tile) __attribute__((always_inline)) {
     return join(buf[tile * 128 + f_lane], buf[tile * 128 + 32 + f_lane]);
   };
 
@@ -301,23 +316,57 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   // (mostly L2 hits: every row block is shared by all column blocks) one stage ahead into a ring of two.  Loads
   // retire in order and a step issues its activation loads before its weight loads, so on entry everything but the
   // four weight loads of the previous step (stage s + 1) has to have landed.
-  auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt2, int s) {
-    if constexpr (WN == 4) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4): the four weight loads of the step before
-    else __builtin_amdgcn_s_waitcnt(0x0F71);                     // vmcnt(1)
+  //
+  // WN = 4: the two halves of the workgroup (waves 0-3 = rows 0..127, waves 4-7 = rows 128..255; one wave of each on
+  // every SIMD) run half a step apart, so that on every SIMD one wave issues matrix instructions while the other
+  // waits for its first LDS reads after a barrier.  Every wave passes two barriers per step, one at its start and
+  // one in the middle (after four of its eight row tiles); the second half passed one more before its first step,
+  // the first half passes one more after its last.  A half stages exactly the activation rows it reads itself, so
+  // only the weight buffers tie the halves together: stage s is complete when the first half starts step s because
+  // the second half waits for its share of it before the barrier in the middle of its step s - 1 (all but the eight
+  // loads of that step have landed), and the buffer that the first half refills during step s (stage s - 1) was
+  // copied into registers by the second half before that same barrier.
+  auto mid_wait = [&]() __attribute__((always_inline)) {
+    if (wm == 1) {
+      if (a_live) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): this step's loads may be in flight
+      else __builtin_amdgcn_s_waitcnt(0x0F74);         // vmcnt(4): this wave loads weights only
+    }
+  };
+  auto step = [&](const u32x4* acur, const u32x4* bcur, u32x4* anxt, u32x4* bnxt2, int s) __attribute__((always_inline)) {
+    // vmcnt(4) / vmcnt(1): the weight loads of the step before may be in flight.  lgkmcnt(0) costs nothing here (the
+    // matrix instructions of the step before have consumed every LDS read) and tells the compiler that no scalar
+    // load is pending: LDS reads and scalar loads share that counter, and while it believes one of the latter may be
+    // in flight it turns the first LDS wait of the step into a wait for all 14 reads instead of the first four.
+    if constexpr (WN == 4) __builtin_amdgcn_s_waitcnt(0x0074);
+    else __builtin_amdgcn_s_waitcnt(0x0071);
     __builtin_amdgcn_s_barrier();        // ... everyone's share has landed, and everyone is done with the stage before
     __builtin_amdgcn_sched_barrier(0);
     if (!rows_live) {
 #pragma unroll
       for (int i = 0; i < kItems; ++i) load_item(anxt, bnxt2, s + 1, s + 2, i);
+      if constexpr (WN == 4) {
+        mid_wait();
+        __builtin_amdgcn_s_barrier();
+      }
       __builtin_amdgcn_sched_barrier(0);
       return;
     }
+    // the operands of the first matrix instruction first
     i32x8 bf[kNT];
+    i32x8 a_cur = read_frag(acur, kMTW * wm + 0);
 #pragma unroll
     for (int t = 0; t < kNT; ++t) bf[t] = read_frag(bcur, 4 * wn + t);
-    i32x8 a_cur = read_frag(acur, kMTW * wm + 0), a_nxt = read_frag(acur, kMTW * wm + 1);
+    i32x8 a_nxt = read_frag(acur, kMTW * wm + 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mt = 0; mt < kMTW; ++mt) {
+      if constexpr (WN == 4) {
+        if (mt == 4) {
+          mid_wait();
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
       const i32x8 af = a_cur;
       a_cur = a_nxt;
       if (mt + 2 < kMTW) a_nxt = read_frag(acur, kMTW * wm + mt + 2);
@@ -350,6 +399,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   for (int i = 4; i < kItems; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
 #pragma unroll
   for (int i = 4; i < kItems; ++i) load_item(lds_a0, lds_b1, s_begin, s_begin + 1, i);
+  if constexpr (WN == 4) {
+    if (wm == 1) {  // the second half starts half a step late; its share of the first weight stage has landed
+      __builtin_amdgcn_s_waitcnt(0x0F74);
+      __builtin_amdgcn_s_barrier();
+    }
+  }
   int s = s_begin;
   for (; s + 6 <= s_end; s += 6) {
     step(lds_a0, lds_b0, lds_a1, lds_b2, s);
@@ -365,6 +420,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   if (s + 2 < s_end) step(lds_a0, lds_b2, lds_a1, lds_b1, s + 2);
   if (s + 3 < s_end) step(lds_a1, lds_b0, lds_a0, lds_b2, s + 3);
   if (s + 4 < s_end) step(lds_a0, lds_b1, lds_a1, lds_b0, s + 4);
+  if constexpr (WN == 4) {
+    if (wm == 0) __builtin_amdgcn_s_barrier();  // the barrier in the middle of the second half's last step
+  }
 
   // ---- epilogue: scales, then a transpose through LDS so that every lane stores 16 contiguous bytes
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
