@@ -55,6 +55,12 @@ __device__ inline KRange astream_k_range(const AstreamArgs& p, int wave) {
   const int slice = (wg_end - r.wg_begin + 7) / 8;
   r.begin = r.wg_begin + wave * slice;
   r.end = r.begin + slice < wg_end ? r.begin + slice : wg_end;
+  // The 64-bit divisions above run on the vector unit, and a value that crosses a basic block in a vector register
+  // counts as divergent from there on: every global -> LDS load whose scalar offset derives from it would be wrapped
+  // in a readfirstlane loop.  The values are uniform; say so.
+  r.wg_begin = __builtin_amdgcn_readfirstlane(r.wg_begin);
+  r.begin = __builtin_amdgcn_readfirstlane(r.begin);
+  r.end = __builtin_amdgcn_readfirstlane(r.end);
   return r;
 }
 
@@ -133,11 +139,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     for (int i = 0; i < CNT; ++i) {
       const bool live = ok && i < count;  // uniform
       t.w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, live ? w_lane : 0x80000000u,
-                                                                               live ? kt * 1024 + i * (int)w_stride : 0, 2));
+                                                                               __builtin_amdgcn_readfirstlane(live ? kt * 1024 + i * (int)w_stride : 0), 2));
 #pragma unroll
       for (int gi = 0; gi < GPT; ++gi)
         t.sz[i][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, live ? sz_lane : 0x80000000u,
-                                                           live ? (kt * GPT + gi) * 64 + i * (int)sz_stride : 0, 0);
+                                                           __builtin_amdgcn_readfirstlane(live ? (kt * GPT + gi) * 64 + i * (int)sz_stride : 0), 0);
     }
   };
   // half h of k tile kt: 32-k steps 2h and 2h + 1 of all row tiles, as loaded (before the lane permutation)
@@ -356,11 +362,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     for (int i = 0; i < CNT; ++i) {
       const bool live = ok && i < count;  // uniform
       t.w[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, live ? w_lane : 0x80000000u,
-                                                                               live ? kt * 1024 + i * (int)w_stride : 0, 2));
+                                                                               __builtin_amdgcn_readfirstlane(live ? kt * 1024 + i * (int)w_stride : 0), 2));
 #pragma unroll
       for (int gi = 0; gi < GPT; ++gi)
         t.sz[i][gi] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, live ? sz_lane : 0x80000000u,
-                                                           live ? (kt * GPT + gi) * 64 + i * (int)sz_stride : 0, 0);
+                                                           __builtin_amdgcn_readfirstlane(live ? (kt * GPT + gi) * 64 + i * (int)sz_stride : 0), 0);
     }
   };
   // half h of k tile kt into this wave's part of `buf`.  A tile past the slice repeats the slice's first tile (the
