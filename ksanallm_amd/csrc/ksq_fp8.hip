@@ -297,8 +297,8 @@ __global__ __launch_bounds__(256) void fp8_stream_kernel(Fp8Args p) {
   const int nt = blockIdx.x * 4 + wave;
   if (nt >= p.ntiles) return;  // wave-uniform; no block-level barrier below
   const int split = blockIdx.y, mblock = blockIdx.z;
-  const int kb_begin = (int)(((long)p.KB * split) / p.ksplit);
-  const int kb_end = (int)(((long)p.KB * (split + 1)) / p.ksplit);
+  int kb_begin, kb_end;
+  split_range(p.KB, split, p.ksplit, &kb_begin, &kb_end);
   const int m0 = mblock * 16 * MT;
 
   int wrow = nt * 16 + c;

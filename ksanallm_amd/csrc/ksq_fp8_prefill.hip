@@ -392,7 +392,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   };
 
   // k stages of this launch's split (all of them unless this is the tail launch)
-  const int s_begin = (int)(((long)p.KS * blockIdx.y) / p.ksplit), s_end = (int)(((long)p.KS * (blockIdx.y + 1)) / p.ksplit);
+  int s_begin, s_end;
+  split_range(p.KS, blockIdx.y, p.ksplit, &s_begin, &s_end);
 #pragma unroll
   for (int i = 0; i < 4; ++i) load_item(lds_a0, lds_b0, s_begin, s_begin, i);
 #pragma unroll

@@ -94,6 +94,24 @@ __device__ inline ksq_f32x4 load_agent(const ksq_f32x4* p) {
   return __builtin_bit_cast(ksq_f32x4, w);
 }
 
+// Units [begin, end) of split `split` of `ksplit` over `total` k units: floor(total * split / ksplit) and the same for
+// split + 1.  One split, the common case, costs nothing.  Otherwise 32-bit divisions; a 64-bit one is some 150 scalar
+// instructions, and two of them in front of a wave's first load show in a kernel that lasts a few microseconds.  The
+// quotients come from the vector unit and are uniform: readfirstlane says so (a value that crosses a basic block in a
+// vector register otherwise counts as divergent, and loads whose scalar offset derives from it get wrapped in loops).
+__device__ inline void split_range(int total, int split, int ksplit, int* begin, int* end) {
+  if (ksplit <= 1) {
+    *begin = 0;
+    *end = total;
+  } else if (total < (1 << 26)) {  // ksplit <= 32: the products fit
+    *begin = __builtin_amdgcn_readfirstlane((int)((unsigned)(total * split) / (unsigned)ksplit));
+    *end = __builtin_amdgcn_readfirstlane((int)((unsigned)(total * (split + 1)) / (unsigned)ksplit));
+  } else {
+    *begin = __builtin_amdgcn_readfirstlane((int)(((long)total * split) / ksplit));
+    *end = __builtin_amdgcn_readfirstlane((int)(((long)total * (split + 1)) / ksplit));
+  }
+}
+
 // A wave that has parked its partial tile (store_agent) arrives at the tile's counter; every lane makes the call.
 // Returns true, in every lane, in the wave that finds the count complete: that wave then reads all splits' tiles
 // (load_agent).  Ordering: the tile's stores are agent-scope atomics, performed beyond the XCD's L2, and

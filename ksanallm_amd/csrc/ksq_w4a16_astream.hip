@@ -50,8 +50,8 @@ struct KRange {
 };
 __device__ inline KRange astream_k_range(const AstreamArgs& p, int wave) {
   KRange r;
-  r.wg_begin = (int)(((long)p.KT * blockIdx.y) / p.ksplit);
-  const int wg_end = (int)(((long)p.KT * (blockIdx.y + 1)) / p.ksplit);
+  int wg_end;
+  split_range(p.KT, blockIdx.y, p.ksplit, &r.wg_begin, &wg_end);
   const int slice = (wg_end - r.wg_begin + 7) / 8;
   r.begin = r.wg_begin + wave * slice;
   r.end = r.begin + slice < wg_end ? r.begin + slice : wg_end;

@@ -51,8 +51,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, j = lane >> 4;
   const int split = blockIdx.y;
-  const int wg_begin = (int)(((long)p.KT * split) / p.ksplit);
-  const int wg_end = (int)(((long)p.KT * (split + 1)) / p.ksplit);
+  int wg_begin, wg_end;
+  split_range(p.KT, split, p.ksplit, &wg_begin, &wg_end);
   const int kt0 = wg_begin + wave * TPW;  // first k tile of this wave
   const int nt_begin = blockIdx.x * p.nt_per_wg;
   int count = p.ntiles - nt_begin;

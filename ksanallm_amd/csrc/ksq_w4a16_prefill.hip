@@ -526,7 +526,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
   };
 
   // k tiles of this split
-  const int kt0 = (int)(((long)p.KT * blockIdx.y) / p.ksplit), kt1 = (int)(((long)p.KT * (blockIdx.y + 1)) / p.ksplit);
+  int kt0, kt1;
+  split_range(p.KT, blockIdx.y, p.ksplit, &kt0, &kt1);
   load_tile(lds_a0, b0, kt0);
   load_tile(lds_a1, b1, kt0 + 1);
   load_tile(lds_a2, b2, kt0 + 2);

@@ -60,8 +60,8 @@ w4a16_stream_kernel(StreamArgs p) {
   const int nt0 = grp * NT;
   const int split = blockIdx.y, mblock = blockIdx.z;
   // k range of the workgroup, then of this wave's slice; every slice runs the same number of ring rounds
-  const int wg_begin = (int)(((long)p.KT * split) / p.ksplit);
-  const int wg_end = (int)(((long)p.KT * (split + 1)) / p.ksplit);
+  int wg_begin, wg_end;
+  split_range(p.KT, split, p.ksplit, &wg_begin, &wg_end);
   const int wg_tiles = wg_end - wg_begin;
   const int kt_begin = wg_begin + (wg_tiles * slice) / KS;
   const int kt_end = wg_begin + (wg_tiles * (slice + 1)) / KS;
