@@ -242,11 +242,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
       const int q = wave - first, i = q / MT, mt = q - i * MT;
       const int nt = nt_begin + b * NB + i;
       const bool valid = b * NB + i < count && 16 * mt < p.M;
+      // The slices are added in wave order (deterministic), kRB reads in flight at a time: the weight ring is live in
+      // registers here, so all NW at once do not fit, but every group of reads is one LDS round trip on the path to
+      // the store, and for the last batch nothing else hides it.
+      constexpr int kRB = (MT == 1 && TPW <= 2 && D <= 4 && NW >= 8) ? 8 : 4;
       f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w4 = 0; w4 < NW; w4 += 4) {  // four slices at a time: the weight ring is live in registers here
+      for (int w0 = 0; w0 < NW; w0 += kRB) {
+        f32x4 part[kRB];
 #pragma unroll
-        for (int ww = w4; ww < w4 + 4; ++ww) sum += rb[(q * NW + ww) * 64 + lane];
+        for (int ww = 0; ww < kRB; ++ww) part[ww] = rb[(q * NW + w0 + ww) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ww = 0; ww < kRB; ++ww) sum += part[ww];
         __builtin_amdgcn_sched_barrier(0);
       }
       bool store = valid;
