@@ -325,11 +325,20 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
       const int i = wave / MT, mt = wave - i * MT;
       const int nt = nt_begin + b * NB + i;
       const bool valid = b * NB + i < count && 16 * mt < p.M;
+      // added in wave order (deterministic), eight reads in flight at a time: the weight ring is live in registers
+      // here, so all NW at once do not fit, but every group of reads is one LDS round trip on the way to the store
+      // (where the activation fragments and the ring leave the registers for it: otherwise the reads would spill)
+      constexpr int kOperandRegs = (MT * TPW + D) * 8;
+      constexpr int kRB = ((NW == 16 && kOperandRegs <= 48) || (NW == 8 && kOperandRegs <= 160)) ? 8 : 4;
       f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w4 = 0; w4 < NW; w4 += 4) {  // four slices at a time: the weight ring is live in registers here
+      for (int w0 = 0; w0 < NW; w0 += kRB) {
+        f32x4 part[kRB];
 #pragma unroll
-        for (int ww = w4; ww < w4 + 4; ++ww) sum += rb[(wave * NW + ww) * 64 + lane];
+        for (int ww = 0; ww < kRB; ++ww) part[ww] = rb[(wave * NW + w0 + ww) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ww = 0; ww < kRB; ++ww) sum += part[ww];
         __builtin_amdgcn_sched_barrier(0);
       }
       bool store = valid;

@@ -259,9 +259,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   __syncthreads();
   for (int q = wave; q < kTiles; q += kWaves) {
     const int i = q / MT, mt = q - i * MT;
+    // all eight reads first (one LDS round trip instead of four), then the sum in wave order
+    f32x4 part[kWaves];
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) part[ww] = red[(q * kWaves + ww) * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ww = 0; ww < kWaves; ++ww) sum += red[(q * kWaves + ww) * 64 + lane];
+    for (int ww = 0; ww < kWaves; ++ww) sum += part[ww];
     if (i < count) astream_finish_tile<T, MT>(p, sum, nt_begin + i, mt, lane);
   }
 }
@@ -491,9 +496,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   for (int q = wave; q < kTiles; q += kWaves) {
     const int i = q / MT, mt = q - i * MT;
     const f32x4* src = q < kFirst ? red0 + q * kWaves * 64 : red1 + (q - kFirst) * kWaves * 64;
+    // all eight reads first (one LDS round trip instead of four), then the sum in wave order
+    f32x4 part[kWaves];
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) part[ww] = src[ww * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ww = 0; ww < kWaves; ++ww) sum += src[ww * 64 + lane];
+    for (int ww = 0; ww < kWaves; ++ww) sum += part[ww];
     if (i < count) astream_finish_tile<T, MT>(p, sum, nt_begin + i, mt, lane);
   }
 }
