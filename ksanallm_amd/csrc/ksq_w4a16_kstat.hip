@@ -44,6 +44,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   using O = Ops<T>;
   constexpr int DPG = 4 / GPT;
   constexpr int D = NB * TPW;  // ring depth = one batch
+  constexpr bool kRowSums = MT == 1 && TPW * GPT <= 2 && D <= 4;  // see the prologue (where the registers allow)
   static_assert(NB * MT * NW <= 64 && NB * MT <= NW && NW % (NB * MT) == 0, "reduction: two buffers of <= 64 KiB");
   __shared__ f32x4 red[2 * NB * MT * NW * 64];
 
@@ -172,6 +173,30 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
       }
   }
 
+  // Bias and zero point: the nibbles enter the matrix instruction as bias + u, so every (column, group) owes
+  // -sum_k a_k (bias_k + z).  With one row tile and few k tiles per wave the two sums over the wave's activations,
+  // sum_k a_k and -sum_k a_k bias_k (the bias alternates between 1024 and 64 inside a word for fp16), are computed
+  // once here, by the matrix cores against constant operands, and every (column tile, group) starts its
+  // accumulator from -z sum_k a_k - sum_k a_k bias_k: half the matrix instructions of the loop.  Elsewhere the
+  // registers for the sums are not there, and the correction stays a second matrix instruction per 32-k step.
+  f32x4 asum[kRowSums ? TPW : 1][GPT], abias[kRowSums ? TPW : 1][GPT];
+  if constexpr (kRowSums) {
+    const uint32_t ones = O::kOnes;
+    const u32x4 one4 = {ones, ones, ones, ones}, nbias = O::correction(0u);
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int gi = 0; gi < GPT; ++gi) {
+        asum[t][gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+        abias[t][gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dd = 0; dd < DPG; ++dd) {
+          asum[t][gi] = O::mfma(af[0][t][gi * DPG + dd], one4, asum[t][gi]);
+          abias[t][gi] = O::mfma(af[0][t][gi * DPG + dd], nbias, abias[t][gi]);
+        }
+      }
+  }
+
   uint16_t* out = static_cast<uint16_t*>(p.out);
   const int sz_lane = c * 4;
   for (int b = 0; b < nbatches; ++b) {
@@ -202,19 +227,32 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
         for (int gi = 0; gi < GPT; ++gi) {
           const uint32_t szw = szq[slot][gi];
           const uint32_t z = (szw >> 16) & 15u;
-          const u32x4 corr = O::correction(z | (z << 16));
           const float s = O::scale_to_float(szw);
           f32x4 P[MT];
+          if constexpr (kRowSums) {
+            // sum_k a (bias_k + u) starts from -sum_k a bias_k - z sum_k a, both sums known since the prologue
+            const float zf = (float)z;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int e = 0; e < 4; ++e) P[0][e] = __builtin_fmaf(-zf, asum[t][gi][e], abias[t][gi][e]);
 #pragma unroll
-          for (int dd = 0; dd < DPG; ++dd) {
-            const int d = gi * DPG + dd;
-            const u32x4 bw = O::unpack(wq[slot][d], m_lo, m_hi, c_lo, c_hi);
+            for (int dd = 0; dd < DPG; ++dd) {
+              const int d = gi * DPG + dd;
+              const u32x4 bw = O::unpack(wq[slot][d], m_lo, m_hi, c_lo, c_hi);
+              P[0] = O::mfma(af[0][t][d], bw, P[0]);
+            }
+          } else {
+            const u32x4 corr = O::correction(z | (z << 16));
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-              P[mt] = O::mfma(af[mt][t][d], corr, P[mt]);
-              P[mt] = O::mfma(af[mt][t][d], bw, P[mt]);
+            for (int mt = 0; mt < MT; ++mt) P[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int dd = 0; dd < DPG; ++dd) {
+              const int d = gi * DPG + dd;
+              const u32x4 bw = O::unpack(wq[slot][d], m_lo, m_hi, c_lo, c_hi);
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) {
+                P[mt] = O::mfma(af[mt][t][d], corr, P[mt]);
+                P[mt] = O::mfma(af[mt][t][d], bw, P[mt]);
+              }
             }
           }
 #pragma unroll
