@@ -346,7 +346,7 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
     }
   }
   if (m <= (size_t)env_int("KSQ_W4_KSTAT_MAX_M", 64) && env_int("KSQ_W4_KSTAT", 1) != 0) {
-    KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace_bytes);
+    KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace_bytes, g);
     if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s, epi);
   }
   W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace_bytes);

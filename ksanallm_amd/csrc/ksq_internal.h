@@ -210,7 +210,9 @@ struct KstatPlan {
   int nb;        // column tiles per batch (= ring depth / tpw)
   size_t partial_bytes;
 };
-KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+// g = the group size where the caller knows it (it picks the batch size only; the workspace a plan needs does not
+// depend on it)
+KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, size_t g = 0);
 int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* act, const void* weight,
                        const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
                         const Epilogue& epi = Epilogue());

@@ -386,7 +386,7 @@ static bool env_round4() {
   return !(e && atoi(e) == 0);
 }
 
-KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, size_t g) {
   KstatPlan p{};
   const size_t ntiles = n / kTileN, ktiles = k / kTileK;
   p.ok = m >= 1 && m <= 64 && ntiles * 4 <= (size_t)kCountersPerSlot;
@@ -443,6 +443,11 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
     // the next in finer steps (measured at Llama-2-7B gate_up, eight tiles per workgroup: 14.0 -> 12.3 us at M = 1,
     // 15.0 -> 13.3 at M = 16; qkv, four tiles per workgroup, is 3 % faster in one batch)
     p.nb = p.nt_per_wg >= 5 ? 2 : (p.nt_per_wg >= 3 ? 4 : (p.nt_per_wg >= 2 ? 2 : 1));
+    // Two k tiles per wave and one group per k tile: batches of two keep the ring at four tiles, where the kernel
+    // takes bias and zero point from the activations' row sums instead of a second matrix instruction per step
+    // (Llama-2-7B qkv, three tiles per workgroup: 8.9 -> 8.3 us at M = 16, 8.1 -> 7.6 at one token).  Not with K
+    // split over workgroups, where every batch ends in a hand-over (Llama-3-70B o: 10.9 -> 11.7 us in batches of two).
+    if (g == kTileK && p.tpw == 2 && p.nb == 4 && ksplit == 1) p.nb = 2;
     if (p.tpw >= 3 && p.nb > 2) p.nb = 2;                       // register budget of 16 waves per workgroup
     if (p.tpw >= 4) p.nb = 1;
   } else {
