@@ -420,10 +420,11 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   // (beyond four with at most two k tiles per wave, where the batches are two tiles each, whole batches of two: six
   // tiles stay six -- at gate_up of Llama-2-7B 11.6 .. 11.9 us against 12.3 .. 13.0 with eight at M = 1, level at
   // M = 16; with four k tiles per wave, Llama-3-70B gate_up, sixteen tiles beat fourteen by 2 %)
-  // (and three tiles stay three where the kernel takes the row-sum form, see below: a workgroup on every CU, one
-  // tile a batch -- Llama-2-7B qkv at one token 7.5 -> 7.0 us, level at M = 16)
+  // (and three tiles stay three where a batch is one tile anyway: where the kernel takes the row-sum form, see below
+  // -- a workgroup on every CU, Llama-2-7B qkv at one token 7.5 -> 7.0 us and 8.2 -> 7.9 at M = 16 -- and with four k
+  // tiles per wave, Llama-3-70B qkv 11.7 -> 11.1 and 13.2 -> 12.4)
   const bool row_sums = p.mt == 1 && g == kTileK && p.tpw == 2 && ksplit == 1;
-  const bool three = row_sums && p.nt_per_wg == 3;
+  const bool three = p.mt == 1 && (row_sums || p.tpw >= 4) && p.nt_per_wg == 3;
   if (p.mt == 1 && p.nt_per_wg >= 3 && env_round4() && !three)
     p.nt_per_wg = (p.nt_per_wg <= 4 || p.tpw >= 3) ? (p.nt_per_wg + 3) & ~3 : (p.nt_per_wg + 1) & ~1;
   if (const char* e = tuning_env("KSQ_W4_KSTAT_NT_PER_WG")) {  // tuning / test override: "v" or "ntiles:v,ntiles:v"
