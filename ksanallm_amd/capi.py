@@ -43,45 +43,49 @@ class KsqError(RuntimeError):
 _lib = None
 
 
+def _bind(L):
+    """Declare the argument and result types of every entry point of include/ksq.h on a loaded library."""
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    psz = ctypes.POINTER(ctypes.c_size_t)
+    L.ksq_version.restype = ci
+    L.ksq_last_error_string.restype = ctypes.c_char_p
+    L.ksq_device_compute_units.restype = ci
+    L.ksq_w4a16_repack_sizes.argtypes = [sz, sz, sz, psz, psz]
+    L.ksq_w4a16_repack.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, vp, vp]
+    L.ksq_w4a16_repack_host.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, vp]
+    L.ksq_w4a16_workspace_bytes.argtypes = [sz, sz, sz, psz]
+    L.ksq_w4a16_gemm.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, sz, vp]
+    L.ksq_fp8_quantize.argtypes = [ci, vp, sz, sz, ci, vp, vp, vp]
+    L.ksq_fp8_rescale.argtypes = [vp, vp, sz, vp, vp, vp]
+    L.ksq_fp8_convert_weight.argtypes = [ci, vp, sz, sz, vp, vp, vp]
+    L.ksq_fp8_convert_weight_per_channel.argtypes = [ci, vp, sz, sz, vp, vp, vp]
+    L.ksq_fp8_merge_qkv_scales.argtypes = [ci, vp, vp, vp, sz, sz, sz, vp, sz, vp, vp]
+    L.ksq_fp8_workspace_bytes.argtypes = [sz, sz, sz, psz]
+    L.ksq_fp8_gemm.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, vp, sz, vp]
+    L.ksq_w4a16_repack_ex.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, ci, vp, vp, vp]
+    L.ksq_w4a16_repack_ex_host.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, ci, vp, vp]
+    L.ksq_gptq_act_order_perm.argtypes = [vp, sz, sz, vp]
+    L.ksq_permute_columns.argtypes = [vp, vp, vp, sz, sz, vp]
+    L.ksq_w4a16_workspace_bytes_ex.argtypes = [sz, sz, sz, ci, psz]
+    L.ksq_w4a16_gemm_ex.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, ci, vp, vp, sz, vp]
+    L.ksq_fp8_gemm_ex.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
+    L.ksq_interleave_halves.argtypes = [vp, vp, sz, sz, vp]
+    L.ksq_w4a16_gemm_static_scratch.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp]
+    L.ksq_fp8_gemm_dynamic_workspace_bytes.argtypes = [sz, sz, sz, psz]
+    L.ksq_fp8_gemm_dynamic.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
+    for name in EXPORTS:
+        if name not in ("ksq_last_error_string",):
+            getattr(L, name).restype = ci
+    return L
+
+
 def lib():
     """Load libksq.so; raises if it has not been built (there is no fallback path)."""
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise KsqError(ERR_HIP, f"{LIB_PATH} is missing: build it with `python -m ksanallm_amd.build`")
-        L = ctypes.CDLL(LIB_PATH)
-        vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
-        psz = ctypes.POINTER(ctypes.c_size_t)
-        L.ksq_version.restype = ci
-        L.ksq_last_error_string.restype = ctypes.c_char_p
-        L.ksq_device_compute_units.restype = ci
-        L.ksq_w4a16_repack_sizes.argtypes = [sz, sz, sz, psz, psz]
-        L.ksq_w4a16_repack.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, vp, vp]
-        L.ksq_w4a16_repack_host.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, vp]
-        L.ksq_w4a16_workspace_bytes.argtypes = [sz, sz, sz, psz]
-        L.ksq_w4a16_gemm.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, sz, vp]
-        L.ksq_fp8_quantize.argtypes = [ci, vp, sz, sz, ci, vp, vp, vp]
-        L.ksq_fp8_rescale.argtypes = [vp, vp, sz, vp, vp, vp]
-        L.ksq_fp8_convert_weight.argtypes = [ci, vp, sz, sz, vp, vp, vp]
-        L.ksq_fp8_convert_weight_per_channel.argtypes = [ci, vp, sz, sz, vp, vp, vp]
-        L.ksq_fp8_merge_qkv_scales.argtypes = [ci, vp, vp, vp, sz, sz, sz, vp, sz, vp, vp]
-        L.ksq_fp8_workspace_bytes.argtypes = [sz, sz, sz, psz]
-        L.ksq_fp8_gemm.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, vp, sz, vp]
-        L.ksq_w4a16_repack_ex.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, ci, vp, vp, vp]
-        L.ksq_w4a16_repack_ex_host.argtypes = [ci, vp, ci, vp, vp, ci, sz, sz, sz, vp, ci, vp, vp]
-        L.ksq_gptq_act_order_perm.argtypes = [vp, sz, sz, vp]
-        L.ksq_permute_columns.argtypes = [vp, vp, vp, sz, sz, vp]
-        L.ksq_w4a16_workspace_bytes_ex.argtypes = [sz, sz, sz, ci, psz]
-        L.ksq_w4a16_gemm_ex.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, ci, vp, vp, sz, vp]
-        L.ksq_fp8_gemm_ex.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
-        L.ksq_interleave_halves.argtypes = [vp, vp, sz, sz, vp]
-        L.ksq_w4a16_gemm_static_scratch.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp]
-        L.ksq_fp8_gemm_dynamic_workspace_bytes.argtypes = [sz, sz, sz, psz]
-        L.ksq_fp8_gemm_dynamic.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
-        for name in EXPORTS:
-            if name not in ("ksq_last_error_string",):
-                getattr(L, name).restype = ci
-        _lib = L
+        _lib = _bind(ctypes.CDLL(LIB_PATH))
     return _lib
 
 

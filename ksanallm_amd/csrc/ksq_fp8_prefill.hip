@@ -60,15 +60,26 @@ __device__ inline u32x4 raw_rsrc(const void* base, size_t bytes) {
   const uint64_t a = reinterpret_cast<uint64_t>(base);
   return u32x4{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)bytes, 0x00020000u};
 }
-__device__ inline uint32_t lds_addr(const void* p) {
+#if defined(KSQ_EMU)
+typedef uintptr_t lds_addr_t;  // host build: LDS is host memory
+__device__ inline lds_addr_t lds_addr(const void* p) { return reinterpret_cast<uintptr_t>(p); }
+__device__ inline void load_lds_opaque(u32x4 rsrc, lds_addr_t lds, uint32_t voff, uint32_t soff) {
+  const uint64_t base = (uint64_t)rsrc[0] | ((uint64_t)(rsrc[1] & 0xffffu) << 32);
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(base), 0, (int)rsrc[2], 0);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr) reinterpret_cast<void*>(lds), 16, voff, soff, 0, 0);
+}
+#else
+typedef uint32_t lds_addr_t;
+__device__ inline lds_addr_t lds_addr(const void* p) {
   return (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p);
 }
-__device__ inline void load_lds_opaque(u32x4 rsrc, uint32_t lds, uint32_t voff, uint32_t soff) {
+__device__ inline void load_lds_opaque(u32x4 rsrc, lds_addr_t lds, uint32_t voff, uint32_t soff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory");
 }
+#endif
 
 __device__ inline i32x8 join(u32x4 lo, u32x4 hi) {
   i32x8 v;
@@ -207,6 +218,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
     for (int t = 0; t < kNT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) epi[(4 * j + i) * kEpiStride + 16 * t + r] = acc[mt][t][i] * ws[t];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
       const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
@@ -218,6 +230,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * as;
       if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
     }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // ... and its reads, before the next row tile overwrites the slab
   }
 }
 

@@ -72,6 +72,20 @@ constexpr int kCounterSlots = 64;
 constexpr int kCountersPerSlot = 16384;
 unsigned* counter_slot_device_ptr(hipStream_t stream);  // the stream's region (device address) or nullptr
 
+// ---- the few places where the kernels speak to the compiler or the machine in assembly ----------------------------------
+// A host build of the kernels (the CPU emulation that the tests use to walk every kernel's addressing, KSQ_EMU) has
+// neither register classes nor wait counters; everything else in the kernels is plain C++ plus builtins.
+#if defined(KSQ_EMU)
+#define KSQ_PIN_SGPR(x) ((void)(x))
+#define KSQ_PIN_VGPR(x) ((void)(x))
+#define KSQ_WAIT_ALL_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)  // where the emulated lanes of a wave meet
+#else
+// keeps a constant in a scalar / vector register instead of rematerialising it as a literal at every use
+#define KSQ_PIN_SGPR(x) asm volatile("" : "+s"(x))
+#define KSQ_PIN_VGPR(x) asm volatile("" : "+v"(x))
+#define KSQ_WAIT_ALL_VMEM() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+#endif
+
 #if defined(__HIPCC__)
 // Split-K partial tiles cross workgroups (and XCDs, each with its own L2) through agent-scope relaxed atomics: the
 // stores write through and the loads miss the non-coherent caches, so no whole-cache write-back or invalidate is
@@ -122,7 +136,7 @@ __device__ inline void split_range(int total, int split, int ksplit, int* begin,
 // (Llama-2-7B o at M = 64 10.6 -> 31.7 us, down at M = 16 11.0 -> 15.2 us, Qwen-72B FP8 gate_up at M = 64 137 ->
 // 1432 us), so the hand-over stays with the atomics and the wait.
 __device__ inline bool splitk_arrive_last(unsigned* counter, int lane, int ksplit) {
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  KSQ_WAIT_ALL_VMEM();
   unsigned arrived = 0;
   if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   arrived = __builtin_amdgcn_readfirstlane(arrived);

@@ -167,10 +167,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   };
 
   uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
-  asm volatile("" : "+s"(m_lo));
-  asm volatile("" : "+v"(c_lo));
-  asm volatile("" : "+v"(c_hi));
-  asm volatile("" : "+v"(m_hi));
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(c_lo);
+  KSQ_PIN_VGPR(c_hi);
+  KSQ_PIN_VGPR(m_hi);
 
   f32x4 acc[CNT][MT];
 #pragma unroll
@@ -395,10 +395,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   };
 
   uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
-  asm volatile("" : "+s"(m_lo));
-  asm volatile("" : "+v"(c_lo));
-  asm volatile("" : "+v"(c_hi));
-  asm volatile("" : "+v"(m_hi));
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(c_lo);
+  KSQ_PIN_VGPR(c_hi);
+  KSQ_PIN_VGPR(m_hi);
 
   f32x4 acc[CNT][MT];
 #pragma unroll

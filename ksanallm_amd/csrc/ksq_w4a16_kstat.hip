@@ -60,17 +60,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   count = count < p.nt_per_wg ? count : p.nt_per_wg;
   const int nbatches = (p.nt_per_wg + NB - 1) / NB;  // same for every workgroup
 
-  // Resources start at (nt_begin, kt0) and end with the wave's tiles of the last column tile of the workgroup, so
-  // column tiles past the range read as zero; k tiles past the end of the split are parked at an offset that stays
-  // out of range for every column tile (the range is far below 2^31 bytes).
+  // Resources start at (nt_begin, kt0) and end with the wave's live k tiles of the last column tile of the workgroup,
+  // so column tiles past the range read as zero: the prefetch of column tile `count` lands KT tiles further on, and
+  // KT >= live.  (With TPW in place of `live` a wave with fewer live k tiles than TPW -- K = 128 under an
+  // instantiation with two k tiles per wave -- had tile `count` in range, and the last workgroup read 1 KiB past the
+  // end of the weights and 64 GPT bytes past the scale/zero words.)  k tiles past the end of the split are parked at
+  // an offset that stays out of range for every column tile (the range is far below 2^31 bytes).
   const size_t kt0c = kt0 < p.KT ? (size_t)kt0 : (size_t)p.KT - 1;
   const char* wb = static_cast<const char*>(p.weight) + ((size_t)nt_begin * p.KT + kt0c) * 1024;
   const char* sb = static_cast<const char*>(p.sz) + ((size_t)nt_begin * p.G + kt0c * GPT) * 64;
   const bool any = count > 0 && kt0 < wg_end;
+  const int live = wg_end - kt0 < TPW ? wg_end - kt0 : TPW;
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(wb), 0, any ? ((count - 1) * p.KT + TPW) * 1024 : 0, 0x00020000);
+      const_cast<char*>(wb), 0, any ? ((count - 1) * p.KT + live) * 1024 : 0, 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_sz = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(sb), 0, any ? ((count - 1) * p.G + TPW * GPT) * 64 : 0, 0x00020000);
+      const_cast<char*>(sb), 0, any ? ((count - 1) * p.G + live * GPT) * 64 : 0, 0x00020000);
   const __amdgpu_buffer_rsrc_t rs_a =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
   unsigned w_off[TPW];
@@ -124,10 +128,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   };
 
   uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
-  asm volatile("" : "+s"(m_lo));
-  asm volatile("" : "+v"(c_lo));
-  asm volatile("" : "+v"(c_hi));
-  asm volatile("" : "+v"(m_hi));
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(c_lo);
+  KSQ_PIN_VGPR(c_hi);
+  KSQ_PIN_VGPR(m_hi);
 
   __builtin_amdgcn_sched_barrier(0);
   // With more than one batch per workgroup, every wave's activation loads are issued before any wave's weight

@@ -249,10 +249,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 
   uint32_t m_lo = Ops<_Float16>::kMaskLo, m_hi = Ops<_Float16>::kMaskHi, g_lo = Ops<_Float16>::kMagicLo,
            g_hi = Ops<_Float16>::kMagicHi;
-  asm volatile("" : "+s"(m_lo));
-  asm volatile("" : "+v"(g_lo));
-  asm volatile("" : "+v"(g_hi));
-  asm volatile("" : "+v"(m_hi));
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(g_lo);
+  KSQ_PIN_VGPR(g_hi);
+  KSQ_PIN_VGPR(m_hi);
 
   // Activation fragments are read from LDS four at a time (half of the row tiles of one 32-k step), one half ahead
   // of the matrix instructions that use them, so that the LDS latency hides behind 16 MFMAs.
@@ -471,10 +471,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
 
   uint32_t m_lo = Ops<_Float16>::kMaskLo, m_hi = Ops<_Float16>::kMaskHi, g_lo = Ops<_Float16>::kMagicLo,
            g_hi = Ops<_Float16>::kMagicHi;
-  asm volatile("" : "+s"(m_lo));
-  asm volatile("" : "+v"(g_lo));
-  asm volatile("" : "+v"(g_hi));
-  asm volatile("" : "+v"(m_hi));
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(g_lo);
+  KSQ_PIN_VGPR(g_hi);
+  KSQ_PIN_VGPR(m_hi);
 
   auto read_step = [&](u32x4 (&a)[kRows], const u32x4* buf, int ks) {
 #pragma unroll

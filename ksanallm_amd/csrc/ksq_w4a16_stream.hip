@@ -137,10 +137,10 @@ w4a16_stream_kernel(StreamArgs p) {
 
   // constants of the unpack kept in registers so that each output register costs one v_and_or_b32
   uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
-  asm volatile("" : "+s"(m_lo));
-  asm volatile("" : "+v"(c_lo));
-  asm volatile("" : "+v"(c_hi));
-  asm volatile("" : "+v"(m_hi));
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(c_lo);
+  KSQ_PIN_VGPR(c_hi);
+  KSQ_PIN_VGPR(m_hi);
 
   // Software pipeline inside the wave.  A step issues the MFMAs of tile i from activation fragments that were
   // read from LDS at the end of step i - 1, and only then folds the group sums of tile i - 1 into the

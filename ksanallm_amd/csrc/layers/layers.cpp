@@ -177,8 +177,11 @@ Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, c
   size_t weight_bytes = 0, sz_bytes = 0;
   ThrowOnKsqError(ksq_w4a16_repack_sizes(k, n, groupsize, &weight_bytes, &sz_bytes), "ksq_w4a16_repack_sizes");
   if (scales.dtype != TYPE_FP16 && scales.dtype != TYPE_BF16) KLLM_THROW("RepackGroupQuantWeight: scales must be fp16 or bf16.");
-  CreateTensor(weight, {k, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);  // same shape as ksana's "*.weight"
-  CreateTensor(weight_sz, {k / groupsize, n}, TYPE_UINT32, rank, MEMORY_DEVICE);
+  // ksana's "*.weight" shape, with K rounded up to whole k tiles of 128 as the repack writes it (K = 64 x odd under
+  // group size 64 gains half a tile of padding: the sizes are the library's, never k * n / 2 computed here)
+  const size_t kp = weight_bytes / (n / 2);
+  CreateTensor(weight, {kp, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);
+  CreateTensor(weight_sz, {sz_bytes / (4 * n), n}, TYPE_UINT32, rank, MEMORY_DEVICE);
   const int src = KsqLayout(layout);
   if (perm != nullptr && (perm->dtype != TYPE_INT32 || perm->GetElementNumber() != k))
     KLLM_THROW("RepackGroupQuantWeight: perm must be int32 [k].");
@@ -212,8 +215,8 @@ Status RepackFusedGroupQuantWeight(GroupWeightLayout layout, const std::vector<G
   if (st != TYPE_FP16 && st != TYPE_BF16) KLLM_THROW("RepackFusedGroupQuantWeight: scales must be fp16 or bf16.");
   size_t weight_bytes = 0, sz_bytes = 0;
   ThrowOnKsqError(ksq_w4a16_repack_sizes(k, n, groupsize, &weight_bytes, &sz_bytes), "ksq_w4a16_repack_sizes");
-  CreateTensor(weight, {k, n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);
-  CreateTensor(weight_sz, {k / groupsize, n}, TYPE_UINT32, rank, MEMORY_DEVICE);
+  CreateTensor(weight, {weight_bytes / (n / 2), n / 2}, TYPE_UINT8, rank, MEMORY_DEVICE);  // K in whole k tiles
+  CreateTensor(weight_sz, {sz_bytes / (4 * n), n}, TYPE_UINT32, rank, MEMORY_DEVICE);
   size_t n0 = 0;
   for (const GroupWeightPart& part : parts) {
     // columns n0 .. n0 + part.n - 1 are the column tiles n0 / 16 .. of the fused buffers: a contiguous range of each

@@ -62,6 +62,13 @@ class W4Case:
         return orc.dequant(self.u, self.scales, ORC_DT[self.dtype], self.z, self.g)
 
 
+def _sync(device):
+    import torch
+
+    if torch.device(device).type == "cuda":
+        torch.cuda.synchronize()
+
+
 class W4Device:
     """The case on the GPU: repacked through ksq_w4a16_repack from the layout native to its kind."""
 
@@ -92,7 +99,7 @@ class W4Device:
         else:
             zk, zeros = capi.ZERO_UINT8, torch.from_numpy(c.z).to(device)
         capi.w4a16_repack(lay, src, zk, zeros, scales, capi_dtype(c.dtype), c.K, c.N, c.g, self.weight, self.sz)
-        torch.cuda.synchronize()
+        _sync(device)
         self.act = torch.from_numpy(c.act.view(np.int16)).to(device).view(torch_dtype(c.dtype))
         ws = capi.w4a16_workspace_bytes(max(c.M, 1), c.N, c.K)
         self.workspace = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)
@@ -109,7 +116,7 @@ class W4Device:
         out = torch.full((m, c.N), float("nan"), dtype=torch_dtype(c.dtype), device=self.device)
         capi.w4a16_gemm(capi_dtype(c.dtype), out, act, self.weight, self.sz, m, c.N, c.K, c.g,
                         self.workspace if use_workspace else None, self.workspace_bytes if use_workspace else 0)
-        torch.cuda.synchronize()
+        _sync(self.device)
         return out
 
     def gemm_f32(self, **kw):

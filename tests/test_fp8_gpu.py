@@ -334,7 +334,7 @@ def test_merge_qkv_scales(gpu):
     wq[(wq & 0x7F) == 0x7F] = 0x2a
     scales = [np.array([v], dtype=np.float32) for v in (0.021, 0.0503, 0.0127)]
     d_scales = [torch.from_numpy(x).to(gpu) for x in scales]
-    dw = torch.from_numpy(wq).to(gpu)
+    dw = torch.from_numpy(wq.copy()).to(gpu)  # rescaled in place: never the host array itself
     out_s = torch.zeros(1, dtype=torch.float32, device=gpu)
     capi.fp8_merge_qkv_scales(capi.FP8_MERGE_MAX, *d_scales, nq, nk, nv, dw, K, out_s)
     torch.cuda.synchronize()
@@ -344,7 +344,7 @@ def test_merge_qkv_scales(gpu):
     nz = (want_w & 0x7F) != 0
     assert np.array_equal(got[nz], want_w[nz]) and np.all((got[~nz] & 0x7F) == 0)
 
-    dw2 = torch.from_numpy(wq).to(gpu)
+    dw2 = torch.from_numpy(wq.copy()).to(gpu)
     chan = torch.zeros(nq + nk + nv, dtype=torch.float32, device=gpu)
     capi.fp8_merge_qkv_scales(capi.FP8_MERGE_PER_CHANNEL, *d_scales, nq, nk, nv, None, K, chan)
     torch.cuda.synchronize()

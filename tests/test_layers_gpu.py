@@ -102,6 +102,38 @@ def test_group_matmul_layer_widened(gpu, tmp_path, dtype, extra, layout, M):
     orc.assert_parity(got, want, f"GroupMatMulLayer {layout} {extra} {dtype}")
 
 
+@pytest.mark.parametrize("dtype,M,parts", [("f16", 16, None), ("bf16", 70, None), ("f16", 5, [64, 32, 32]),
+                                           ("bf16", 130, [64, 64])])
+def test_group_matmul_layer_k_not_a_multiple_of_128(gpu, tmp_path, dtype, M, parts):
+    """K = 192 under group size 64: the repack pads the last k tile, so the repacked tensors are larger than
+    k * n / 2 bytes and k / g * n words -- the layer must size them as the library says (single and fused weight)."""
+    _odd_k_case(_run, tmp_path, dtype, M, parts)
+
+
+def _odd_k_case(run, tmp_path, dtype, M, parts):
+    K, g = 192, 64
+    N = sum(parts) if parts else 128
+    case = W4Case(640 + M, M, K, N, g=g, kind="awq", dtype=dtype)
+    d = str(tmp_path)
+    n0 = 0
+    for i, w in enumerate(parts or []):
+        orc.awq_pack(np.ascontiguousarray(case.u[:, n0:n0 + w])).tofile(f"{d}/qweight_{i}.bin")
+        orc.awq_pack(np.ascontiguousarray(case.z[:, n0:n0 + w])).tofile(f"{d}/qzeros_{i}.bin")
+        np.ascontiguousarray(case.scales[:, n0:n0 + w]).tofile(f"{d}/scales_{i}.bin")
+        n0 += w
+    case.awq_qweight().tofile(d + "/qweight.bin")
+    case.awq_qzeros().tofile(d + "/qzeros.bin")
+    case.scales.tofile(d + "/scales.bin")
+    case.act.tofile(d + "/act.bin")
+    args = ["w4a16", d, dtype, M, K, N, g, "awq", "awq", "awq"]
+    if parts:
+        args.append("parts:" + ":".join(map(str, parts)))
+    rc, out = run(args)
+    assert rc == 0 and out.splitlines()[-1] == f"OK {M} {N} {DTYPE_ENUM[dtype]}", out
+    got = orc.from_bits(np.fromfile(d + "/out.bin", dtype=np.uint16).reshape(M, N), ORC_DT[dtype])
+    orc.assert_parity(got, case.oracle(), f"GroupMatMulLayer K=192 g=64 {dtype} parts={parts}")
+
+
 @pytest.mark.parametrize("dtype,M", [("f16", 16), ("bf16", 70)])
 def test_group_matmul_layer_fused_from_separate_projections(gpu, tmp_path, dtype, M):
     """q_proj / k_proj / v_proj of an AWQ checkpoint as three tensors, repacked side by side into one fused weight
