@@ -58,6 +58,7 @@ class Layer:
     """One decoder layer's four AWQ weights, generated on the GPU and repacked through the C ABI."""
 
     def __init__(self, torch, capi, device, seed, dtype, keep_source=False):
+        self.dtype = dtype
         self.weights = []
         self.source = []
         gen = torch.Generator(device=device)
@@ -223,8 +224,9 @@ def prefill_shape(torch, capi, stream, k, n, w, sz, M, dtype_name, gen):
 
 def prefill(torch, capi, layer, stream, gen, dtype_name="bf16", M=4096):
     """configs[2] (bf16 activations, M = 512 / 2048 / 4096): TFLOP/s per shape against the dense MFMA peak, bf16
-    conversion kernel included.  The weights are the fp16-scaled set of layer 0 re-used with bf16 activations only for
-    timing (the arithmetic is the same); weight copies rotate, activations and outputs do not."""
+    conversion kernel included.  `layer` has to be repacked for the element type of the leg (bf16 scales carry a
+    column exponent that the fp16-scaled set does not); weight copies rotate, activations and outputs do not."""
+    assert layer.dtype == (capi.BF16 if dtype_name == "bf16" else capi.F16), "weights repacked for the other element type"
     table = {}
     for name, k, n, w, sz in layer.weights:
         us = prefill_shape(torch, capi, stream, k, n, w, sz, M, dtype_name, gen)
@@ -246,10 +248,21 @@ def mfma_half(table):
             "per_shape": {name: table[name]["TFLOPs"] for name, _, _ in SHAPES_7B}}
 
 
-def fp8_weights(torch, dev, gen, k, n):
+def fp8_weights(torch, capi, dev, gen, k, n):
+    """configs[4]: weights N(0,1) * 0.02 in bf16, [k, n], converted by the library's own load-time step
+    (ksq_fp8_convert_weight_per_channel: transpose to [n, k] e4m3 with one fp32 scale per output channel); enough
+    distinct copies that no launch finds its weights in the last-level cache."""
     ncopies = ncopies_for(k * n)
-    ws = [torch.randint(0, 120, (n, k), dtype=torch.uint8, device=dev, generator=gen) for _ in range(ncopies)]
-    wscale = torch.rand(n, device=dev, generator=gen) * 0.01 + 1e-3
+    ws, wscale = [], None
+    for _ in range(ncopies):
+        src = (torch.randn((k, n), device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        wq = torch.empty((n, k), dtype=torch.uint8, device=dev)
+        sc = torch.empty(n, dtype=torch.float32, device=dev)
+        capi.fp8_convert_weight_per_channel(capi.BF16, src, k, n, wq, sc)
+        torch.cuda.synchronize()
+        del src
+        ws.append(wq)
+        wscale = sc  # the copies differ in bytes, not in distribution: one scale vector serves the timing
     return ws, wscale
 
 
@@ -293,7 +306,7 @@ def fp8_sweep(torch, capi, dev, stream):
     gen.manual_seed(3)
     table = {}
     for name, k, n in SHAPES_72B:
-        ws, wscale = fp8_weights(torch, dev, gen, k, n)
+        ws, wscale = fp8_weights(torch, capi, dev, gen, k, n)
         row = {"copies": len(ws)}
         for M in (1, 64, 256, 2048):
             uq, ug, ud = fp8_case(torch, capi, dev, stream, gen, ws, wscale, k, n, M, 32 if M <= 64 else (16 if M < 2048 else 4))
@@ -430,7 +443,7 @@ def run_only(torch, capi, dev, stream, leg):
         if parts[1] == "prefill":
             shape, M, dt = parts[2] if parts[2] != "gate" else "gate_up", int(parts[-2][1:]), parts[-1]
             name, k, n = next(s for s in SHAPES_7B if s[0] == shape)
-            layer = Layer(torch, capi, dev, 1000, capi.F16)
+            layer = Layer(torch, capi, dev, 1000, capi.BF16 if dt == "bf16" else capi.F16)
             _, _, _, w, sz = next(x for x in layer.weights if x[0] == shape)
             us = prefill_shape(torch, capi, stream, k, n, w, sz, M, dt, gen)
             tf = 2.0 * M * k * n / us / 1e6
@@ -453,7 +466,7 @@ def run_only(torch, capi, dev, stream, leg):
         shape = "gate_up" if parts[1] == "gate" else parts[1]
         M = int(parts[-1][1:])
         name, k, n = next(s for s in SHAPES_72B if s[0] == shape)
-        ws, wscale = fp8_weights(torch, dev, gen, k, n)
+        ws, wscale = fp8_weights(torch, capi, dev, gen, k, n)
         uq, ug, ud = fp8_case(torch, capi, dev, stream, gen, ws, wscale, k, n, M, 32 if M <= 64 else 4)
         if M <= 64:
             b = fp8_bytes(M, k, n)
@@ -512,6 +525,14 @@ def main():
         for _, k, n, w, sz in layers[i % len(layers)].weights:
             capi.w4a16_gemm(dtype, outs[n], acts[k], w, sz, M, n, k, GROUP, workspace, ws_bytes, sp)
 
+    # which kernel instantiation serves each GEMM of the step (the library's launch log, read back per call)
+    capi.set_launch_log(True)
+    launched = {}
+    for name, k, n, w, sz in layers[0].weights:
+        capi.w4a16_gemm(dtype, outs[n], acts[k], w, sz, M, n, k, GROUP, workspace, ws_bytes, sp)
+        launched[name] = capi.last_launch()
+    capi.set_launch_log(False)
+
     with torch.cuda.stream(stream):
         for i in range(args.warmup):
             step(i)
@@ -546,11 +567,19 @@ def main():
     launches = args.steps * len(SHAPES_7B)
     avg_launch_us = gpu_ms * 1e3 / launches
     achieved = (step_bytes / len(SHAPES_7B)) / (avg_launch_us * 1e-6) / 1e9
-    traffic = None
+    # HBM traffic per launch comes from a rocprofv3 --pmc run of this same command (profiles/): it is attached only if
+    # that run launched the very kernel instantiations that this run did
+    traffic, traffic_note, profiled = None, None, {}
     if os.path.exists(TRAFFIC_FILE):
         for line in open(TRAFFIC_FILE):
             if line.startswith("traffic_bytes_per_launch:"):
                 traffic = float(line.split(":")[1])
+            if line.startswith("launched "):
+                name, what = line[len("launched "):].split(":", 1)
+                profiled[name.strip()] = what.strip()
+        if profiled != launched:
+            traffic = None
+            traffic_note = "profiles/ was taken with other kernel instantiations than this run launched: not attached"
 
     result = {
         "metric": METRIC,
@@ -582,14 +611,19 @@ def main():
             "traffic": traffic,
             "avg_launch_us": round(avg_launch_us, 3),
             "launches": launches,
+            "launched": launched,
         },
     }
+    if traffic_note:
+        result["roofline"]["traffic_note"] = traffic_note
     if args.only == "headline":
         print(json.dumps(result), flush=True)
         return
 
-    # the TFLOP/s half of the metric: always measured, carried inside `roofline`
-    m4096 = prefill(torch, capi, layers[0], stream, gen)
+    # the TFLOP/s half of the metric: always measured, carried inside `roofline`; configs[2] has bf16 activations, so
+    # its weights are repacked with bf16 scales (the same values cast)
+    layer_bf16 = Layer(torch, capi, dev, 1000, capi.BF16)
+    m4096 = prefill(torch, capi, layer_bf16, stream, gen)
     result["roofline"]["mfma"] = mfma_half(m4096)
 
     extra = {}
@@ -601,9 +635,11 @@ def main():
                 extra[f"decode_m{m2}"] = per_shape(torch, capi, layers[0], stream, m2, dtype, gen)
         extra["fused_m16"] = fused(torch, capi, layers[0], stream, M, dtype, dev, gen)
         extra["prefill_m4096_f16"] = prefill(torch, capi, layers[0], stream, gen, "f16")
-        extra["prefill_m2048"] = prefill(torch, capi, layers[0], stream, gen, M=2048)
-        extra["prefill_m512"] = prefill(torch, capi, layers[0], stream, gen, M=512)
-        extra["prefill_m128"] = prefill(torch, capi, layers[0], stream, gen, M=128)  # between configs[1] and [2]
+        extra["prefill_m2048"] = prefill(torch, capi, layer_bf16, stream, gen, M=2048)
+        extra["prefill_m512"] = prefill(torch, capi, layer_bf16, stream, gen, M=512)
+        extra["prefill_m128"] = prefill(torch, capi, layer_bf16, stream, gen, M=128)  # between configs[1] and [2]
+        extra["prefill_m512_f16"] = prefill(torch, capi, layers[0], stream, gen, "f16", M=512)
+        del layer_bf16
         del layers[1:]
         torch.cuda.empty_cache()
         extra["fp8_cfg4"] = fp8_sweep(torch, capi, dev, stream)

@@ -116,6 +116,25 @@ const char* ksq_last_error_string(void);
 /* Number of the compute units of the current device that the launch heuristics use (0 on failure). */
 int ksq_device_compute_units(void);
 
+/* Diagnostics (no counterpart in the reference): with the log switched on, every GEMM entry point records what it
+ * launched -- kernel, template arguments, grid -- and ksq_last_launch_string() returns that of the calling thread's last
+ * GEMM call ("" before the first).  Off by default: the launch path then formats nothing. */
+void ksq_set_launch_log(int enabled);
+const char* ksq_last_launch_string(void);
+
+/* Split-K arrival counters in the caller's memory (no counterpart in the reference; its split-K semaphores live in the
+ * workspace of every call, LK/asymmetric_gemm/fpA_intB_gemm/fpA_intB_gemm_template.h:498-504).
+ * The kernels that split K across workgroups count arrivals in device memory that has to be zero between launches;
+ * they return it to zero themselves.  By default that memory is the library's, one region per stream.  A caller can
+ * bind KSQ_SPLITK_COUNTER_BYTES of its own device memory (256-byte aligned, zero-filled once by the caller) to a
+ * stream: every later GEMM call on that stream -- and every graph captured from it while the binding holds -- uses it.
+ * That is how two graphs captured from one stream can be replayed at the same time (bind different memory before each
+ * capture), how more streams than the library has regions keep their split-K plans, and how a process recovers after
+ * a kernel was aborted mid-flight (bind freshly zeroed memory).  counters == NULL removes the binding.  The memory
+ * must stay valid while a launch or a captured graph that uses it can still run. */
+#define KSQ_SPLITK_COUNTER_BYTES 65536
+int ksq_bind_splitk_counters(void* stream, void* counters, size_t bytes);
+
 /* ------------------------------------------------------------------ W4A16: load-time repack
  *
  * Replaces CutlassPreprocessWeightsForMixedGemmWarpper / preprocess_weights_for_mixed_gemm
@@ -185,7 +204,8 @@ int ksq_permute_columns(void* out, const void* in, const int32_t* perm, size_t m
  * each.  The arrival counters of the split-K kernels are library-owned device memory, one region per stream (the
  * first 64 streams per device that launch a split-K kernel; later streams get the same results without split-K):
  * launches on one stream never overlap, so no launch shares counters with one in flight -- with one exception:
- * two HIP graphs captured from the same stream and replayed at the same time on different streams would. */
+ * two HIP graphs captured from the same stream and replayed at the same time on different streams would, unless the
+ * caller binds counters of its own before each capture (ksq_bind_splitk_counters above). */
 int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes);
 
 int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,

@@ -30,7 +30,9 @@ EXPORTS = [
     "ksq_w4a16_repack_ex", "ksq_w4a16_repack_ex_host", "ksq_gptq_act_order_perm", "ksq_permute_columns",
     "ksq_w4a16_workspace_bytes_ex", "ksq_w4a16_gemm_ex", "ksq_fp8_gemm_ex", "ksq_interleave_halves",
     "ksq_w4a16_gemm_static_scratch", "ksq_fp8_gemm_dynamic_workspace_bytes", "ksq_fp8_gemm_dynamic",
+    "ksq_set_launch_log", "ksq_last_launch_string", "ksq_bind_splitk_counters",
 ]
+SPLITK_COUNTER_BYTES = 65536
 STATIC_SCRATCH_BYTES = 64 << 20
 
 
@@ -73,8 +75,12 @@ def _bind(L):
     L.ksq_w4a16_gemm_static_scratch.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp]
     L.ksq_fp8_gemm_dynamic_workspace_bytes.argtypes = [sz, sz, sz, psz]
     L.ksq_fp8_gemm_dynamic.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, ci, vp, vp, sz, vp]
+    L.ksq_set_launch_log.argtypes = [ci]
+    L.ksq_set_launch_log.restype = None
+    L.ksq_last_launch_string.restype = ctypes.c_char_p
+    L.ksq_bind_splitk_counters.argtypes = [vp, vp, sz]
     for name in EXPORTS:
-        if name not in ("ksq_last_error_string",):
+        if name not in ("ksq_last_error_string", "ksq_set_launch_log", "ksq_last_launch_string"):
             getattr(L, name).restype = ci
     return L
 
@@ -108,6 +114,21 @@ def _check(code):
 
 def version():
     return lib().ksq_version()
+
+
+def set_launch_log(enabled=True):
+    lib().ksq_set_launch_log(1 if enabled else 0)
+
+
+def last_launch():
+    """What the calling thread's last GEMM call launched (needs set_launch_log first)."""
+    return lib().ksq_last_launch_string().decode()
+
+
+def bind_splitk_counters(stream, counters, nbytes=None):
+    """Bind caller-owned, zero-filled device memory as the split-K arrival counters of `stream` (None unbinds)."""
+    n = 0 if counters is None else (nbytes if nbytes is not None else counters.numel() * counters.element_size())
+    _check(lib().ksq_bind_splitk_counters(stream, _addr(counters), n))
 
 
 def device_compute_units():

@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 
 #include "ksq_internal.h"
@@ -19,6 +20,23 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+static std::atomic<int> g_launch_log{0};
+static thread_local char g_launch[384] = "";
+
+void note_launch(const char* fmt, ...) {
+  if (!g_launch_log.load(std::memory_order_relaxed)) return;
+  const size_t used = strlen(g_launch);
+  if (used + 2 >= sizeof(g_launch)) return;
+  if (used) {  // several launches behind one entry point: "a + b"
+    memcpy(g_launch + used, " + ", 4);
+  }
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_launch + strlen(g_launch), sizeof(g_launch) - strlen(g_launch), fmt, ap);
+  va_end(ap);
+}
+void reset_launch_note() { g_launch[0] = 0; }
+
 // ---- per-device state -----------------------------------------------------------------------------------------
 static __device__ __align__(256) unsigned g_splitk_counters[kCounterSlots * kCountersPerSlot];
 // Scratch of ksq_w4a16_gemm_static_scratch: stands in for the caller's workspace.  In host code this name is only a
@@ -27,6 +45,7 @@ static __device__ __align__(256) unsigned char g_static_scratch[KSQ_STATIC_SCRAT
 
 namespace {
 constexpr int kMaxDevices = 16;
+constexpr int kMaxBoundStreams = 256;
 struct PerDevice {
   std::once_flag once;
   bool ok = false;
@@ -36,6 +55,9 @@ struct PerDevice {
   std::mutex slot_mutex;
   int slots_used = 0;
   hipStream_t slot_owner[kCounterSlots] = {};
+  int bound_used = 0;  // caller-owned counters, by stream (ksq_bind_splitk_counters)
+  hipStream_t bound_stream[kMaxBoundStreams] = {};
+  unsigned* bound_ptr[kMaxBoundStreams] = {};
 };
 PerDevice g_dev[kMaxDevices];
 
@@ -71,10 +93,14 @@ const DeviceInfo* device_info() {
   return pd ? &pd->info : nullptr;
 }
 
+// A stream's counters: the caller's own (ksq_bind_splitk_counters) if it bound any, else the stream's region of the
+// library's array, claimed on first use.
 unsigned* counter_slot_device_ptr(hipStream_t stream) {
   PerDevice* pd = current_device_state();
   if (!pd) return nullptr;
   std::lock_guard<std::mutex> lock(pd->slot_mutex);
+  for (int i = 0; i < pd->bound_used; ++i)
+    if (pd->bound_stream[i] == stream && pd->bound_ptr[i]) return pd->bound_ptr[i];
   int slot = 0;
   while (slot < pd->slots_used && pd->slot_owner[slot] != stream) ++slot;
   if (slot == pd->slots_used) {
@@ -82,6 +108,38 @@ unsigned* counter_slot_device_ptr(hipStream_t stream) {
     pd->slot_owner[pd->slots_used++] = stream;
   }
   return pd->counters + (size_t)slot * kCountersPerSlot;
+}
+
+// Whether counter_slot_device_ptr would succeed, without claiming a region: the planners ask before they plan a split,
+// the launchers claim when a split is in the plan, so a stream that never splits never owns a region.
+bool counter_slot_available(hipStream_t stream) {
+  PerDevice* pd = current_device_state();
+  if (!pd) return false;
+  std::lock_guard<std::mutex> lock(pd->slot_mutex);
+  for (int i = 0; i < pd->bound_used; ++i)
+    if (pd->bound_stream[i] == stream && pd->bound_ptr[i]) return true;
+  for (int slot = 0; slot < pd->slots_used; ++slot)
+    if (pd->slot_owner[slot] == stream) return true;
+  return pd->slots_used < kCounterSlots;
+}
+
+static int bind_counters(hipStream_t stream, unsigned* counters) {
+  PerDevice* pd = current_device_state();
+  if (!pd) return KSQ_ERR_HIP;
+  std::lock_guard<std::mutex> lock(pd->slot_mutex);
+  int i = 0;
+  while (i < pd->bound_used && pd->bound_stream[i] != stream) ++i;
+  if (i == pd->bound_used) {
+    if (counters == nullptr) return KSQ_OK;  // nothing bound: nothing to undo
+    int free_i = 0;
+    while (free_i < pd->bound_used && pd->bound_ptr[free_i]) ++free_i;  // reuse an unbound entry
+    i = free_i;
+    if (i == kMaxBoundStreams) return fail(KSQ_ERR_UNSUPPORTED, "%d streams already have counters bound", kMaxBoundStreams);
+    if (i == pd->bound_used) ++pd->bound_used;
+    pd->bound_stream[i] = stream;
+  }
+  pd->bound_ptr[i] = counters;
+  return KSQ_OK;
 }
 
 static unsigned char* static_scratch_device_ptr() {
@@ -196,6 +254,18 @@ int ksq_version(void) { return 100; }
 
 const char* ksq_last_error_string(void) { return g_error; }
 
+void ksq_set_launch_log(int enabled) { g_launch_log.store(enabled ? 1 : 0); }
+
+const char* ksq_last_launch_string(void) { return g_launch; }
+
+int ksq_bind_splitk_counters(void* stream, void* counters, size_t bytes) {
+  KSQ_REQUIRE(counters == nullptr || bytes >= (size_t)KSQ_SPLITK_COUNTER_BYTES, KSQ_ERR_INVALID_ARGUMENT,
+              "%zu bytes of counters; %zu are needed", bytes, (size_t)KSQ_SPLITK_COUNTER_BYTES);
+  KSQ_REQUIRE((reinterpret_cast<uintptr_t>(counters) & 255) == 0, KSQ_ERR_INVALID_ARGUMENT,
+              "counters must be 256-byte aligned");
+  return bind_counters(static_cast<hipStream_t>(stream), static_cast<unsigned*>(counters));
+}
+
 int ksq_device_compute_units(void) {
   const DeviceInfo* di = device_info();
   return di ? di->cus : 0;
@@ -278,6 +348,7 @@ int ksq_w4a16_workspace_bytes_ex(size_t max_m, size_t n, size_t k, int act_order
 int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
                       size_t k, size_t g, const int32_t* act_perm, int epilogue, const void* bias, void* workspace,
                       size_t workspace_bytes, void* stream) {
+  reset_launch_note();
   KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
   KSQ_REQUIRE(out && act && weight && sz, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
   KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
@@ -332,7 +403,7 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, workspace_bytes, s, epi);
   // The kernels below split K across workgroups through arrival counters owned per stream; a stream that got none
   // (more streams than counter regions) is planned as if it had no workspace: same results, no split.
-  if (workspace_bytes && !counter_slot_device_ptr(s)) workspace_bytes = 0;
+  if (workspace_bytes && !counter_slot_available(s)) workspace_bytes = 0;
   if (w4a16_astream_supported(m, n, k)) {
     // Measured on Llama-2 7B and 70B shapes: with three or four row tiles the accumulator-stationary kernel is
     // never slower than the k-stationary one.  With two it wins while every workgroup gets one to four column

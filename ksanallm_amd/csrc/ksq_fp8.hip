@@ -643,7 +643,7 @@ int ksq_fp8_gemm_dynamic(int dtype, void* out, const void* act, const void* w_q,
   const char* sw = tuning_env("KSQ_FP8_FUSED_QUANT");  // tuning / test switch: 0 = never, 1 = up to eight rows
   const size_t fused_rows = sw ? (atoi(sw) == 0 ? 0 : 8) : 1;
   if (m <= fused_rows && k % 128 == 0 && m * k * 2 < 0x7FFFFF00ull) {
-    if (gemm_ws && !counter_slot_device_ptr(s)) gemm_ws = nullptr, gemm_ws_bytes = 0;
+    if (gemm_ws && !counter_slot_available(s)) gemm_ws = nullptr, gemm_ws_bytes = 0;
     const Fp8KstatPlan kp = fp8_kstat_plan(m, n, k, di->cus, gemm_ws_bytes, true);
     if (kp.ok && kp.nb <= 2 && kp.tpw <= 4 && (kp.ksplit == 1 || sw)) {
       Epilogue epi;
@@ -674,6 +674,7 @@ int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_s
 int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
                     const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
                     int epilogue, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+  reset_launch_note();
   KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
               "bad epilogue %d", epilogue);
   KSQ_REQUIRE(epilogue != KSQ_EPILOGUE_BIAS || (bias && (reinterpret_cast<uintptr_t>(bias) & 15) == 0),
@@ -704,7 +705,7 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
                               workspace, workspace ? workspace_bytes : 0, static_cast<hipStream_t>(stream), epi);
   if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) workspace = nullptr;
   // split-K needs the stream's arrival counters; a stream that got none is planned as if it had no workspace
-  if (workspace && !counter_slot_device_ptr(static_cast<hipStream_t>(stream))) workspace = nullptr;
+  if (workspace && !counter_slot_available(static_cast<hipStream_t>(stream))) workspace = nullptr;
   if (m <= 64) {
     const char* e = tuning_env("KSQ_FP8_KSTAT");  // tuning / test switch: 0 sends small m to the streaming kernel
     if (!(e && atoi(e) == 0)) {
@@ -741,6 +742,7 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
   KSQ_REQUIRE(plan.mblocks <= 65535, KSQ_ERR_UNSUPPORTED, "m too large");
   dim3 grid((unsigned)((a.ntiles + 3) / 4), (unsigned)plan.ksplit, (unsigned)plan.mblocks);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  note_launch("fp8_stream_kernel<mt=%d> grid=(%u,%u,%u)", plan.MT, grid.x, grid.y, grid.z);
   if (out_dtype == KSQ_F16) launch_fp8_stream<_Float16>(plan.MT, a, grid, s);
   else launch_fp8_stream<__bf16>(plan.MT, a, grid, s);
   KSQ_HIP_TRY(hipGetLastError());

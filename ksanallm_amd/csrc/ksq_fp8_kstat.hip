@@ -538,6 +538,8 @@ int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const v
     KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
+  note_launch("fp8_kstat_kernel<mt=%d,tpw=%d,nb=%d%s> grid=(%d,%d) nt_per_wg=%d", plan.mt, plan.tpw, plan.nb,
+              act_src ? ",fused" : "", plan.grid_x, plan.ksplit, plan.nt_per_wg);
   if (act_src != nullptr) {
     const bool ok = out_dtype == KSQ_F16 ? launch_fused<_Float16>(plan.tpw, plan.nb, a, grid, s)
                                          : launch_fused<__bf16>(plan.tpw, plan.nb, a, grid, s);

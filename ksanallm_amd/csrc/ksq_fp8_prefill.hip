@@ -633,6 +633,9 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     // without a tail launch the one launch covers everything, rounded up to a multiple of eight; with one, the main
     // launch covers whole rounds (a multiple of eight by itself)
     const size_t main_tiles = (ks > 1 || quarters) ? total - (size_t)tail_tiles : tile_grid(a.mblocks, a.nblocks);
+    if (main_tiles) note_launch("fp8_prefill256_kernel grid=(%zu)", main_tiles);
+    if (quarters) note_launch("fp8_prefill256_kernel<quarters> tiles=%d", tail_tiles);
+    else if (ks > 1) note_launch("fp8_prefill256_kernel<ksplit=%d> tiles=%d + fp8_tail_reduce_kernel", ks, tail_tiles);
     if (main_tiles == 0) {
       // every tile is in the split launch
     } else if (out_dtype == KSQ_F16) {
@@ -668,6 +671,7 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     a.nblocks = (int)((n + kBN - 1) / kBN);
     KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
     const dim3 grid(tile_grid(a.mblocks, a.nblocks));
+    note_launch("fp8_prefill_kernel grid=(%u)", grid.x);
     if (out_dtype == KSQ_F16)
       hipLaunchKernelGGL(fp8_prefill_kernel<_Float16>, grid, dim3(256), 0, s, a);
     else

@@ -23,6 +23,12 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
     if (!(cond)) return ::ksq::fail((code), __VA_ARGS__); \
   } while (0)
 
+// ---- launch log ----------------------------------------------------------------------------------------------------
+// What the last GEMM entry point on this thread launched (kernel, template arguments, grid), for ksq_last_launch_string;
+// a no-op unless ksq_set_launch_log(1) was called, so the launch path of a serving process formats nothing.
+void note_launch(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void reset_launch_note();  // at the top of every GEMM entry point
+
 // ---- tuning / test overrides -------------------------------------------------------------------------------
 // The launch planners can be overridden through KSQ_* environment variables.  They are looked up only in a process
 // that had KSQ_TUNING=1 in its environment when the library was first used: otherwise this returns nullptr without
@@ -71,6 +77,8 @@ __host__ __device__ inline int frag_nibble_of(int e) { return (e & 1) ? 4 + (e >
 constexpr int kCounterSlots = 64;
 constexpr int kCountersPerSlot = 16384;
 unsigned* counter_slot_device_ptr(hipStream_t stream);  // the stream's region (device address) or nullptr
+bool counter_slot_available(hipStream_t stream);        // the same answer without claiming a region
+static_assert(kCountersPerSlot * 4 == KSQ_SPLITK_COUNTER_BYTES, "ksq.h states the size of a counter region");
 
 // ---- the few places where the kernels speak to the compiler or the machine in assembly ----------------------------------
 // A host build of the kernels (the CPU emulation that the tests use to walk every kernel's addressing, KSQ_EMU) has

@@ -517,41 +517,47 @@ constexpr int cnt_max_of(int mt, bool lds) {
   return GPT == 1 ? 3 : 2;
 }
 
+// false: no instantiation for (mt, cnt, lds) -- nothing was launched
 template <typename T, int GPT>
-void launch(int mt, int cnt, bool lds, const AstreamArgs& a, dim3 grid, hipStream_t s) {
+bool launch(int mt, int cnt, bool lds, const AstreamArgs& a, dim3 grid, hipStream_t s) {
   const dim3 block(512);
+  bool launched = false;
 #define KSQ_GO(MT, CNT)                                                                         \
   do {                                                                                          \
     if (lds) {                                                                                  \
-      if constexpr (CNT <= cnt_max_of<T, GPT>(MT, true))                                        \
+      if constexpr (CNT <= cnt_max_of<T, GPT>(MT, true)) {                                      \
         hipLaunchKernelGGL((w4a16_astream_lds_kernel<T, GPT, MT, CNT>), grid, block, 0, s, a);  \
+        launched = true;                                                                        \
+      }                                                                                         \
     } else {                                                                                    \
-      if constexpr (CNT <= cnt_max_of<T, GPT>(MT, false))                                       \
+      if constexpr (CNT <= cnt_max_of<T, GPT>(MT, false)) {                                     \
         hipLaunchKernelGGL((w4a16_astream_kernel<T, GPT, MT, CNT>), grid, block, 0, s, a);      \
+        launched = true;                                                                        \
+      }                                                                                         \
     }                                                                                           \
   } while (0)
-  // the caller keeps cnt within cnt_max_of
   if (mt <= 2) {
     if (cnt == 1) KSQ_GO(2, 1);
     else if (cnt == 2) KSQ_GO(2, 2);
     else if (cnt == 3) KSQ_GO(2, 3);
-    else KSQ_GO(2, 4);
+    else if (cnt == 4) KSQ_GO(2, 4);
   } else if (mt == 3) {
     if (cnt == 1) KSQ_GO(3, 1);
     else if (cnt == 2) KSQ_GO(3, 2);
     else if (cnt == 3) KSQ_GO(3, 3);
-    else KSQ_GO(3, 4);
+    else if (cnt == 4) KSQ_GO(3, 4);
   } else {
     if (cnt == 1) KSQ_GO(4, 1);
     else if (cnt == 2) KSQ_GO(4, 2);
     else if (cnt == 3) KSQ_GO(4, 3);
-    else KSQ_GO(4, 4);
+    else if (cnt == 4) KSQ_GO(4, 4);
   }
 #undef KSQ_GO
+  return launched;
 }
 
 template <typename T, int GPT>
-void plan_and_launch(int mt, int cus, const AstreamArgs& a, hipStream_t s) {
+bool plan_and_launch(int mt, int cus, const AstreamArgs& a, hipStream_t s) {
   // column tiles per workgroup: one workgroup per CU (per CU and split) if that needs no more than fit, else the
   // split into whole rounds of workgroups that wastes least
   const int wgs = cus / a.ksplit > 0 ? cus / a.ksplit : 1;
@@ -574,8 +580,11 @@ void plan_and_launch(int mt, int cus, const AstreamArgs& a, hipStream_t s) {
   int cnt = plan(cnt_max_of<T, GPT>(mt, true));
   bool lds = cnt >= 3;
   if (const char* e = tuning_env("KSQ_W4_ASTREAM_LDS")) lds = atoi(e) != 0;  // tuning / test override
-  if (!lds) cnt = plan(cnt_max_of<T, GPT>(mt, false));
-  launch<T, GPT>(mt, cnt, lds, a, dim3((unsigned)((a.ntiles + cnt - 1) / cnt), (unsigned)a.ksplit), s);
+  cnt = plan(cnt_max_of<T, GPT>(mt, lds));  // the limit of the form that runs, whichever way it was chosen
+  const dim3 grid((unsigned)((a.ntiles + cnt - 1) / cnt), (unsigned)a.ksplit);
+  note_launch("%s<mt=%d,cnt=%d,gpt=%d> grid=(%u,%u)", lds ? "w4a16_astream_lds_kernel" : "w4a16_astream_kernel", mt,
+              cnt, GPT, grid.x, grid.y);
+  return launch<T, GPT>(mt, cnt, lds, a, grid, s);
 }
 
 }  // namespace
@@ -634,13 +643,13 @@ int w4a16_launch_astream(int dtype, const AstreamPlan& plan, void* out, const vo
   }
   const int mt = plan.mt;
   const int gpt = (int)(kTileK / g);
+  bool launched;
   if (dtype == KSQ_F16) {
-    if (gpt == 1) plan_and_launch<_Float16, 1>(mt, cus, a, s);
-    else plan_and_launch<_Float16, 2>(mt, cus, a, s);
+    launched = gpt == 1 ? plan_and_launch<_Float16, 1>(mt, cus, a, s) : plan_and_launch<_Float16, 2>(mt, cus, a, s);
   } else {
-    if (gpt == 1) plan_and_launch<__bf16, 1>(mt, cus, a, s);
-    else plan_and_launch<__bf16, 2>(mt, cus, a, s);
+    launched = gpt == 1 ? plan_and_launch<__bf16, 1>(mt, cus, a, s) : plan_and_launch<__bf16, 2>(mt, cus, a, s);
   }
+  KSQ_REQUIRE(launched, KSQ_ERR_UNSUPPORTED, "no accumulator-stationary kernel for %d row tiles of this element type", mt);
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

@@ -502,6 +502,9 @@ int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* 
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
   const int gpt = (int)(kTileK / g);
+  note_launch("w4a16_kstat_kernel<mt=%d,tpw=%d,nb=%d,nw=%d,gpt=%d,ppi=%d> grid=(%d,%d) nt_per_wg=%d", plan.mt, plan.tpw,
+              plan.nb, plan.nw, gpt, plan.mt == 1 ? (m <= 4 ? 16 : (m <= 8 ? 8 : 4)) : 4, plan.grid_x, plan.ksplit,
+              plan.nt_per_wg);
   if (dtype == KSQ_F16) {
     if (gpt == 1) launch<_Float16, 1>(plan, a, grid, s);
     else launch<_Float16, 2>(plan, a, grid, s);

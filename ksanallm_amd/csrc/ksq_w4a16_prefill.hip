@@ -801,6 +801,12 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     block = dim3(64 * nw * plan.kg);
   }
   const int gpt = (int)(kTileK / g);
+  if (dtype != KSQ_F16) note_launch("bf16_rows_to_f16_kernel grid=(%zu)", m);
+  if (plan.rows == 64)
+    note_launch("w4a16_mid_kernel<gpt=%d,knt=%d> grid=(%u,%u)", gpt, plan.knt, grid.x, grid.y);
+  else
+    note_launch("w4a16_prefill_kernel<gpt=%d,nw=%d,kg=%d> grid=(%u)", gpt, plan.nw, plan.kg, grid.x);
+  if (plan.ksplit > 1) note_launch("w4a16_splitk_reduce_kernel");
   if (dtype == KSQ_F16) {
     launch_typed<_Float16>(a, gpt, nw, plan.kg, grid, block, s);
   } else {

@@ -401,6 +401,8 @@ int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* ac
   KSQ_REQUIRE(plan.mblocks <= 65535 && plan.ksplit <= 65535, KSQ_ERR_UNSUPPORTED, "grid too large");
   dim3 grid((unsigned)((a.ngroups + 3) / 4), (unsigned)plan.ksplit, (unsigned)plan.mblocks);
   const int gpt = (int)(kTileK / g);
+  note_launch("w4a16_stream_kernel<mt=%d,nt=%d,gpt=%d,slices=%d> grid=(%u,%u,%u)", plan.MT, plan.NT, gpt, plan.slices,
+              grid.x, grid.y, grid.z);
   if (dtype == KSQ_F16) launch_mt<_Float16>(plan.MT, plan.NT, gpt, plan.slices, a, grid, s);
   else launch_mt<__bf16>(plan.MT, plan.NT, gpt, plan.slices, a, grid, s);
   KSQ_HIP_TRY(hipGetLastError());

@@ -7,6 +7,16 @@
 
 namespace ksana_llm {
 
+// layouts a 4-bit group-quantized weight can arrive in (see RepackGroupQuantWeight below)
+enum GroupWeightLayout {
+  GROUP_WEIGHT_GPTQ_INT32,
+  GROUP_WEIGHT_AWQ_INT32,
+  GROUP_WEIGHT_ROWMAJOR_INT4,
+  GROUP_WEIGHT_CUTLASS_SM80,
+  GROUP_WEIGHT_CUTLASS_SM90,
+  GROUP_WEIGHT_MARLIN  // Marlin tiles; scales in Marlin order; qzeros (AWQ) as Marlin zero points
+};
+
 template <typename T, DataType WT>
 class GroupMatMulLayer : public BaseLayer {
  public:
@@ -32,7 +42,17 @@ class GroupMatMulLayer : public BaseLayer {
   // interleaved gate/up weight (KSQ_EPILOGUE_SILU_MUL) into the GEMM.  The bias tensor must outlive the layer.
   void SetEpilogue(int kind, const Tensor* bias = nullptr);
 
+  // Which of the reference loader's CUTLASS layouts a weight is in when it reaches Forward without having been
+  // repacked (its `.scales` still T [k/g, n], `.zeros` additive T or null): the loader's preprocess is architecture
+  // dependent (LK/asymmetric_gemm/cutlass_preprocessors.cpp:504), so a loader carried over unchanged states which
+  // one it ran.  GROUP_WEIGHT_CUTLASS_SM80 by default; a Marlin back end (Init) overrides this.  Such a weight is
+  // converted once, at its first Forward: its bytes are rewritten in place into the fragment order and the combined
+  // scale/zero words are kept by the library (ForgetAdoptedGroupQuantWeights frees them).
+  void SetLoaderLayout(int group_weight_layout) { loader_layout_ = static_cast<GroupWeightLayout>(group_weight_layout); }
+
  private:
+  void AdoptLoaderWeight(const Tensor& weight_tensor, void** weight, void** sz);
+  GroupWeightLayout loader_layout_ = GROUP_WEIGHT_CUTLASS_SM80;
   bool is_awq_ = false;
   bool is_gptq_desc_ = false;
   bool is_k_full_ = true;
@@ -53,14 +73,6 @@ class GroupMatMulLayer : public BaseLayer {
 // loader can be followed by this call.  `perm` (int32 [k] on the device, from SortGptqGIdx) repacks a desc_act
 // checkpoint with its rows grouped and is bound to weight.perm; `interleave_gate_up` repacks a fused [gate | up]
 // weight with its column pairs interleaved for the SiLU-mul epilogue.
-enum GroupWeightLayout {
-  GROUP_WEIGHT_GPTQ_INT32,
-  GROUP_WEIGHT_AWQ_INT32,
-  GROUP_WEIGHT_ROWMAJOR_INT4,
-  GROUP_WEIGHT_CUTLASS_SM80,
-  GROUP_WEIGHT_CUTLASS_SM90,
-  GROUP_WEIGHT_MARLIN  // Marlin tiles; scales in Marlin order; qzeros (AWQ) as Marlin zero points
-};
 Status RepackGroupQuantWeight(GroupWeightLayout layout, const Tensor& qweight, const Tensor* qzeros, bool zeros_additive,
                               const Tensor& scales, size_t k, size_t n, size_t groupsize, Tensor& weight,
                               Tensor& weight_sz, int rank, Stream& stream, Tensor* perm = nullptr,
@@ -84,5 +96,9 @@ Status RepackFusedGroupQuantWeight(GroupWeightLayout layout, const std::vector<G
 // perm = stable argsort of a desc_act checkpoint's g_idx (MarlinSortGIdx, quant_weight.cpp:455-460), on the host.
 // Throws unless every group has exactly `groupsize` rows.
 Status SortGptqGIdx(const std::vector<int32_t>& g_idx, size_t groupsize, std::vector<int32_t>& perm);
+
+// Frees the scale/zero words (and padded weights) of every loader-format weight that a GroupMatMulLayer converted at
+// its first Forward; call it when the model's weights are released.
+void ForgetAdoptedGroupQuantWeights(int rank);
 
 }  // namespace ksana_llm

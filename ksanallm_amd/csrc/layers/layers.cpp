@@ -3,7 +3,9 @@
 // KS/layers/nvidia/{group_matmul,fp8_matmul}_layer.cpp and the kernel library do.
 #include <hip/hip_runtime_api.h>
 
+#include <mutex>
 #include <sstream>
+#include <unordered_map>
 
 #include "fp8_matmul_layer.h"
 #include "group_matmul_layer.h"
@@ -55,6 +57,64 @@ Status DestroyTensor(Tensor& tensor, int rank) {
 }
 
 // ---------------------------------------------------------------------------------------------- GroupMatMulLayer
+namespace {
+
+// Weights that reached Forward as the reference's own loader leaves them (QuantWeight::ConvertGroupTensor,
+// KS/models/quant/quant_weight.cpp:463-660: "*.weight" preprocessed for its CUTLASS or Marlin back end, `.scales` in
+// T, `.zeros` additive in T) and were converted on their first use: the bytes of the loader's tensor now hold the
+// fragment order (same size), the scale/zero words live here.  Keyed by the loader's device pointer and shared by
+// all layers of the process, since one layer object serves the same projection of every decoder layer.
+struct AdoptedWeight {
+  void* weight = nullptr;  // what the GEMM reads: the loader's own tensor, or `padded` when K had to be padded
+  Tensor sz;
+  Tensor padded;
+};
+std::mutex g_adopted_mutex;
+std::unordered_map<const void*, AdoptedWeight> g_adopted;
+
+}  // namespace
+
+void ForgetAdoptedGroupQuantWeights(int rank) {
+  std::lock_guard<std::mutex> lock(g_adopted_mutex);
+  for (auto& kv : g_adopted) {
+    DestroyTensor(kv.second.sz, rank);
+    DestroyTensor(kv.second.padded, rank);
+  }
+  g_adopted.clear();
+}
+
+template <typename T, DataType WT>
+void GroupMatMulLayer<T, WT>::AdoptLoaderWeight(const Tensor& weight_tensor, void** weight, void** sz) {
+  std::lock_guard<std::mutex> lock(g_adopted_mutex);
+  auto it = g_adopted.find(weight_tensor.refer_ptr);
+  if (it == g_adopted.end()) {
+    // First use: not safe under graph capture (it allocates and synchronises); the warm-up step that every serving
+    // engine runs before it captures takes care of that.
+    const GroupWeightLayout layout = backend_ == MARLIN_BACKEND ? GROUP_WEIGHT_MARLIN : loader_layout_;
+    Stream& stream = context_->GetComputeStreams()[rank_];
+    Tensor fresh, fresh_sz;
+    RepackGroupQuantWeight(layout, weight_tensor, weight_tensor.zeros, /*zeros_additive=*/true, *weight_tensor.scales,
+                           max_k_, max_n_, groupsize_, fresh, fresh_sz, rank_, stream);
+    AdoptedWeight ad;
+    ad.sz = fresh_sz;
+    const size_t loader_bytes = max_k_ * max_n_ / 2;
+    if (fresh.GetTotalBytes() == loader_bytes) {
+      hipError_t e = hipMemcpyAsync(weight_tensor.refer_ptr, fresh.refer_ptr, loader_bytes, hipMemcpyDeviceToDevice,
+                                    static_cast<hipStream_t>(stream.Get()));
+      if (e == hipSuccess) e = hipStreamSynchronize(static_cast<hipStream_t>(stream.Get()));
+      if (e != hipSuccess) KLLM_THROW(std::string("GroupMatMulLayer: adopting a loader-format weight: ") + hipGetErrorString(e));
+      DestroyTensor(fresh, rank_);
+      ad.weight = weight_tensor.refer_ptr;
+    } else {  // K = 64 x odd: the fragment order pads the last k tile and no longer fits the loader's tensor
+      ad.padded = fresh;
+      ad.weight = fresh.refer_ptr;
+    }
+    it = g_adopted.emplace(weight_tensor.refer_ptr, ad).first;
+  }
+  *weight = it->second.weight;
+  *sz = it->second.sz.refer_ptr;
+}
+
 template <typename T, DataType WT>
 Status GroupMatMulLayer<T, WT>::Init(const std::vector<std::any>& parameters, std::shared_ptr<Context> context,
                                      int rank) {
@@ -117,6 +177,11 @@ Status GroupMatMulLayer<T, WT>::Forward(const std::vector<Tensor>& input_tensors
     }
     void* p_qweight_tensor = weight_tensor.GetPtr<void>();
     void* p_sz_tensor = weight_tensor.scales->GetPtr<void>();
+    if (weight_tensor.scales->dtype == TYPE_FP16 || weight_tensor.scales->dtype == TYPE_BF16) {
+      // not repacked by RepackGroupQuantWeight: the reference loader's own output, converted on first use
+      if (is_gptq_desc_) KLLM_THROW("GroupMatMulLayer: a desc_act weight must be repacked with its perm at load time.");
+      AdoptLoaderWeight(weight_tensor, &p_qweight_tensor, &p_sz_tensor);
+    }
 
     const size_t m = input_tensors[0].shape[0];
     const size_t n = max_n_;

@@ -61,7 +61,8 @@ static int RunW4(int argc, char** argv) {
   const std::string dir = argv[2];
   const size_t m = atol(argv[4]), k = atol(argv[5]), n = atol(argv[6]), g = atol(argv[7]);
   const std::string method = argv[8], layout = argv[9], zeros = argv[10];
-  const std::string extra = argc > 11 ? argv[11] : "none";  // none | desc | silu | bias | parts:n0:n1:..
+  // none | desc | silu | bias | parts:n0:n1:.. | adopt (no load-time repack: the loader's own tensors reach Forward)
+  const std::string extra = argc > 11 ? argv[11] : "none";
   const DataType dt = TypeTraits<T>::kDataType;
   auto context = std::make_shared<Context>(1);
 
@@ -125,6 +126,13 @@ static int RunW4(int argc, char** argv) {
     }
     RepackFusedGroupQuantWeight(GROUP_WEIGHT_AWQ_INT32, parts, false, k, g, weight, weight_sz, 0,
                                 context->GetComputeStreams()[0]);
+  } else if (extra == "adopt") {
+    // what KsanaLLM's own loader hands the layer: "*.weight" as its back end preprocessed it, with `.scales` and the
+    // additive `.zeros` bound (KS/models/quant/quant_weight.cpp:632-636); the layer converts it at its first Forward
+    weight = qweight;
+    weight.dtype = TYPE_I4_GROUP;
+    weight.scales = &scales;
+    weight.zeros = const_cast<Tensor*>(zp);
   } else {
     RepackGroupQuantWeight(lay, qweight, zp, additive, scales, k, n, g, weight, weight_sz, 0,
                            context->GetComputeStreams()[0], extra == "desc" ? &perm : nullptr, extra == "silu");
@@ -145,6 +153,11 @@ static int RunW4(int argc, char** argv) {
   holder->t = weight;
   auto layer = factory.ForWeight(*holder, "model.layers.0.self_attn.query_key_value.weight", dt);
 
+  if (extra == "adopt") {
+    auto group = std::dynamic_pointer_cast<GroupMatMulLayer<T, TYPE_I4_GROUP>>(layer);
+    if (!group) throw std::runtime_error("harness did not build a GroupMatMulLayer");
+    group->SetLoaderLayout(lay);
+  }
   Tensor bias;
   if (extra == "silu" || extra == "bias") {
     auto group = std::dynamic_pointer_cast<GroupMatMulLayer<T, TYPE_I4_GROUP>>(layer);
@@ -164,6 +177,11 @@ static int RunW4(int argc, char** argv) {
   std::vector<Tensor> outputs = {out};
   Status st = layer->Forward({act, weight}, outputs);
   if (!st.OK()) throw std::runtime_error("Forward returned " + st.GetMessage());
+  if (extra == "adopt") {  // the second call finds the converted weight: same tensor, nothing to do
+    st = layer->Forward({act, weight}, outputs);
+    if (!st.OK()) throw std::runtime_error("second Forward returned " + st.GetMessage());
+    ForgetAdoptedGroupQuantWeights(0);
+  }
   Download(outputs[0], dir + "/out.bin");
   std::cout << "OK " << outputs[0].shape[0] << " " << outputs[0].shape[1] << " " << outputs[0].dtype << std::endl;
   return 0;

@@ -59,6 +59,12 @@ def test_group_matmul_layer_k_not_a_multiple_of_128(on_cpu, tmp_path, dtype, M, 
     cases._odd_k_case(_run, tmp_path, dtype, M, parts)
 
 
+@pytest.mark.parametrize("dtype,layout,kind,M", [("f16", "cutlass80", "awq", 16), ("bf16", "cutlass80", "gptq", 70),
+                                                 ("f16", "cutlass90", "awq", 5)])
+def test_group_matmul_layer_takes_the_reference_loaders_tensors_at_forward(on_cpu, tmp_path, dtype, layout, kind, M):
+    cases._adopt_case(_run, tmp_path, dtype, layout, kind, M)
+
+
 @pytest.mark.parametrize("dtype,wscales,static,M", [("f16", "1", 0, 16), ("bf16", "n", 0, 70), ("f16", "1", 1, 5)])
 def test_fp8_matmul_layer_forward(on_cpu, tmp_path, dtype, wscales, static, M):
     cases.test_fp8_matmul_layer_forward(None, tmp_path, dtype, wscales, static, M)

@@ -59,6 +59,7 @@ test_prefill_bf16_row_magnitudes = w4.test_prefill_bf16_row_magnitudes
 test_bf16_scales_far_outside_the_fp16_range = w4.test_bf16_scales_far_outside_the_fp16_range
 test_k_odd_multiple_of_64 = w4.test_k_odd_multiple_of_64
 test_no_workspace_still_correct = w4.test_no_workspace_still_correct
+test_caller_bound_split_k_counters_and_launch_log = w4.test_caller_bound_split_k_counters_and_launch_log
 test_k_tiles_per_wave = w4.test_k_tiles_per_wave
 
 # ---- FP8 -------------------------------------------------------------------------------------------------------------------

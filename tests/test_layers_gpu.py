@@ -102,6 +102,31 @@ def test_group_matmul_layer_widened(gpu, tmp_path, dtype, extra, layout, M):
     orc.assert_parity(got, want, f"GroupMatMulLayer {layout} {extra} {dtype}")
 
 
+@pytest.mark.parametrize("dtype,layout,kind,M", [("f16", "cutlass80", "awq", 16), ("bf16", "cutlass80", "gptq", 70),
+                                                 ("f16", "cutlass90", "awq", 5)])
+def test_group_matmul_layer_takes_the_reference_loaders_tensors_at_forward(gpu, tmp_path, dtype, layout, kind, M):
+    """No load-time repack at all: the weight reaches Forward as KsanaLLM's loader leaves it (CUTLASS-preprocessed
+    bytes, `.scales` in T, `.zeros` additive in T or absent) and is converted on first use; two calls, same result."""
+    _adopt_case(_run, tmp_path, dtype, layout, kind, M)
+
+
+def _adopt_case(run, tmp_path, dtype, layout, kind, M):
+    K, N, g = 1024, 384, 128
+    case = W4Case(660 + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    d = str(tmp_path)
+    orc.cutlass_preprocess(case.rowmajor(), int(layout[-2:])).tofile(d + "/qweight.bin")
+    zeros = "none"
+    if kind == "awq":
+        orc.awq_additive_zeros(case.scales, ORC_DT[dtype], case.z).tofile(d + "/qzeros.bin")
+        zeros = "additive"
+    case.scales.tofile(d + "/scales.bin")
+    case.act.tofile(d + "/act.bin")
+    rc, out = run(["w4a16", d, dtype, M, K, N, g, kind, layout, zeros, "adopt"])
+    assert rc == 0 and out.splitlines()[-1] == f"OK {M} {N} {DTYPE_ENUM[dtype]}", out
+    got = orc.from_bits(np.fromfile(d + "/out.bin", dtype=np.uint16).reshape(M, N), ORC_DT[dtype])
+    orc.assert_parity(got, case.oracle(), f"GroupMatMulLayer loader tensors at Forward {layout} {kind} {dtype}")
+
+
 @pytest.mark.parametrize("dtype,M,parts", [("f16", 16, None), ("bf16", 70, None), ("f16", 5, [64, 32, 32]),
                                            ("bf16", 130, [64, 64])])
 def test_group_matmul_layer_k_not_a_multiple_of_128(gpu, tmp_path, dtype, M, parts):

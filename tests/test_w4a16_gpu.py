@@ -370,6 +370,39 @@ def test_k_odd_multiple_of_64(gpu, dtype, kind, M, K, N):
     assert e.value.code == capi.ERR_WORKSPACE
 
 
+def test_caller_bound_split_k_counters_and_launch_log(gpu):
+    """Split-K with the arrival counters in the caller's memory: same bits as with the library's, the memory is back at
+    zero after every launch, and the launch log names the kernel and its split."""
+    import torch
+
+    from ksanallm_amd import capi
+
+    case = W4Case(1777, 16, 1408, 272, kind="awq", dtype="f16")
+    dev = W4Device(case, gpu)
+    big = torch.empty(8 << 20, dtype=torch.uint8, device=gpu)
+    dev.workspace, dev.workspace_bytes = big, big.numel()
+    capi.set_launch_log(True)
+    try:
+        with _env(KSQ_W4_KSPLIT=3):
+            ref = dev.gemm_f32()
+            assert "w4a16_kstat_kernel" in capi.last_launch() and ",3)" in capi.last_launch(), capi.last_launch()
+            mine = torch.zeros(capi.SPLITK_COUNTER_BYTES + 256, dtype=torch.uint8, device=gpu)
+            mine = mine[(-mine.data_ptr()) % 256:][:capi.SPLITK_COUNTER_BYTES]
+            capi.bind_splitk_counters(None, mine)
+            try:
+                got1, got2 = dev.gemm_f32(), dev.gemm_f32()
+            finally:
+                capi.bind_splitk_counters(None, None)
+            again = dev.gemm_f32()
+    finally:
+        capi.set_launch_log(False)
+    assert int(mine.to(torch.int32).abs().sum().item()) == 0, "the counters did not return to zero"
+    assert np.array_equal(ref, got1) and np.array_equal(ref, got2) and np.array_equal(ref, again)
+    orc.assert_parity(ref, case.oracle(), "bound counters")
+    with pytest.raises(capi.KsqError):
+        capi.bind_splitk_counters(None, mine, 1024)  # too small
+
+
 def test_no_workspace_still_correct(gpu):
     case = W4Case(1300, 16, 4096, 512, kind="gptq", dtype="f16")
     dev = W4Device(case, gpu)
