@@ -326,6 +326,52 @@ def fp8_sweep(torch, capi, dev, stream):
     return table
 
 
+def fp8_rowmax_chain(torch, capi, dev, stream):
+    """The per-token quantisation's max pass moved into the GEMM that produces the tensor: the Qwen-72B o projection
+    (K = N = 8192, FP8) with and without the row maxima in its epilogue, and the quantiser of its output (bf16
+    [M, 8192]) with its own max pass and without (one read)."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(9)
+    k = n = 8192
+    ws, wscale = fp8_weights(torch, capi, dev, gen, k, n)
+    table = {}
+    for M in (8, 64, 2048):
+        act = torch.randn((M, k), device=dev, generator=gen).to(torch.bfloat16)
+        aq = torch.empty((M, k), dtype=torch.uint8, device=dev)
+        ascale = torch.empty(M, dtype=torch.float32, device=dev)
+        capi.fp8_quantize(capi.BF16, act, M, k, capi.FP8_PER_TOKEN_DYNAMIC, aq, ascale, stream.cuda_stream)
+        out = torch.empty((M, n), dtype=torch.bfloat16, device=dev)
+        rowmax = torch.zeros(M, dtype=torch.float32, device=dev)
+        oq = torch.empty((M, n), dtype=torch.uint8, device=dev)
+        oscale = torch.empty(M, dtype=torch.float32, device=dev)
+        wsb = capi.fp8_workspace_bytes(M, n, k)
+        wk = torch.empty(max(wsb, 256), dtype=torch.uint8, device=dev)
+        sp = stream.cuda_stream
+        reps = max(16 if M <= 64 else 4, len(ws))
+
+        def gemm(i):
+            capi.fp8_gemm(capi.BF16, out, aq, ascale, M, ws[i % len(ws)], wscale, n, M, n, k, wk, wsb, sp)
+
+        def gemm_rowmax(i):
+            capi.fill_zero_f32(rowmax, M, sp)
+            capi.fp8_gemm_rowmax(capi.BF16, out, aq, ascale, M, ws[i % len(ws)], wscale, n, M, n, k, rowmax,
+                                 capi.EPILOGUE_NONE, None, wk, wsb, sp)
+
+        def quant2(i):
+            capi.fp8_quantize(capi.BF16, out, M, n, capi.FP8_PER_TOKEN_DYNAMIC, oq, oscale, sp)
+
+        def quant1(i):
+            capi.fp8_quantize_rows_from_absmax(capi.BF16, out, M, n, rowmax, oq, oscale, sp)
+
+        table[f"m{M}"] = {"gemm_us": round(time_graph(torch, stream, gemm, reps), 1),
+                          "zero_fill_and_gemm_with_row_maxima_us": round(time_graph(torch, stream, gemm_rowmax, reps), 1),
+                          "quantize_two_pass_us": round(time_graph(torch, stream, quant2, 16), 1),
+                          "quantize_from_row_maxima_us": round(time_graph(torch, stream, quant1, 16), 1)}
+    del ws
+    torch.cuda.empty_cache()
+    return table
+
+
 def gptq_70b_sweep(torch, capi, dev, stream):
     """configs[3]: symmetric GPTQ int4 g=128, fp16, the Llama-3-70B shapes at M = 1, 32 (HBM-bound: GB/s against the
     HBM peak) and 256 (TFLOP/s against the dense MFMA peak), and 128 as a batch between the two."""
@@ -643,6 +689,7 @@ def main():
         del layers[1:]
         torch.cuda.empty_cache()
         extra["fp8_cfg4"] = fp8_sweep(torch, capi, dev, stream)
+        extra["fp8_row_maxima_from_producer"] = fp8_rowmax_chain(torch, capi, dev, stream)
         extra["gptq_70b_cfg3"] = gptq_70b_sweep(torch, capi, dev, stream)
     if not args.no_cpu:
         del layers[1:]

@@ -309,6 +309,30 @@ int ksq_fp8_gemm_dynamic(int dtype, void* out, const void* act, const void* w_q,
  * per-channel scales (row_bytes = 4). */
 int ksq_interleave_halves(void* out, const void* in, size_t rows, size_t row_bytes, void* stream);
 
+/* ------------------------------------------------------------------ row maxima from the producing GEMM
+ *
+ * The producer's half of folding the per-token FP8 quantisation into its neighbour (no counterpart in the reference,
+ * whose quantiser makes a max pass of its own over the tensor: LU/cuda_fp8_utils.cu:85-127, merging blocks by atomic
+ * maximum on the float bits, :111-115 -- the same merge is used here, from the GEMM's epilogue).
+ *
+ * ksq_w4a16_gemm_rowmax / ksq_fp8_gemm_rowmax are ksq_w4a16_gemm_ex (without act_perm) / ksq_fp8_gemm_ex; in
+ * addition the largest |out[row, :]| of every row -- of the values as stored, after the epilogue -- is merged into
+ * row_absmax[row] (fp32 [m]) by atomic maximum.  row_absmax must hold zeros on entry (ksq_fill_zero_f32, which is
+ * safe to record into a HIP graph), or the maxima of columns that another call contributed.
+ * ksq_fp8_quantize_rows_from_absmax is then ksq_fp8_quantize(KSQ_FP8_PER_TOKEN_DYNAMIC) without its max pass:
+ * act_scale[r] = max(row_absmax[r] / 448, 1 / (448 * 512)), one read of act; bit-identical bytes and scales when
+ * row_absmax holds the rows' maxima. */
+int ksq_fill_zero_f32(float* p, size_t count, void* stream);
+int ksq_w4a16_gemm_rowmax(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                          size_t k, size_t group_size, int epilogue, const void* bias, float* row_absmax,
+                          void* workspace, size_t workspace_bytes, void* stream);
+int ksq_fp8_gemm_rowmax(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                        const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                        int epilogue, const void* bias, float* row_absmax, void* workspace, size_t workspace_bytes,
+                        void* stream);
+int ksq_fp8_quantize_rows_from_absmax(int dtype, const void* act, size_t m, size_t k, const float* row_absmax,
+                                      void* act_q, float* act_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,7 @@ EXPORTS = [
     "ksq_w4a16_workspace_bytes_ex", "ksq_w4a16_gemm_ex", "ksq_fp8_gemm_ex", "ksq_interleave_halves",
     "ksq_w4a16_gemm_static_scratch", "ksq_fp8_gemm_dynamic_workspace_bytes", "ksq_fp8_gemm_dynamic",
     "ksq_set_launch_log", "ksq_last_launch_string", "ksq_bind_splitk_counters",
+    "ksq_fill_zero_f32", "ksq_w4a16_gemm_rowmax", "ksq_fp8_gemm_rowmax", "ksq_fp8_quantize_rows_from_absmax",
 ]
 SPLITK_COUNTER_BYTES = 65536
 STATIC_SCRATCH_BYTES = 64 << 20
@@ -79,6 +80,10 @@ def _bind(L):
     L.ksq_set_launch_log.restype = None
     L.ksq_last_launch_string.restype = ctypes.c_char_p
     L.ksq_bind_splitk_counters.argtypes = [vp, vp, sz]
+    L.ksq_fill_zero_f32.argtypes = [vp, sz, vp]
+    L.ksq_w4a16_gemm_rowmax.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, ci, vp, vp, vp, sz, vp]
+    L.ksq_fp8_gemm_rowmax.argtypes = [ci, vp, vp, vp, sz, vp, vp, sz, sz, sz, sz, ci, vp, vp, vp, sz, vp]
+    L.ksq_fp8_quantize_rows_from_absmax.argtypes = [ci, vp, sz, sz, vp, vp, vp, vp]
     for name in EXPORTS:
         if name not in ("ksq_last_error_string", "ksq_set_launch_log", "ksq_last_launch_string"):
             getattr(L, name).restype = ci
@@ -218,6 +223,28 @@ def fp8_gemm_dynamic(dtype, out, act, w_q, w_scale, w_scale_count, m, n, k, epil
                      workspace=None, workspace_bytes=0, stream=None):
     _check(lib().ksq_fp8_gemm_dynamic(dtype, _addr(out), _addr(act), _addr(w_q), _addr(w_scale), w_scale_count, m, n, k,
                                       epilogue, _addr(bias), _addr(workspace), workspace_bytes, stream))
+
+
+def fill_zero_f32(p, count, stream=None):
+    _check(lib().ksq_fill_zero_f32(_addr(p), count, stream))
+
+
+def w4a16_gemm_rowmax(dtype, out, act, weight, sz, m, n, k, group_size, row_absmax, epilogue=EPILOGUE_NONE, bias=None,
+                      workspace=None, workspace_bytes=0, stream=None):
+    _check(lib().ksq_w4a16_gemm_rowmax(dtype, _addr(out), _addr(act), _addr(weight), _addr(sz), m, n, k, group_size,
+                                       epilogue, _addr(bias), _addr(row_absmax), _addr(workspace), workspace_bytes, stream))
+
+
+def fp8_gemm_rowmax(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k, row_absmax,
+                    epilogue=EPILOGUE_NONE, bias=None, workspace=None, workspace_bytes=0, stream=None):
+    _check(lib().ksq_fp8_gemm_rowmax(out_dtype, _addr(out), _addr(act_q), _addr(act_scale), act_scale_count, _addr(w_q),
+                                     _addr(w_scale), w_scale_count, m, n, k, epilogue, _addr(bias), _addr(row_absmax),
+                                     _addr(workspace), workspace_bytes, stream))
+
+
+def fp8_quantize_rows_from_absmax(dtype, act, m, k, row_absmax, act_q, act_scale, stream=None):
+    _check(lib().ksq_fp8_quantize_rows_from_absmax(dtype, _addr(act), m, k, _addr(row_absmax), _addr(act_q),
+                                                   _addr(act_scale), stream))
 
 
 def fp8_quantize(dtype, act, m, k, mode, act_q, act_scale, stream=None):

@@ -345,9 +345,9 @@ int ksq_w4a16_workspace_bytes_ex(size_t max_m, size_t n, size_t k, int act_order
   return KSQ_OK;
 }
 
-int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
-                      size_t k, size_t g, const int32_t* act_perm, int epilogue, const void* bias, void* workspace,
-                      size_t workspace_bytes, void* stream) {
+static int w4a16_gemm_impl(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                           size_t k, size_t g, const int32_t* act_perm, int epilogue, const void* bias,
+                           float* row_absmax, void* workspace, size_t workspace_bytes, void* stream) {
   reset_launch_note();
   KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
   KSQ_REQUIRE(out && act && weight && sz, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
@@ -398,6 +398,7 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   Epilogue epi;
   epi.kind = epilogue;
   epi.bias = bias;
+  epi.row_absmax = row_absmax;
   if (env_int("KSQ_W4_FORCE_STREAM", 0) == 0 && w4a16_prefill_supported(dtype, m, n, k, g, di->cus) &&
       workspace_bytes >= w4a16_prefill_workspace_bytes(dtype, m, k))
     return w4a16_launch_prefill(dtype, out, act, weight, sz, m, n, k, g, workspace, workspace_bytes, s, epi);
@@ -422,6 +423,22 @@ int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight,
   }
   W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace_bytes);
   return w4a16_launch_stream(dtype, plan, out, act, weight, sz, m, n, k, g, workspace, s, epi);
+}
+
+int ksq_w4a16_gemm_ex(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                      size_t k, size_t g, const int32_t* act_perm, int epilogue, const void* bias, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  return w4a16_gemm_impl(dtype, out, act, weight, sz, m, n, k, g, act_perm, epilogue, bias, nullptr, workspace,
+                         workspace_bytes, stream);
+}
+
+int ksq_w4a16_gemm_rowmax(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,
+                          size_t k, size_t g, int epilogue, const void* bias, float* row_absmax, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  KSQ_REQUIRE(row_absmax != nullptr && (reinterpret_cast<uintptr_t>(row_absmax) & 3) == 0, KSQ_ERR_INVALID_ARGUMENT,
+              "row_absmax is null or misaligned");
+  return w4a16_gemm_impl(dtype, out, act, weight, sz, m, n, k, g, nullptr, epilogue, bias, row_absmax, workspace,
+                         workspace_bytes, stream);
 }
 
 int ksq_w4a16_gemm(int dtype, void* out, const void* act, const void* weight, const void* sz, size_t m, size_t n,

@@ -28,43 +28,66 @@ __device__ inline float epi_silu(float x) { return x / (1.0f + __expf(-x)); }
 template <typename T>
 __device__ inline void epi_store_acc(const Epilogue& ep, uint16_t* out, epi_f32x4 v, int row0, int col, int M, int N,
                                      bool ok) {
+  uint16_t bits[4];
+  bool mine = ok;
+  size_t width = (size_t)N;
+  int ocol = col;
   if (ep.kind == KSQ_EPILOGUE_SILU_MUL) {
     // value of the neighbouring lane (lane ^ 1): DPP quad permutation [1, 0, 3, 2].  The elements are copied into
     // scalars first: a bit cast applied to a vector element directly reads element 0 whatever the index.
-    epi_f32x4 up;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float mine = v[e];
-      up[e] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, mine), 0xB1, 0xF, 0xF, true));
+      const float gate = v[e];
+      const float up = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, gate), 0xB1, 0xF, 0xF, true));
+      bits[e] = epi_bits<T>(epi_silu(gate) * up);
     }
-    if (ok && !(col & 1)) {
-      const size_t half = (size_t)(N >> 1);
+    mine = ok && !(col & 1);
+    width = (size_t)(N >> 1);
+    ocol = col >> 1;
+  } else {
+    float b = 0.f;
+    if (ep.kind == KSQ_EPILOGUE_BIAS && ok) b = epi_float<T>(static_cast<const uint16_t*>(ep.bias)[col]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (row0 + e < M) out[(size_t)(row0 + e) * half + (col >> 1)] = epi_bits<T>(epi_silu(v[e]) * up[e]);
-    }
-    return;
+    for (int e = 0; e < 4; ++e) bits[e] = epi_bits<T>(v[e] + b);
   }
-  if (!ok) return;
-  float b = 0.f;
-  if (ep.kind == KSQ_EPILOGUE_BIAS) b = epi_float<T>(static_cast<const uint16_t*>(ep.bias)[col]);
+  if (mine) {
 #pragma unroll
-  for (int e = 0; e < 4; ++e)
-    if (row0 + e < M) out[(size_t)(row0 + e) * N + col] = epi_bits<T>(v[e] + b);
+    for (int e = 0; e < 4; ++e)
+      if (row0 + e < M) out[(size_t)(row0 + e) * width + ocol] = bits[e];
+  }
+  if (ep.row_absmax) {
+    // The largest |stored value| of every row, for whoever quantises this output per token next: the 16 lanes that
+    // hold a row's 16 columns of this tile agree on their maximum, one of them folds it into row_absmax[row] with an
+    // atomic maximum on the bit pattern (non-negative floats order like unsigned integers), as the reference's
+    // quantiser merges its blocks (LU/cuda_fp8_utils.cu:111-115).  Uniform over the wave: every lane gets here.
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float a = (mine && row0 + e < M) ? __builtin_fabsf(epi_float<T>(bits[e])) : 0.f;
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) a = __builtin_fmaxf(a, __shfl_xor(a, off));
+      if ((col & 15) == 0 && row0 + e < M)
+        atomicMax(reinterpret_cast<unsigned*>(ep.row_absmax) + (row0 + e), __builtin_bit_cast(unsigned, a));
+    }
+  }
 }
 
-// Row segment: src[0..7] = results at (row, col .. col + 7), col a multiple of 8 and col + 8 <= N, row < M.
+// Row segment: src[0..7] = results at (row, col .. col + 7), col a multiple of 8 and col + 8 <= N, row < M.  Returns the
+// largest |stored value| of the segment.
 template <typename T>
-__device__ inline void epi_store_row8(const Epilogue& ep, uint16_t* out, const float (&src)[8], int row, int col,
-                                      int N) {
+__device__ inline float epi_store_row8(const Epilogue& ep, uint16_t* out, const float (&src)[8], int row, int col,
+                                       int N) {
+  float mx = 0.f;
   if (ep.kind == KSQ_EPILOGUE_SILU_MUL) {
     epi_u32x2 packed;
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
-      packed[q] = (uint32_t)epi_bits<T>(epi_silu(src[4 * q]) * src[4 * q + 1]) |
-                  ((uint32_t)epi_bits<T>(epi_silu(src[4 * q + 2]) * src[4 * q + 3]) << 16);
+    for (int q = 0; q < 2; ++q) {
+      const uint16_t lo = epi_bits<T>(epi_silu(src[4 * q]) * src[4 * q + 1]);
+      const uint16_t hi = epi_bits<T>(epi_silu(src[4 * q + 2]) * src[4 * q + 3]);
+      packed[q] = (uint32_t)lo | ((uint32_t)hi << 16);
+      mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(epi_float<T>(lo)), __builtin_fabsf(epi_float<T>(hi))));
+    }
     *reinterpret_cast<epi_u32x2*>(out + (size_t)row * (size_t)(N >> 1) + (col >> 1)) = packed;
-    return;
+    return mx;
   }
   float b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (ep.kind == KSQ_EPILOGUE_BIAS) {
@@ -77,9 +100,29 @@ __device__ inline void epi_store_row8(const Epilogue& ep, uint16_t* out, const f
   }
   epi_u32x4 packed;
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-    packed[q] = (uint32_t)epi_bits<T>(src[2 * q] + b[2 * q]) | ((uint32_t)epi_bits<T>(src[2 * q + 1] + b[2 * q + 1]) << 16);
+  for (int q = 0; q < 4; ++q) {
+    const uint16_t lo = epi_bits<T>(src[2 * q] + b[2 * q]), hi = epi_bits<T>(src[2 * q + 1] + b[2 * q + 1]);
+    packed[q] = (uint32_t)lo | ((uint32_t)hi << 16);
+    mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(epi_float<T>(lo)), __builtin_fabsf(epi_float<T>(hi))));
+  }
   *reinterpret_cast<epi_u32x4*>(out + (size_t)row * N + col) = packed;
+  return mx;
+}
+
+// The tile kernels' form: every lane of the wave makes the call, `live` says whether this lane has a segment to store;
+// the eight lanes lane & ~7 .. hold the same row (when `row_ok`), so with ep.row_absmax set they agree on the row's
+// maximum over their 64 columns before one of them merges it.
+template <typename T>
+__device__ inline void epi_store_row8_wave(const Epilogue& ep, uint16_t* out, const float (&src)[8], int row, int col,
+                                           int N, bool live, bool row_ok, int lane) {
+  float mx = 0.f;
+  if (live) mx = epi_store_row8<T>(ep, out, src, row, col, N);
+  if (ep.row_absmax) {
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) mx = __builtin_fmaxf(mx, __shfl_xor(mx, off));
+    if ((lane & 7) == 0 && row_ok)
+      atomicMax(reinterpret_cast<unsigned*>(ep.row_absmax) + row, __builtin_bit_cast(unsigned, mx));
+  }
 }
 
 }  // namespace ksq

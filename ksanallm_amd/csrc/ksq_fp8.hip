@@ -90,6 +90,27 @@ __global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* x, const 
     qr[i] = quantize_one(load_as_float<T>(xr, i), s);
 }
 
+// per-token with the rows' maxima known (merged in by the GEMM that produced x): the scale, then one pass over the row.
+// VEC: rows of whole 16-byte chunks (k % 8 == 0 and 16-byte aligned rows), eight elements per thread and step.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void quantize_rows_from_absmax_kernel(const uint16_t* x, size_t k, const float* row_absmax,
+                                                                        uint8_t* q, float* scale) {
+  const size_t row = blockIdx.x;
+  const float s = fmaxf(row_absmax[row] / kE4m3Max, kMinScale);
+  if (threadIdx.x == 0) scale[row] = s;
+  if constexpr (VEC) {
+    const u32x4* xv = reinterpret_cast<const u32x4*>(x + row * k);
+    u32x2* qv = reinterpret_cast<u32x2*>(q + row * k);
+    for (size_t i = threadIdx.x; i < k / 8; i += 256) {
+      float f[8];
+      fp8ops::unpack8<T>(xv[i], f);
+      qv[i] = fp8ops::quantize8(f, s);
+    }
+  } else {
+    for (size_t i = threadIdx.x; i < k; i += 256) q[row * k + i] = quantize_one(load_as_float<T>(x + row * k, i), s);
+  }
+}
+
 // per-token: one block per row computes the row's scale and quantises the row
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_per_token_kernel(const uint16_t* x, size_t k, uint8_t* q,
@@ -671,9 +692,10 @@ int ksq_fp8_gemm(int out_dtype, void* out, const void* act_q, const float* act_s
                          KSQ_EPILOGUE_NONE, nullptr, workspace, workspace_bytes, stream);
 }
 
-int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
-                    const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
-                    int epilogue, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+static int fp8_gemm_impl(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                         const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                         int epilogue, const void* bias, float* row_absmax, void* workspace, size_t workspace_bytes,
+                         void* stream) {
   reset_launch_note();
   KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
               "bad epilogue %d", epilogue);
@@ -684,6 +706,7 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
   Epilogue epi;
   epi.kind = epilogue;
   epi.bias = bias;
+  epi.row_absmax = row_absmax;
   KSQ_REQUIRE(out_dtype == KSQ_F16 || out_dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", out_dtype);
   KSQ_REQUIRE(out && act_q && w_q, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
   // the reference layer refuses a missing weight scale (KS/layers/nvidia/fp8_matmul_layer.cpp:49-51)
@@ -745,6 +768,56 @@ int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* ac
   note_launch("fp8_stream_kernel<mt=%d> grid=(%u,%u,%u)", plan.MT, grid.x, grid.y, grid.z);
   if (out_dtype == KSQ_F16) launch_fp8_stream<_Float16>(plan.MT, a, grid, s);
   else launch_fp8_stream<__bf16>(plan.MT, a, grid, s);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+int ksq_fp8_gemm_ex(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                    const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                    int epilogue, const void* bias, void* workspace, size_t workspace_bytes, void* stream) {
+  return fp8_gemm_impl(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k, epilogue,
+                       bias, nullptr, workspace, workspace_bytes, stream);
+}
+
+int ksq_fp8_gemm_rowmax(int out_dtype, void* out, const void* act_q, const float* act_scale, size_t act_scale_count,
+                        const void* w_q, const float* w_scale, size_t w_scale_count, size_t m, size_t n, size_t k,
+                        int epilogue, const void* bias, float* row_absmax, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+  KSQ_REQUIRE(row_absmax != nullptr && (reinterpret_cast<uintptr_t>(row_absmax) & 3) == 0, KSQ_ERR_INVALID_ARGUMENT,
+              "row_absmax is null or misaligned");
+  return fp8_gemm_impl(out_dtype, out, act_q, act_scale, act_scale_count, w_q, w_scale, w_scale_count, m, n, k, epilogue,
+                       bias, row_absmax, workspace, workspace_bytes, stream);
+}
+
+int ksq_fill_zero_f32(float* p, size_t count, void* stream) {
+  KSQ_REQUIRE(p != nullptr || count == 0, KSQ_ERR_INVALID_ARGUMENT, "null pointer");
+  if (count == 0) return KSQ_OK;
+  KSQ_REQUIRE(count < (1ull << 31), KSQ_ERR_UNSUPPORTED, "count too large");
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     p, (int)count);
+  KSQ_HIP_TRY(hipGetLastError());
+  return KSQ_OK;
+}
+
+// scale[r] = max(row_absmax[r] / 448, floor), then the quantisation pass of the per-token mode on its own
+int ksq_fp8_quantize_rows_from_absmax(int dtype, const void* act, size_t m, size_t k, const float* row_absmax,
+                                      void* act_q, float* act_scale, void* stream) {
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(act && act_q && act_scale && row_absmax, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
+  if (m == 0 || k == 0) return KSQ_OK;
+  KSQ_REQUIRE(m < (1ull << 31), KSQ_ERR_UNSUPPORTED, "m=%zu too large", m);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint16_t* x = static_cast<const uint16_t*>(act);
+  uint8_t* q = static_cast<uint8_t*>(act_q);
+  const bool vec = k % 8 == 0 && (reinterpret_cast<uintptr_t>(act) & 15) == 0 && (reinterpret_cast<uintptr_t>(act_q) & 7) == 0;
+  const dim3 grid((unsigned)m), block(256);
+  if (dtype == KSQ_F16) {
+    if (vec) hipLaunchKernelGGL((quantize_rows_from_absmax_kernel<_Float16, true>), grid, block, 0, s, x, k, row_absmax, q, act_scale);
+    else hipLaunchKernelGGL((quantize_rows_from_absmax_kernel<_Float16, false>), grid, block, 0, s, x, k, row_absmax, q, act_scale);
+  } else {
+    if (vec) hipLaunchKernelGGL((quantize_rows_from_absmax_kernel<__bf16, true>), grid, block, 0, s, x, k, row_absmax, q, act_scale);
+    else hipLaunchKernelGGL((quantize_rows_from_absmax_kernel<__bf16, false>), grid, block, 0, s, x, k, row_absmax, q, act_scale);
+  }
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

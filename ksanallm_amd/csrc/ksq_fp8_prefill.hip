@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
       float vals[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * as;
-      if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
+      epi_store_row8_wave<T>(p.epi, out, vals, row, col, p.N, row < p.M && col + 8 <= p.N, row < p.M, lane);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);  // ... and its reads, before the next row tile overwrites the slab
   }
@@ -476,7 +476,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
       float vals[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * as;
-      if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
+      epi_store_row8_wave<T>(p.epi, out, vals, row, col, p.N, row < p.M && col + 8 <= p.N, row < p.M, lane);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -507,7 +507,8 @@ __global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) 
     const float w = p.w_scale[p.w_scale_per_col ? col + q : 0];
     vals[q] = ((q < 4 ? lo[q] : hi[q - 4]) * w) * as;  // the order of the one-launch epilogue: column scale, then row scale
   }
-  epi_store_row8<T>(p.epi, static_cast<uint16_t*>(p.out), vals, row, col, p.N);
+  const float mx = epi_store_row8<T>(p.epi, static_cast<uint16_t*>(p.out), vals, row, col, p.N);
+  if (p.epi.row_absmax) atomicMax(reinterpret_cast<unsigned*>(p.epi.row_absmax) + row, __builtin_bit_cast(unsigned, mx));
 }
 
 }  // namespace

@@ -188,6 +188,7 @@ const DeviceInfo* device_info();  // of the current device; nullptr on failure
 struct Epilogue {
   int kind = KSQ_EPILOGUE_NONE;
   const void* bias = nullptr;  // T [n], 16-byte aligned
+  float* row_absmax = nullptr;  // [m]: largest |stored value| per row, merged in by atomic maximum (or none)
 };
 
 // ---- launch plans ------------------------------------------------------------------------------------------

@@ -371,7 +371,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       float vals[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs * cf[q];
-      if (row < p.M && col + 8 <= p.N) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
+      epi_store_row8_wave<T>(p.epi, out, vals, row, col, p.N, row < p.M && col + 8 <= p.N, row < p.M, lane);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void w
       float vals[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs * cf[q];
-      if (live) epi_store_row8<T>(p.epi, out, vals, row, col, p.N);
+      epi_store_row8_wave<T>(p.epi, out, vals, row, col, p.N, live, row < p.M, lane);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -615,7 +615,8 @@ __global__ __launch_bounds__(256) void w4a16_splitk_reduce_kernel(const float* _
   if (sz) column_factors(sz, G, col, cf);  // bf16 scales: the column's 2^E
   const float vals[8] = {lo[0] * rs * cf[0], lo[1] * rs * cf[1], lo[2] * rs * cf[2], lo[3] * rs * cf[3],
                          hi[0] * rs * cf[4], hi[1] * rs * cf[5], hi[2] * rs * cf[6], hi[3] * rs * cf[7]};
-  epi_store_row8<T>(epi, out, vals, (int)row, col, N);
+  const float mx = epi_store_row8<T>(epi, out, vals, (int)row, col, N);
+  if (epi.row_absmax) atomicMax(reinterpret_cast<unsigned*>(epi.row_absmax) + row, __builtin_bit_cast(unsigned, mx));
 }
 
 template <typename T>

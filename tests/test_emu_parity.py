@@ -94,4 +94,6 @@ test_act_perm_without_workspace_is_refused = nxt.test_act_perm_without_workspace
 test_silu_mul_epilogue = nxt.test_silu_mul_epilogue
 test_bias_epilogue = nxt.test_bias_epilogue
 test_fp8_epilogues = nxt.test_fp8_epilogues
+test_w4a16_gemm_row_maxima_feed_the_quantiser = nxt.test_w4a16_gemm_row_maxima_feed_the_quantiser
+test_fp8_gemm_row_maxima = nxt.test_fp8_gemm_row_maxima
 test_static_scratch_matches_workspace_entry_point = noalloc.test_static_scratch_matches_workspace_entry_point

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as orc
-from tests.ksq_testlib import ORC_DT, W4Case, capi_dtype, torch_dtype
+from tests.ksq_testlib import ORC_DT, W4Case, W4Device, capi_dtype, torch_dtype
 
 pytestmark = pytest.mark.gpu
 
@@ -353,3 +353,81 @@ def test_fp8_epilogues(gpu, out_dtype, per_channel, M, kstat, K, epilogue):
                          K, epi, bias, ws, ws_bytes)
     torch.cuda.synchronize()
     orc.assert_parity(out.float().cpu().numpy(), want, f"fp8 {epilogue} M={M} per_channel={per_channel}")
+
+
+# ---- F2, producer side: row maxima out of the GEMM's epilogue, consumed by the per-token FP8 quantiser ------------------
+ROWMAX_CASES = [("kstat", 5, {}), ("kstat", 16, {}), ("kstat_splitk", 16, {"KSQ_W4_KSPLIT": 2}),
+                ("astream", 40, {"KSQ_W4_ASTREAM": 1}), ("astream_lds", 64, {"KSQ_W4_ASTREAM": 1, "KSQ_W4_ASTREAM_LDS": 1}),
+                ("stream", 9, {"KSQ_W4_KSTAT": 0}), ("rows64", 100, {"KSQ_W4_PREFILL_ROWS": 64}),
+                ("rows64_splitk", 100, {"KSQ_W4_PREFILL_ROWS": 64, "KSQ_W4_PREFILL_KSPLIT": 2}),
+                ("rows128", 200, {"KSQ_W4_PREFILL_ROWS": 128}), ("auto", 300, {})]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("epilogue", ["none", "silu_mul"])
+@pytest.mark.parametrize("route,M,env", ROWMAX_CASES)
+def test_w4a16_gemm_row_maxima_feed_the_quantiser(gpu, dtype, epilogue, route, M, env):
+    """ksq_w4a16_gemm_rowmax: the output equals the plain GEMM's bit for bit, row_absmax is exactly the largest |out| of
+    every row as stored, and the one-pass quantiser fed with it writes the bytes and scales of the two-pass one."""
+    import torch
+
+    from ksanallm_amd import capi
+
+    case = W4Case(2300 + M, M, 1024, 544, g=128, kind="awq", dtype=dtype)
+    dev = W4Device(case, gpu)
+    big = torch.empty(16 << 20, dtype=torch.uint8, device=gpu)
+    epi = capi.EPILOGUE_SILU_MUL if epilogue == "silu_mul" else capi.EPILOGUE_NONE
+    cols = case.N // 2 if epi == capi.EPILOGUE_SILU_MUL else case.N
+    tdt, cdt = torch_dtype(dtype), capi_dtype(dtype)
+    ref = torch.full((M, cols), float("nan"), dtype=tdt, device=gpu)
+    out = torch.full((M, cols), float("nan"), dtype=tdt, device=gpu)
+    rowmax = torch.full((M,), 123.0, dtype=torch.float32, device=gpu)
+    with _env(**env):
+        capi.w4a16_gemm_ex(cdt, ref, dev.act, dev.weight, dev.sz, M, case.N, case.K, case.g, None, epi, None, big, big.numel())
+        capi.fill_zero_f32(rowmax, M)
+        capi.w4a16_gemm_rowmax(cdt, out, dev.act, dev.weight, dev.sz, M, case.N, case.K, case.g, rowmax, epi, None, big,
+                               big.numel())
+    torch.cuda.synchronize()
+    assert torch.equal(ref.view(torch.int16), out.view(torch.int16)), route
+    want = out.float().abs().max(dim=1).values
+    assert torch.equal(rowmax, want), (route, rowmax[:4], want[:4])
+    # consumer: one pass with the known maxima == max pass + quantise
+    q1 = torch.empty((M, cols), dtype=torch.uint8, device=gpu)
+    s1 = torch.empty(M, dtype=torch.float32, device=gpu)
+    q2, s2 = torch.empty_like(q1), torch.empty_like(s1)
+    capi.fp8_quantize(cdt, out, M, cols, capi.FP8_PER_TOKEN_DYNAMIC, q1, s1)
+    capi.fp8_quantize_rows_from_absmax(cdt, out, M, cols, rowmax, q2, s2)
+    torch.cuda.synchronize()
+    assert torch.equal(s1, s2) and torch.equal(q1, q2), route
+
+
+@pytest.mark.parametrize("out_dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,env", [(1, 1024, {}), (16, 1024, {}), (16, 1024, {"KSQ_FP8_KSTAT": 0}), (40, 1024, {}),
+                                     (100, 1024, {}), (300, 1024, {}), (300, 4096, {"KSQ_FP8_TAIL_KSPLIT": 2}),
+                                     (130, 1024, {"KSQ_FP8_PREFILL_TILE": 128}), (7, 1008, {})])
+def test_fp8_gemm_row_maxima(gpu, out_dtype, M, K, env):
+    import torch
+
+    from ksanallm_amd import capi
+
+    rng = np.random.default_rng(2400 + M)
+    N = 528
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    xq = codes[rng.integers(0, len(codes), size=(M, K))] & np.uint8(0xBF)
+    wq = codes[rng.integers(0, len(codes), size=(N, K))] & np.uint8(0xBF)
+    xs = ((rng.random(M) + 0.5) * 1e-2).astype(np.float32)
+    ws = ((rng.random(N) + 0.5) * 1e-2).astype(np.float32)
+    tdt, cdt = torch_dtype(out_dtype), capi_dtype(out_dtype)
+    dx, dw = torch.from_numpy(xq).to(gpu), torch.from_numpy(wq).to(gpu)
+    dxs, dws = torch.from_numpy(xs).to(gpu), torch.from_numpy(ws).to(gpu)
+    wsb = capi.fp8_workspace_bytes(M, N, K)
+    wk = torch.empty(max(wsb, 256), dtype=torch.uint8, device=gpu)
+    ref = torch.full((M, N), float("nan"), dtype=tdt, device=gpu)
+    out = torch.full((M, N), float("nan"), dtype=tdt, device=gpu)
+    rowmax = torch.zeros(M, dtype=torch.float32, device=gpu)
+    with _env(**env):
+        capi.fp8_gemm_ex(cdt, ref, dx, dxs, M, dw, dws, N, M, N, K, capi.EPILOGUE_NONE, None, wk, wsb)
+        capi.fp8_gemm_rowmax(cdt, out, dx, dxs, M, dw, dws, N, M, N, K, rowmax, capi.EPILOGUE_NONE, None, wk, wsb)
+    torch.cuda.synchronize()
+    assert torch.equal(ref.view(torch.int16), out.view(torch.int16))
+    assert torch.equal(rowmax, out.float().abs().max(dim=1).values)
