@@ -171,6 +171,12 @@ static int env_int(const char* name, int dflt) {
 // be sliced inside a workgroup (reduced through LDS); measured slower than one slice on MI355X for the decode
 // shapes, so it is off by default (KSQ_W4_SLICES selects it).
 W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
+  return w4a16_plan_with(m, n, k, cus, workspace_bytes, 0, 0);
+}
+
+// nt / ks: column tiles per wave and K splits asked for (0 = the planner's own choice); the split still shrinks to
+// what the workspace holds
+W4Plan w4a16_plan_with(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int nt, int ks) {
   W4Plan p{};
   const size_t ntiles = n / kTileN, ktiles = k / kTileK;
   const size_t simds = (size_t)cus * 4;
@@ -184,6 +190,7 @@ W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes)
     p.mblocks = (int)((m + 63) / 64);
     p.NT = 2;
   }
+  if (nt == 1 || nt == 2 || nt == 4) p.NT = nt;
   int nt_env = env_int("KSQ_W4_NT", 0);
   if (nt_env == 1 || nt_env == 2 || nt_env == 4) p.NT = nt_env;
   p.slices = 1;
@@ -200,6 +207,7 @@ W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes)
     if (wanted > cap) wanted = cap;
     if (wanted < 1) wanted = 1;
     ksplit = wanted;
+    if (ks >= 1 && (size_t)ks <= ktiles) ksplit = (size_t)ks;
     int ks_env = env_int("KSQ_W4_KSPLIT", 0);
     if (ks_env >= 1 && (size_t)ks_env <= ktiles) ksplit = (size_t)ks_env;
     if (ngroups * (size_t)p.mblocks > (size_t)kCountersPerSlot) ksplit = 1;
@@ -315,6 +323,10 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
     if (mm - 15 > max_m) break;
     W4Plan p = w4a16_plan(mm, n, k, cus, (size_t)-1);
     if (p.partial_bytes > best) best = p.partial_bytes;
+    if (mm == 16) {  // the four-way split of the streaming kernel that a very long K is routed to at 9 .. 16 rows
+      const W4Plan lp = w4a16_plan_with(mm, n, k, cus, (size_t)-1, 2, 4);
+      if (lp.partial_bytes > best) best = lp.partial_bytes;
+    }
     KstatPlan kp = w4a16_kstat_plan(mm < max_m ? mm : max_m, n, k, cus, (size_t)-1);
     if (kp.ok && kp.partial_bytes > best) best = kp.partial_bytes;
     const size_t am = mm < max_m ? mm : max_m;
@@ -419,6 +431,18 @@ static int w4a16_gemm_impl(int dtype, void* out, const void* act, const void* we
   }
   if (m <= (size_t)env_int("KSQ_W4_KSTAT_MAX_M", 64) && env_int("KSQ_W4_KSTAT", 1) != 0) {
     KstatPlan kp = w4a16_kstat_plan(m, n, k, di->cus, workspace_bytes, g);
+    // A K that the k-stationary kernel would split four ways or more across workgroups (nine to sixteen rows; fewer
+    // rows walk K in phases instead): every workgroup then covers a quarter of K or less for many column tiles and
+    // ends every batch in a hand-over.  The streaming kernel with two column tiles per wave and four splits is the
+    // faster one there (Llama-3-70B down, K = 28672, sixteen rows: 38.4 -> 31.5 us).
+    const bool long_k = kp.ok && !kp.phases && kp.mt == 1 && kp.ksplit >= 4 && env_int("KSQ_W4_LONG_K_STREAM", 1) != 0;
+    if (long_k) {
+      W4Plan lp = w4a16_plan(m, n, k, di->cus, workspace_bytes);
+      if (lp.ksplit > 1) {  // the workspace holds its partial tiles
+        lp = w4a16_plan_with(m, n, k, di->cus, workspace_bytes, 2, 4);
+        if (lp.ksplit == 4) return w4a16_launch_stream(dtype, lp, out, act, weight, sz, m, n, k, g, workspace, s, epi);
+      }
+    }
     if (kp.ok) return w4a16_launch_kstat(dtype, kp, out, act, weight, sz, m, n, k, g, workspace, s, epi);
   }
   W4Plan plan = w4a16_plan(m, n, k, di->cus, workspace_bytes);

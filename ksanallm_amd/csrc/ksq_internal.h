@@ -202,6 +202,7 @@ struct W4Plan {
   bool prefill;  // true: LDS-tiled MFMA kernel, false: streaming kernel
 };
 W4Plan w4a16_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);
+W4Plan w4a16_plan_with(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes, int nt, int ks);
 
 int w4a16_launch_stream(int dtype, const W4Plan& plan, void* out, const void* act, const void* weight,
                         const void* sz, size_t m, size_t n, size_t k, size_t g, void* workspace, hipStream_t s,
@@ -231,6 +232,7 @@ struct KstatPlan {
   int nt_per_wg; // column tiles per workgroup
   int grid_x;
   int nb;        // column tiles per batch (= ring depth / tpw)
+  bool phases;   // K walked in phases inside the workgroup (w4a16_kphase_kernel) instead of split over grid.y
   size_t partial_bytes;
 };
 // g = the group size where the caller knows it (it picks the batch size only; the workspace a plan needs does not

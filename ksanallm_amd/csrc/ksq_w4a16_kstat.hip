@@ -318,6 +318,172 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 }
 
+// The same k-stationary decomposition for a K too long for one pass (more k tiles than 16 waves hold as activation
+// fragments) at one to eight rows: instead of splitting K over workgroups -- partial tiles through memory, arrival
+// counters, and a workgroup that covers a fraction of K for many column tiles -- the workgroup walks K in phases of
+// 16 x TPW k tiles.  Every wave keeps its own fp32 partial tile of each of the workgroup's NB column tiles across
+// the phases; per phase it swaps in the activation fragments of its next TPW k tiles (requested a phase ahead in
+// the compact form they are loaded in: few rows, so few registers) and streams the NB x TPW weight tiles through the
+// same register ring.  Nothing is shared between waves until the one reduction through LDS at the end: no barrier
+// and no hand-over in the loop.  With few rows the activations are a small part of what a compute unit loads
+// (one or two instructions per k tile against NB of weights); with sixteen rows they would be four per k tile, which
+// is why this form stops at eight.
+template <typename T, int GPT, int TPW, int NB, int PPI>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void w4a16_kphase_kernel(KstatArgs p) {
+  static_assert(PPI == 8 || PPI == 16, "up to eight rows");
+  constexpr int NW = 16, API = 16 / PPI, DPG = 4 / GPT, D = NB * TPW, KP = NW * TPW;
+  constexpr int GW = TPW * GPT, SZR = (NB * GW * 16 + 63) / 64;
+  using O = Ops<T>;
+  __shared__ f32x4 red[NB * NW * 64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, j = lane >> 4;
+  const int nt_begin = blockIdx.x * NB;
+  int count = p.ntiles - nt_begin;
+  count = count < NB ? count : NB;
+  const int nphases = (p.KT + KP - 1) / KP;
+  const int kt0 = wave * TPW;  // first k tile of this wave in phase 0; phase ph adds ph * KP
+
+  // Resources start at (nt_begin, kt0) and end with the last k tile of the workgroup's last column tile: a column tile
+  // past `count` starts KT tiles further on and is out of range whatever the phase.  k tiles past K (the last phase
+  // of the last waves) are parked out of range explicitly.
+  const size_t kt0c = kt0 < p.KT ? (size_t)kt0 : (size_t)p.KT - 1;
+  const bool any = count > 0 && kt0 < p.KT;
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(p.weight) + ((size_t)nt_begin * p.KT + kt0c) * 1024), 0,
+      any ? ((count - 1) * p.KT + (p.KT - kt0)) * 1024 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_sz = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(static_cast<const char*>(p.sz) + ((size_t)nt_begin * p.G + kt0c * GPT) * 64), 0,
+      any ? ((count - 1) * p.G + (p.KT - kt0) * GPT) * 64 : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.act), 0, (int)((size_t)p.M * p.K * 2), 0x00020000);
+  const unsigned w_stride = (unsigned)p.KT * 1024u, sz_stride = (unsigned)p.G * 64u;
+
+  u32x4 araw[TPW][API];  // the next phase's activations as loaded: lane l = row l / PPI, piece i * PPI + l % PPI
+  auto load_a = [&](int ph) {
+    const int lr = lane / PPI, lp = lane % PPI;
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int i = 0; i < API; ++i) {
+        const int kt = kt0 + ph * KP + t;
+        const bool ok = lr < p.M && kt < p.KT;
+        const unsigned ao = ok ? ((unsigned)lr * p.K + kt * kTileK + 8 * (i * PPI + lp)) * 2u : 0x80000000u;
+        araw[t][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ao, 0, 0));
+      }
+  };
+  u32x4 wq[D];
+  uint32_t szraw[SZR];
+  auto fetch = [&](int slot, int i, int t, int ph) {
+    const bool ok = kt0 + ph * KP + t < p.KT;
+    const unsigned off = ok ? (unsigned)(ph * KP + t) * 1024u + lane * 16u + i * w_stride : 0x80000000u;
+    wq[slot] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, off, 0, 2));
+  };
+  auto fetch_sz = [&](int ph) {
+#pragma unroll
+    for (int r = 0; r < SZR; ++r) {
+      const int f = 64 * r + lane, i = f / (16 * GW), gq = (f >> 4) % GW;
+      const bool ok = i < NB && kt0 + ph * KP + gq / GPT < p.KT;
+      const unsigned off = ok ? (unsigned)i * sz_stride + (unsigned)(ph * KP * GPT + gq) * 64u + (unsigned)c * 4u : 0x80000000u;
+      szraw[r] = __builtin_amdgcn_raw_buffer_load_b32(rs_sz, off, 0, 0);
+    }
+  };
+
+  uint32_t m_lo = O::kMaskLo, m_hi = O::kMaskHi, c_lo = O::kMagicLo, c_hi = O::kMagicHi;
+  KSQ_PIN_SGPR(m_lo);
+  KSQ_PIN_VGPR(c_lo);
+  KSQ_PIN_VGPR(c_hi);
+  KSQ_PIN_VGPR(m_hi);
+
+  load_a(0);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_sz(0);
+#pragma unroll
+  for (int q = 0; q < D; ++q) {
+    fetch(q, q / TPW, q % TPW, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  f32x4 acc[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int sz_lane = c * 4;
+  for (int ph = 0; ph < nphases; ++ph) {
+    // this phase's activation fragments: lane 16 j + c takes piece 4 d + j of row c, loaded by instruction
+    // (4 d + j) / PPI, lane c * PPI + (4 d + j) % PPI; rows that were not loaded are zero
+    u32x4 af[TPW][4];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const int piece = 4 * d + j;
+        const int from = (c * PPI + piece % PPI) * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint32_t v;
+          if constexpr (PPI == 8) v = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)araw[t][d >> 1][q]);
+          else v = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)araw[t][0][q]);
+          af[t][d][q] = c < 64 / PPI ? v : 0u;
+        }
+      }
+    uint32_t szq[D][GPT];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int gi = 0; gi < GPT; ++gi) {
+          const int f16 = (i * TPW + t) * GPT + gi;
+          szq[i * TPW + t][gi] = (uint32_t)__builtin_amdgcn_ds_bpermute(sz_lane + 64 * (f16 & 3), (int)szraw[f16 >> 2]);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+    load_a(ph + 1);  // a phase past the end is parked: nothing is read
+    fetch_sz(ph + 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) {
+        const int slot = i * TPW + t;
+#pragma unroll
+        for (int gi = 0; gi < GPT; ++gi) {
+          const uint32_t szw = szq[slot][gi];
+          const uint32_t z = (szw >> 16) & 15u;
+          const float s = O::scale_to_float(szw);
+          const u32x4 corr = O::correction(z | (z << 16));
+          f32x4 P = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int dd = 0; dd < DPG; ++dd) {
+            const int d = gi * DPG + dd;
+            const u32x4 bw = O::unpack(wq[slot][d], m_lo, m_hi, c_lo, c_hi);
+            P = O::mfma(af[t][d], corr, P);
+            P = O::mfma(af[t][d], bw, P);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][e] += s * P[e];
+        }
+        fetch(slot, i, t, ph + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  }
+
+  // ---- the 16 k slices of every column tile, summed in wave order by wave i of tile i
+#pragma unroll
+  for (int i = 0; i < NB; ++i) red[(i * NW + wave) * 64 + lane] = acc[i];
+  __syncthreads();
+  if (wave < NB) {
+    f32x4 part[NW];
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) part[ww] = red[(wave * NW + ww) * 64 + lane];
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) sum += part[ww];
+    // every lane makes the call (the epilogue may exchange lanes); a column tile past the range stores nothing
+    epi_store_acc<T>(p.epi, static_cast<uint16_t*>(p.out), sum, 4 * j, (nt_begin + wave) * 16 + c, p.M, p.N, wave < count);
+  }
+}
+
 #define KSQ_GO4(MT, TPW, NB, NW) \
   hipLaunchKernelGGL((w4a16_kstat_kernel<T, GPT, MT, TPW, NB, NW, 4>), grid, dim3(64 * NW), 0, s, a)
 // one row tile: the activation loads widen as the rows get fewer
@@ -369,6 +535,26 @@ void launch(const KstatPlan& pl, const KstatArgs& a, dim3 grid, hipStream_t s) {
 #undef KSQ_GO
 #undef KSQ_GO4
 
+template <typename T, int GPT>
+bool launch_kphase(int nb, int ppi, const KstatArgs& a, dim3 grid, hipStream_t s) {
+#define KSQ_PH(NB, PPI) hipLaunchKernelGGL((w4a16_kphase_kernel<T, GPT, 2, NB, PPI>), grid, dim3(1024), 0, s, a)
+  if (ppi == 16) {
+    if (nb == 1) KSQ_PH(1, 16);
+    else if (nb == 2) KSQ_PH(2, 16);
+    else if (nb == 3) KSQ_PH(3, 16);
+    else if (nb == 4) KSQ_PH(4, 16);
+    else return false;
+  } else {
+    if (nb == 1) KSQ_PH(1, 8);
+    else if (nb == 2) KSQ_PH(2, 8);
+    else if (nb == 3) KSQ_PH(3, 8);
+    else if (nb == 4) KSQ_PH(4, 8);
+    else return false;
+  }
+#undef KSQ_PH
+  return true;
+}
+
 }  // namespace
 
 // Plan of the k-stationary kernel: row tiles (1, 2 or 4), waves per workgroup (16 for one row tile, else 8), k
@@ -403,6 +589,23 @@ KstatPlan w4a16_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t workspa
   if (const char* e = tuning_env("KSQ_W4_KSPLIT")) {  // tuning / test override; never below what the registers need
     const size_t v = (size_t)atoi(e);
     if (v > ksplit && v <= ktiles) ksplit = v;
+  }
+  // One to eight rows and a K that one pass does not cover: phases inside the workgroup instead of a split across
+  // workgroups, where the column tiles alone give every CU one to four of them (see w4a16_kphase_kernel).  Measured
+  // against the split: Llama-3-70B down (K = 28672) at one token 36.6 us, Llama-2-7B down 9.5 us.
+  bool phases = p.mt == 1 && m <= 8 && ksplit >= 2 && ntiles * 4 >= 3 * (size_t)cus && ntiles <= 4 * (size_t)cus;
+  if (const char* e = tuning_env("KSQ_W4_KPHASE")) {  // tuning / test switch: 0 = never, 1 = whenever the kernel can
+    phases = atoi(e) != 0 && p.mt == 1 && m <= 8 && ntiles <= 4 * (size_t)cus && ktiles >= 2;
+  }
+  if (phases) {
+    p.phases = true;
+    p.ksplit = 1;
+    p.tpw = 2;
+    p.nb = (int)((ntiles + (size_t)cus - 1) / (size_t)cus);
+    p.nt_per_wg = p.nb;
+    p.grid_x = (int)((ntiles + p.nb - 1) / p.nb);
+    p.partial_bytes = 0;
+    return p;
   }
   auto need = [&](size_t ks) { return ks <= 1 ? (size_t)0 : ks * ntiles * p.mt * 64 * 16; };
   if (need(ksplit) > workspace_bytes) {
@@ -502,6 +705,16 @@ int w4a16_launch_kstat(int dtype, const KstatPlan& plan, void* out, const void* 
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
   const int gpt = (int)(kTileK / g);
+  if (plan.phases) {
+    const int ppi = m <= 4 ? 16 : 8;
+    note_launch("w4a16_kphase_kernel<tpw=2,nb=%d,gpt=%d,ppi=%d> grid=(%d)", plan.nb, gpt, ppi, plan.grid_x);
+    bool ok;
+    if (dtype == KSQ_F16) ok = gpt == 1 ? launch_kphase<_Float16, 1>(plan.nb, ppi, a, grid, s) : launch_kphase<_Float16, 2>(plan.nb, ppi, a, grid, s);
+    else ok = gpt == 1 ? launch_kphase<__bf16, 1>(plan.nb, ppi, a, grid, s) : launch_kphase<__bf16, 2>(plan.nb, ppi, a, grid, s);
+    KSQ_REQUIRE(ok, KSQ_ERR_UNSUPPORTED, "no phase kernel for %d column tiles per workgroup", plan.nb);
+    KSQ_HIP_TRY(hipGetLastError());
+    return KSQ_OK;
+  }
   note_launch("w4a16_kstat_kernel<mt=%d,tpw=%d,nb=%d,nw=%d,gpt=%d,ppi=%d> grid=(%d,%d) nt_per_wg=%d", plan.mt, plan.tpw,
               plan.nb, plan.nw, gpt, plan.mt == 1 ? (m <= 4 ? 16 : (m <= 8 ? 8 : 4)) : 4, plan.grid_x, plan.ksplit,
               plan.nt_per_wg);

@@ -27,6 +27,12 @@ def w4_cases(full):
         for g, dt, ws in (combos if full else [combos[i % 8], combos[(i + 3) % 8]]):
             if K % g == 0 and (K % 128 == 0 or g == 64):
                 out.append((M, N, K, g, dt, ws))
+    # K long enough that the decode kernels walk it in phases (up to eight rows), split it over workgroups, or hand it
+    # to the streaming kernel with a four-way split (nine to sixteen rows)
+    for i, (K, M, N) in enumerate(itertools.product([6272, 8320, 25088], [1, 4, 5, 8, 9, 16, 17, 33], [16, 272, 4112, 8192])):
+        combos = list(itertools.product([64, 128], ["f16", "bf16"], [True, False]))
+        for g, dt, ws in (combos if full else [combos[i % 8], combos[(i + 5) % 8]]):
+            out.append((M, N, K, g, dt, ws))
     return out
 
 

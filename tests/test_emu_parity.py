@@ -61,6 +61,7 @@ test_k_odd_multiple_of_64 = w4.test_k_odd_multiple_of_64
 test_no_workspace_still_correct = w4.test_no_workspace_still_correct
 test_caller_bound_split_k_counters_and_launch_log = w4.test_caller_bound_split_k_counters_and_launch_log
 test_k_tiles_per_wave = w4.test_k_tiles_per_wave
+test_k_phases_inside_the_workgroup = w4.test_k_phases_inside_the_workgroup
 
 # ---- FP8 -------------------------------------------------------------------------------------------------------------------
 test_per_channel_quantize_reference_shapes = f8.test_per_channel_quantize_reference_shapes

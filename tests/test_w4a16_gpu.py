@@ -370,6 +370,29 @@ def test_k_odd_multiple_of_64(gpu, dtype, kind, M, K, N):
     assert e.value.code == capi.ERR_WORKSPACE
 
 
+@pytest.mark.parametrize("dtype,g", [("f16", 128), ("bf16", 64), ("f16", 64), ("bf16", 128)])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 272), (3, 2176, 528), (4, 4224, 272), (5, 2176, 1040), (8, 8320, 272),
+                                   (2, 384, 4112), (7, 640, 8208), (4, 384, 12304), (1, 256, 16)])
+def test_k_phases_inside_the_workgroup(gpu, dtype, g, M, K, N):
+    """One to eight rows with K walked in phases inside the workgroup (what long K gets instead of a split across
+    workgroups): whole and partial last phases, one to four column tiles per workgroup, a ragged last workgroup; no
+    workspace needed; two runs bit for bit."""
+    from ksanallm_amd import capi
+
+    case = W4Case(1900 + M + K // 128, M, K, N, g=g, kind="awq", dtype=dtype)
+    dev = W4Device(case, gpu)
+    capi.set_launch_log(True)
+    try:
+        with _env(KSQ_W4_KPHASE=1):
+            got1 = dev.gemm_f32(use_workspace=False)
+            assert "w4a16_kphase_kernel" in capi.last_launch(), capi.last_launch()
+            got2 = dev.gemm_f32()
+    finally:
+        capi.set_launch_log(False)
+    orc.assert_parity(got1, case.oracle(), f"k phases M={M} K={K} N={N} {dtype} g={g}")
+    assert np.array_equal(got1, got2)
+
+
 def test_caller_bound_split_k_counters_and_launch_log(gpu):
     """Split-K with the arrival counters in the caller's memory: same bits as with the library's, the memory is back at
     zero after every launch, and the launch log names the kernel and its split."""
