@@ -212,6 +212,7 @@ struct PrefillPlan {
   int knt;     // 64-row kernel: column tiles per wave (1, 2 or 4)
   int nw;      // 128-row kernel: waves side by side (4 or 8)
   int kg;      // 128-row kernel with four waves side by side: k groups of such waves (1 or 2)
+  int ct;      // 128-row kernel: column tiles per wave (4 or 3: 64 or 48 columns)
   int ksplit;  // 64-row kernel: grid.y
   size_t partial_bytes;
 };

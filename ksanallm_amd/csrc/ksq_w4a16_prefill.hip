@@ -143,9 +143,12 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_long_kernel(const uint16
   }
 }
 
-template <typename T, int GPT, int NW, int KG = 1>
+// CT = column tiles per wave: 4 (64 columns: tiles of 256 or 512 columns) or 3 (48 columns: 192 or 384), for
+// widths whose number of tiles falls better on the compute units (a partly filled last round costs a full one).
+template <typename T, int GPT, int NW, int KG = 1, int CT = 4>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
   static_assert(NW == 4 || NW == 8, "four or eight waves side by side");
+  static_assert(CT == 3 || CT == 4, "three or four column tiles per wave");
   // KG = 2: two groups of four waves on the same 128 x 256 tile, the first on the even k tiles, the second on the
   // odd ones, each with its own pair of activation stages; the second group's accumulators reach the first through
   // LDS at the end.  For grids that put one workgroup on a CU: two waves per SIMD instead of one.
@@ -171,11 +174,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   int mb, nb;
   if (!tile_of(tile_logical_id(blockIdx.x, gridDim.x), p.mblocks, p.nblocks, &mb, &nb)) return;  // rounding of the grid
   const int m0 = mb * kBM;
-  const int nt0 = (nb * NW + wave) * kNT;
+  const int nt0 = (nb * NW + wave) * CT;
 
-  __amdgpu_buffer_rsrc_t rs_w[kNT], rs_sz[kNT];
+  __amdgpu_buffer_rsrc_t rs_w[CT], rs_sz[CT];
 #pragma unroll
-  for (int t = 0; t < kNT; ++t) {
+  for (int t = 0; t < CT; ++t) {
     const int nt = nt0 + t;
     const bool ok = nt < p.ntiles;
     const size_t ntc = ok ? (size_t)nt : 0;
@@ -209,15 +212,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   const int a_lane = (c >> 2) * 64 + (c & 3) * 4 + (j ^ (c >> 2));
   const unsigned w_voff = lane * 16u, sz_voff = c * 4u;
 
-  f32x4 acc[kMT][kNT];
+  f32x4 acc[kMT][CT];
 #pragma unroll
   for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
-    for (int t = 0; t < kNT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < CT; ++t) acc[mt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   struct BTile {
-    u32x4 w[kNT];
-    uint32_t sz[kNT][GPT];
+    u32x4 w[CT];
+    uint32_t sz[CT][GPT];
   };
   BTile b0, b1;
 
@@ -234,6 +237,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i],
                                                  (kt < p.KT ? kt : p.KT - 1) * 256, 0, 0);
       }
+    } else if (q >= CT) {  // three column tiles per wave: part 3 carries activations only
     } else if (item == 2) {
       b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
     } else {
@@ -260,9 +264,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
     for (int i = 0; i < 4; ++i) a[i] = buf[(4 * h + i) * 256 + ks * 16 + a_lane];
   };
-  auto mfma_row = [&](const u32x4& a, const u32x4 (&b)[kNT], int mt) {
+  auto mfma_row = [&](const u32x4& a, const u32x4 (&b)[CT], int mt) {
 #pragma unroll
-    for (int t = 0; t < kNT; ++t) acc[mt][t] = O::mfma(a, b[t], acc[mt][t]);
+    for (int t = 0; t < CT; ++t) acc[mt][t] = O::mfma(a, b[t], acc[mt][t]);
   };
   // One k tile.  On entry everything in flight (this tile's activations and weights) has landed and is visible to
   // the whole workgroup, and every wave is done with the other buffer.
@@ -274,9 +278,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     read_half(a0, cur, 0, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      u32x4 b[kNT];
+      u32x4 b[CT];
 #pragma unroll
-      for (int t = 0; t < kNT; ++t) {
+      for (int t = 0; t < CT; ++t) {
         const typename DQ::Consts k = DQ::prepare(bt.sz[t][GPT == 2 ? (ks >> 1) : 0]);
         b[t] = DQ::run(bt.w[t][ks], k, m_lo, m_hi, g_lo, g_hi);
       }
@@ -336,14 +340,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
 #pragma unroll
       for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
-        for (int t = 0; t < kNT; ++t) park[(mt * kNT + t) * 64 + lane] = acc[mt][t];
+        for (int t = 0; t < CT; ++t) park[(mt * CT + t) * 64 + lane] = acc[mt][t];
     }
     __syncthreads();
     if (kg == 1) return;
 #pragma unroll
     for (int mt = 0; mt < kMT; ++mt)
 #pragma unroll
-      for (int t = 0; t < kNT; ++t) acc[mt][t] += park[(mt * kNT + t) * 64 + lane];
+      for (int t = 0; t < CT; ++t) acc[mt][t] += park[(mt * CT + t) * 64 + lane];
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): all of them read before the transposes overwrite the stage
     epi = reinterpret_cast<float*>(park);
   }
@@ -352,12 +356,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
   float cf[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // bf16 scales: 2^E of this lane's eight columns
   if constexpr (kBF16) {
     const int col = ncol0 + (lane & 7) * 8;
-    if (col + 8 <= p.N) column_factors(p.sz, p.G, col, cf);
+    if (col + 8 <= p.N && (lane & 7) * 8 < 16 * CT) column_factors(p.sz, p.G, col, cf);
   }
 #pragma unroll
   for (int mt = 0; mt < kMT; ++mt) {
 #pragma unroll
-    for (int t = 0; t < kNT; ++t)
+    for (int t = 0; t < CT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) epi[(4 * j + i) * kEpiStride + 16 * t + c] = acc[mt][t][i];
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       float vals[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) vals[q] = src[q] * rs * cf[q];
-      epi_store_row8_wave<T>(p.epi, out, vals, row, col, p.N, row < p.M && col + 8 <= p.N, row < p.M, lane);
+      epi_store_row8_wave<T>(p.epi, out, vals, row, col, p.N, row < p.M && col + 8 <= p.N && cc < 16 * CT, row < p.M, lane);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
@@ -620,7 +624,7 @@ __global__ __launch_bounds__(256) void w4a16_splitk_reduce_kernel(const float* _
 }
 
 template <typename T>
-void launch_typed(const PrefillArgs& a, int gpt, int nw, int kg, dim3 grid, dim3 block, hipStream_t s) {
+void launch_typed(const PrefillArgs& a, int gpt, int nw, int kg, int ct, dim3 grid, dim3 block, hipStream_t s) {
   if (nw <= 0) {  // 64-row tiles; -nw = 16-column tiles per wave
     const int knt = -nw;
     if (gpt == 1) {
@@ -634,15 +638,21 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, int kg, dim3 grid, dim3
     }
     return;
   }
+#define KSQ_PF(GPT, NW, KG)                                                                              \
+  do {                                                                                                   \
+    if (ct == 3) hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 3>), grid, block, 0, s, a);    \
+    else hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 4>), grid, block, 0, s, a);            \
+  } while (0)
   if (nw == 4 && kg == 2) {
-    if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 4, 2>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 4, 2>), grid, block, 0, s, a);
+    if (gpt == 1) KSQ_PF(1, 4, 2);
+    else KSQ_PF(2, 4, 2);
     return;
   }
-  if (gpt == 1 && nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 4>), grid, block, 0, s, a);
-  else if (gpt == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 1, 8>), grid, block, 0, s, a);
-  else if (nw == 4) hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 4>), grid, block, 0, s, a);
-  else hipLaunchKernelGGL((w4a16_prefill_kernel<T, 2, 8>), grid, block, 0, s, a);
+  if (gpt == 1 && nw == 4) KSQ_PF(1, 4, 1);
+  else if (gpt == 1) KSQ_PF(1, 8, 1);
+  else if (nw == 4) KSQ_PF(2, 4, 1);
+  else KSQ_PF(2, 8, 1);
+#undef KSQ_PF
 }
 
 }  // namespace
@@ -674,6 +684,7 @@ size_t w4a16_prefill_workspace_bytes(int dtype, size_t m, size_t k) {
 PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes) {
   PrefillPlan p{};
   p.kg = 1;
+  p.ct = 4;
   const size_t ntiles = n / kTileN, kt = k / kTileK, mb128 = (m + 127) / 128;
   // Row tile of the workgroup and, for 128 rows, the waves per workgroup, by a cost model of how the tiles fall on the
   // compute units, in units of the time two 128 x 256 workgroups take side by side on one CU: workgroups run in
@@ -688,8 +699,29 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     return 2.0 * tile * (double)full + (rem == 0 ? 0.0 : rem <= (size_t)cus ? 1.1 * tile : 2.0 * tile);
   };
   // (a grid of at most one 128 x 256 workgroup per CU runs as two k groups of four waves: the price of a full tile)
-  const double cost128w4 = (mb128 * nb16 <= (size_t)cus && kt >= 4) ? 1.0 : rounds_of_two(mb128 * nb16, 1.0);
-  const double cost128w8 = 1.85 * (double)((mb128 * nb32 + (size_t)cus - 1) / (size_t)cus);
+  // Three column tiles per wave instead of four (tiles of 192 / 384 columns): a tile costs 0.88 of the wider one
+  // (the activation stage and the barrier per k tile stay), so it pays where its grid still runs in one round --
+  // which the narrower tiles often fill better -- or saves a round.  Measured at the Llama-2-7B shapes, fp16: qkv
+  // M = 512 60.8 -> 52.5 us (192 workgroups of 128 x 256 -> 256 of 128 x 192), M = 1024 118.9 -> 103.9 (192 of
+  // 128 x 512 -> 256 of 128 x 384); gate_up M = 256 60.5 -> 51.3, M = 512 107.1 -> 90.8; at M >= 2048 the wider
+  // tiles win everywhere (4 to 13 %).
+  double cost128w4 = 0, cost128w8 = 0;
+  int ct_w4 = 4, ct_w8 = 4;
+  for (int ct = 4; ct >= 3; --ct) {
+    const double f = ct == 4 ? 1.0 : 0.88;
+    const size_t nbw4 = (ntiles + 4 * ct - 1) / (4 * ct), nbw8 = (ntiles + 8 * ct - 1) / (8 * ct);
+    const double c4 = (mb128 * nbw4 <= (size_t)cus && kt >= 4) ? f : rounds_of_two(mb128 * nbw4, f);
+    const double c8 = 1.85 * f * (double)((mb128 * nbw8 + (size_t)cus - 1) / (size_t)cus);
+    if (ct == 4 || c4 < 0.99 * cost128w4) {
+      cost128w4 = c4;
+      ct_w4 = ct;
+    }
+    if (ct == 4 || c8 < 0.99 * cost128w8) {
+      cost128w8 = c8;
+      ct_w8 = ct;
+    }
+  }
+  (void)nb32;
   const double cost64 = rounds_of_two(mb64 * nb16, 0.62);
   // a K that the 64-row kernel would split (64 k tiles or more, fewer workgroups than CUs) stays with it
   const bool long_k_few_tiles = kt >= 64 && mb64 * nb16 < (size_t)cus;
@@ -742,15 +774,24 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     p.partial_bytes = need(ks);
   } else {
     p.nw = cost128w8 < cost128w4 ? 8 : 4;
+    p.ct = p.nw == 8 ? ct_w8 : ct_w4;
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 4 || v == 8) {
+        p.nw = v;
+        p.ct = v == 8 ? ct_w8 : ct_w4;
+      }
+    }
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_CT")) {  // tuning / test override
+      const int v = atoi(e);
+      if (v == 3 || v == 4) p.ct = v;
+    }
     // one workgroup per CU at most: two k groups of four waves each
-    p.kg = (p.nw == 4 && mb128 * nb16 <= (size_t)cus && kt >= 4) ? 2 : 1;
+    const size_t nbw = (ntiles + (size_t)(4 * p.ct) - 1) / (size_t)(4 * p.ct);
+    p.kg = (p.nw == 4 && mb128 * nbw <= (size_t)cus && kt >= 4) ? 2 : 1;
     if (const char* e = tuning_env("KSQ_W4_PREFILL_KG")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 1 || (v == 2 && kt >= 2)) p.kg = v;
-    }
-    if (const char* e = tuning_env("KSQ_W4_PREFILL_WAVES")) {  // tuning / test override
-      const int v = atoi(e);
-      if (v == 4 || v == 8) p.nw = v;
     }
     if (p.nw == 8) p.kg = 1;
   }
@@ -795,7 +836,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   } else {
     a.mblocks = (int)((m + kBM - 1) / kBM);
     nw = plan.nw;
-    const int bnt = nw * kNT;
+    const int bnt = nw * plan.ct;
     a.nblocks = (a.ntiles + bnt - 1) / bnt;
     KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
     grid = dim3(tile_grid(a.mblocks, a.nblocks));
@@ -806,10 +847,10 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   if (plan.rows == 64)
     note_launch("w4a16_mid_kernel<gpt=%d,knt=%d> grid=(%u,%u)", gpt, plan.knt, grid.x, grid.y);
   else
-    note_launch("w4a16_prefill_kernel<gpt=%d,nw=%d,kg=%d> grid=(%u)", gpt, plan.nw, plan.kg, grid.x);
+    note_launch("w4a16_prefill_kernel<gpt=%d,nw=%d,kg=%d,ct=%d> grid=(%u)", gpt, plan.nw, plan.kg, plan.ct, grid.x);
   if (plan.ksplit > 1) note_launch("w4a16_splitk_reduce_kernel");
   if (dtype == KSQ_F16) {
-    launch_typed<_Float16>(a, gpt, nw, plan.kg, grid, block, s);
+    launch_typed<_Float16>(a, gpt, nw, plan.kg, plan.ct, grid, block, s);
   } else {
     uint16_t* a16 = static_cast<uint16_t*>(workspace);
     float* row_scale = reinterpret_cast<float*>(static_cast<char*>(workspace) + (m * k * 2 + 255) / 256 * 256);
@@ -823,7 +864,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     else hipLaunchKernelGGL(bf16_rows_to_f16_long_kernel, rows, lanes, 0, s, a_in, a16, row_scale, (int)k);
     a.act = a16;
     a.row_scale = row_scale;
-    launch_typed<__bf16>(a, gpt, nw, plan.kg, grid, block, s);
+    launch_typed<__bf16>(a, gpt, nw, plan.kg, plan.ct, grid, block, s);
   }
   if (plan.ksplit > 1) {  // add the splits up and store
     const size_t stride = (size_t)a.mblocks * 64 * n;

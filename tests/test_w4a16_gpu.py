@@ -137,18 +137,19 @@ def test_forced_split_k_and_tile_widths(gpu, dtype, M, ksplit, nt, slices):
     assert np.array_equal(got1, got2), "split-K result must be deterministic and repeatable"
 
 
-@pytest.mark.parametrize("waves", [4, 8])
+@pytest.mark.parametrize("waves,ct", [(4, 4), (8, 4), (4, 3), (8, 3)])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "awq", 128, 128, 384, 528),    # odd number of k tiles, 33 column tiles: ragged in N for both widths
     ("bf16", "awq", 128, 333, 512, 1040),  # ragged rows, three column blocks of 512
     ("f16", "gptq", 64, 257, 256, 272),    # two groups per k tile
     ("bf16", "gptq", 64, 130, 640, 512),
 ])
-def test_prefill_kernel_widths(gpu, waves, dtype, kind, g, M, K, N):
-    """The large-M kernel in both workgroup widths (128 x 256 and 128 x 512), whichever the planner would pick."""
+def test_prefill_kernel_widths(gpu, waves, ct, dtype, kind, g, M, K, N):
+    """The large-M kernel in its four workgroup widths (four or eight waves side by side, four or three column tiles
+    per wave: 128 x 256, 512, 192, 384), whichever the planner would pick."""
     case = W4Case(1250 + waves + M, M, K, N, g=g, kind=kind, dtype=dtype)
     dev = W4Device(case, gpu)
-    with _env(KSQ_W4_PREFILL_WAVES=waves):
+    with _env(KSQ_W4_PREFILL_ROWS=128, KSQ_W4_PREFILL_WAVES=waves, KSQ_W4_PREFILL_CT=ct):
         got1 = dev.gemm_f32()
         got2 = dev.gemm_f32()
     orc.assert_parity(got1, case.oracle(), f"prefill waves={waves} {dtype} {kind} g={g} M={M}")
@@ -191,20 +192,20 @@ def test_prefill_row_tiles(gpu, rows, nt, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
-@pytest.mark.parametrize("kg", [1, 2])
+@pytest.mark.parametrize("kg,ct", [(1, 4), (2, 4), (2, 3)])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "awq", 128, 65, 640, 528),      # five k tiles: the second k group's last step has no tile
     ("bf16", "awq", 128, 200, 1024, 272),   # eight k tiles, two row blocks, ragged rows and columns
     ("f16", "gptq", 64, 130, 384, 512),     # three k tiles, two groups per tile
     ("bf16", "gptq", 64, 300, 256, 256),    # two k tiles: one step per k group
 ])
-def test_prefill_128_rows_k_groups(gpu, kg, dtype, kind, g, M, K, N):
+def test_prefill_128_rows_k_groups(gpu, kg, ct, dtype, kind, g, M, K, N):
     """The 128-row kernel with four waves side by side, as one group or as two groups that take the even and the odd
     k tiles and add their accumulators through LDS at the end (what the planner picks for grids of at most one
     workgroup per compute unit); twice, bit for bit."""
     case = W4Case(1270 + kg + M, M, K, N, g=g, kind=kind, dtype=dtype)
     dev = W4Device(case, gpu)
-    with _env(KSQ_W4_PREFILL_ROWS=128, KSQ_W4_PREFILL_WAVES=4, KSQ_W4_PREFILL_KG=kg):
+    with _env(KSQ_W4_PREFILL_ROWS=128, KSQ_W4_PREFILL_WAVES=4, KSQ_W4_PREFILL_KG=kg, KSQ_W4_PREFILL_CT=ct):
         got1 = dev.gemm_f32()
         got2 = dev.gemm_f32()
     orc.assert_parity(got1, case.oracle(), f"prefill 128 rows kg={kg} {dtype} {kind} g={g} M={M}")
