@@ -372,6 +372,168 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
   }
 }
 
+// The same decomposition for a K too long for one pass at one to eight rows (more stages than the waves hold as
+// activation fragments): the workgroup walks K in phases of 16 x TPW stages instead of sharing it with other workgroups
+// through partial tiles in memory.  Every wave keeps one fp32 tile per column tile of the workgroup across the phases,
+// swaps in the activation fragments of its next TPW stages (requested a phase ahead, as loaded) and streams the weight
+// rows through the same ring; one reduction over the 16 waves at the end.  No workspace, no counters.
+// AR as above: 4 (at most four rows, one load instruction per phase) or 16.
+template <typename T, int NB, int AR>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void fp8_kphase_kernel(Fp8KstatArgs p) {
+  constexpr int NW = 16, TPW = 2, D = NB * TPW, KP = NW * TPW;
+  static_assert(AR == 4 || AR == 16, "activation rows per load instruction");
+  __shared__ f32x4 red[NB * NW * 64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, j = lane >> 4;
+  const int nt_begin = blockIdx.x * NB;
+  int count = p.ntiles - nt_begin;
+  count = count < NB ? count : NB;
+  const int nphases = (p.KS + KP - 1) / KP;
+  const int s0 = wave * TPW;  // first stage of this wave in phase 0; phase ph adds ph * KP
+
+  int rows = count * 16;
+  if (nt_begin * 16 + rows > p.N) rows = p.N - nt_begin * 16;
+  if (rows < 0) rows = 0;
+  const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(p.wq) + (size_t)nt_begin * 16 * p.K, 0, (int)((size_t)rows * p.K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rs_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.aq), 0, (int)((size_t)p.M * p.K), 0x00020000);
+  const int lr = lane >> 2, lp = lane & 3;
+  const unsigned w_stride = 16u * (unsigned)p.K;
+  // this lane's 16 bytes of (stage s0 + ph * KP + t, half h) inside a row, or out of range (stage past K, piece past K)
+  auto k_byte = [&](int ph, int t, int h) {
+    const int st = s0 + ph * KP + t;
+    const unsigned kb = (unsigned)st * 128u + 64u * h + 16u * lp;
+    return (st < p.KS && kb + 16u <= (unsigned)p.K) ? kb : 0x80000000u;
+  };
+
+  u32x4 wq[D][2];
+  auto fetch = [&](int slot, int i, int t, int ph) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const unsigned kb = k_byte(ph, t, h);
+      const unsigned off = kb != 0x80000000u ? kb + (unsigned)lr * p.K + i * w_stride : 0x80000000u;
+      wq[slot][h] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w, off, 0, 2));
+    }
+  };
+  // the next phase's activations as loaded.  AR = 16: araw[2 t + h], lane l on row l / 4, piece l % 4 of the half
+  // stage; AR = 4: araw[0], lane l on row l / 4 % 4 of half stage l / 16
+  u32x4 araw[AR == 4 ? 1 : 2 * TPW];
+  auto load_a = [&](int ph) {
+    if constexpr (AR == 4) {
+      const int hs = lane >> 4, row = (lane >> 2) & 3;
+      const unsigned kb = k_byte(ph, hs >> 1, hs & 1);
+      const bool ok = kb != 0x80000000u && row < p.M;
+      araw[0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ok ? (unsigned)row * p.K + kb : 0x80000000u, 0, 0));
+    } else {
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const unsigned kb = k_byte(ph, t, h);
+          const bool ok = kb != 0x80000000u && lr < p.M;
+          araw[2 * t + h] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_a, ok ? (unsigned)lr * p.K + kb : 0x80000000u, 0, 0));
+        }
+    }
+  };
+  const int from = (4 * r + j) * 4;
+  auto to_operand = [&](u32x4 lo, u32x4 hi) {
+    i32x8 v;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      v[q] = __builtin_amdgcn_ds_bpermute(from, (int)lo[q]);
+      v[4 + q] = __builtin_amdgcn_ds_bpermute(from, (int)hi[q]);
+    }
+    return v;
+  };
+
+  load_a(0);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int q = 0; q < D; ++q) {
+    fetch(q, q / TPW, q % TPW, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  f32x4 acc[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int ph = 0; ph < nphases; ++ph) {
+    i32x8 af[TPW];
+    if constexpr (AR == 4) {
+      // operand lane 16 j + r takes piece j of row r from lane 16 * hs + 4 r + j of the one load; rows 4 .. 15 are zero
+#pragma unroll
+      for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int src = (16 * (2 * t + h) + 4 * (r & 3) + j) * 4;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int x = __builtin_amdgcn_ds_bpermute(src, (int)araw[0][q]);
+            af[t][4 * h + q] = r < 4 ? x : 0;
+          }
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) af[t] = to_operand(araw[2 * t], araw[2 * t + 1]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    load_a(ph + 1);  // a phase past the end is parked: nothing is read
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int t = 0; t < TPW; ++t) {
+        const int slot = i * TPW + t;
+        const i32x8 bw = to_operand(wq[slot][0], wq[slot][1]);
+        acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(af[t], bw, acc[i], 0, 0, 0, 0, 0, 0);
+        fetch(slot, i, t, ph + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+  }
+
+  // ---- the 16 k slices of every column tile, summed in wave order by wave i of tile i
+#pragma unroll
+  for (int i = 0; i < NB; ++i) red[(i * NW + wave) * 64 + lane] = acc[i];
+  __syncthreads();
+  if (wave < NB) {
+    f32x4 part[NW];
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) part[ww] = red[(wave * NW + ww) * 64 + lane];
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) sum += part[ww];
+    const int col = (nt_begin + wave) * 16 + r, row0 = 4 * j;
+    const float ws = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int row = row0 + e;
+      const float as = p.a_scale[p.a_scale_per_row ? (row < p.M ? row : p.M - 1) : 0];
+      sum[e] = sum[e] * ws * as;
+    }
+    // every lane makes the call (the epilogue may exchange lanes); a column tile past the range stores nothing
+    epi_store_acc<T>(p.epi, static_cast<uint16_t*>(p.out), sum, row0, col, p.M, p.N, wave < count && col < p.N);
+  }
+}
+
+template <typename T>
+bool launch_kphase(int nb, int m, const Fp8KstatArgs& a, dim3 grid, hipStream_t s) {
+#define KSQ_PH(NB)                                                                                    \
+  do {                                                                                                \
+    if (m <= 4) hipLaunchKernelGGL((fp8_kphase_kernel<T, NB, 4>), grid, dim3(1024), 0, s, a);         \
+    else hipLaunchKernelGGL((fp8_kphase_kernel<T, NB, 16>), grid, dim3(1024), 0, s, a);               \
+  } while (0)
+  if (nb == 1) KSQ_PH(1);
+  else if (nb == 2) KSQ_PH(2);
+  else if (nb == 3) KSQ_PH(3);
+  else if (nb == 4) KSQ_PH(4);
+  else return false;
+#undef KSQ_PH
+  return true;
+}
+
 // one row tile and at most four rows: the narrow activation loads
 #define KSQ_GO(MT, TPW, NB, NW)                                                                                   \
   do {                                                                                                            \
@@ -466,6 +628,22 @@ Fp8KstatPlan fp8_kstat_plan(size_t m, size_t n, size_t k, int cus, size_t worksp
     const size_t v = (size_t)atoi(e);
     if (v > ksplit && v <= stages) ksplit = v;
   }
+  // One to eight rows and a K that one pass does not cover: phases inside the workgroup instead of a split across
+  // workgroups, where the column tiles alone give every CU one to four of them (see fp8_kphase_kernel)
+  bool phases = p.mt == 1 && m <= 8 && !fused && ksplit >= 2 && ntiles * 4 >= 3 * (size_t)cus && ntiles <= 4 * (size_t)cus;
+  if (const char* e = tuning_env("KSQ_FP8_KPHASE")) {  // tuning / test switch: 0 = never, 1 = whenever the kernel can
+    phases = atoi(e) != 0 && p.mt == 1 && m <= 8 && !fused && ntiles <= 4 * (size_t)cus && stages >= 2;
+  }
+  if (phases) {
+    p.phases = true;
+    p.ksplit = 1;
+    p.tpw = 2;
+    p.nb = (int)((ntiles + (size_t)cus - 1) / (size_t)cus);
+    p.nt_per_wg = p.nb;
+    p.grid_x = (int)((ntiles + p.nb - 1) / p.nb);
+    p.partial_bytes = 0;
+    return p;
+  }
   if (need(ksplit) > workspace_bytes) {
     p.ok = false;
     return p;
@@ -538,6 +716,15 @@ int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const v
     KSQ_REQUIRE(a.counters != nullptr, KSQ_ERR_HIP, "split-K planned for a stream without arrival counters");
   }
   dim3 grid((unsigned)plan.grid_x, (unsigned)plan.ksplit, 1);
+  if (plan.phases) {
+    KSQ_REQUIRE(act_src == nullptr, KSQ_ERR_UNSUPPORTED, "no fused quantisation in the phase kernel");
+    note_launch("fp8_kphase_kernel<nb=%d,ar=%d> grid=(%d)", plan.nb, m <= 4 ? 4 : 16, plan.grid_x);
+    const bool ok = out_dtype == KSQ_F16 ? launch_kphase<_Float16>(plan.nb, (int)m, a, grid, s)
+                                         : launch_kphase<__bf16>(plan.nb, (int)m, a, grid, s);
+    KSQ_REQUIRE(ok, KSQ_ERR_UNSUPPORTED, "no phase kernel for %d column tiles per workgroup", plan.nb);
+    KSQ_HIP_TRY(hipGetLastError());
+    return KSQ_OK;
+  }
   note_launch("fp8_kstat_kernel<mt=%d,tpw=%d,nb=%d%s> grid=(%d,%d) nt_per_wg=%d", plan.mt, plan.tpw, plan.nb,
               act_src ? ",fused" : "", plan.grid_x, plan.ksplit, plan.nt_per_wg);
   if (act_src != nullptr) {

@@ -263,6 +263,7 @@ struct Fp8KstatPlan {
   int nt_per_wg;  // column tiles per workgroup
   int grid_x;
   int nb;         // column tiles per batch
+  bool phases;    // K walked in phases inside the workgroup (fp8_kphase_kernel) instead of split over grid.y
   size_t partial_bytes;
 };
 // `fused`: plan for the kernel that quantises its own activations (m <= 8)

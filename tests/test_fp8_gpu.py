@@ -291,6 +291,40 @@ def test_gemm_one_row_tile_both_workgroup_shapes(gpu, wide, M, K, N):
     assert np.array_equal(got, got2)
 
 
+@pytest.mark.parametrize("per_channel", [True, False])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 272), (3, 4224, 528), (4, 8320, 264), (5, 2176, 1040), (8, 8208, 272),
+                                   (2, 1008, 4104), (7, 640, 8200), (1, 29568, 272), (6, 4096, 16)])
+def test_gemm_k_phases_inside_the_workgroup(gpu, per_channel, M, K, N):
+    """One to eight rows with K walked in phases inside the workgroup (what a long K gets instead of a split across
+    workgroups): whole and partial last phases, K that is not a multiple of 128, one to four column tiles per
+    workgroup, a ragged last workgroup and a ragged last column tile; no workspace needed; two runs bit for bit."""
+    import os
+
+    from ksanallm_amd import capi
+
+    xq, xs, wq, ws = _fp8_case(470 + M, M, K, N)
+    if not per_channel:
+        xs, ws = xs[:1].copy(), ws[:1].copy()
+    old = os.environ.get("KSQ_FP8_KPHASE")
+    os.environ["KSQ_FP8_KPHASE"] = "1"
+    capi.set_launch_log(True)
+    try:
+        got = _run_gemm(gpu, xq, xs, wq, ws, "bf16", use_workspace=False)
+        assert "fp8_kphase_kernel" in capi.last_launch(), capi.last_launch()
+        got2 = _run_gemm(gpu, xq, xs, wq, ws, "f16")
+        got3 = _run_gemm(gpu, xq, xs, wq, ws, "f16")
+    finally:
+        capi.set_launch_log(False)
+        if old is None:
+            os.environ.pop("KSQ_FP8_KPHASE", None)
+        else:
+            os.environ["KSQ_FP8_KPHASE"] = old
+    want = orc.fp8_gemm(xq, xs, wq, ws)
+    orc.assert_parity(got, want, f"fp8 k phases M={M} K={K} N={N}")
+    orc.assert_parity(got2, want, f"fp8 k phases f16 M={M} K={K} N={N}")
+    assert np.array_equal(got2, got3)
+
+
 @pytest.mark.parametrize("M", [1, 64])
 def test_config4_qwen72b_shape(gpu, M):
     xq, xs, wq, ws = _fp8_case(403, M, 8192, 8192)
