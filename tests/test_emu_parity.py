@@ -58,6 +58,7 @@ test_planner_choices_without_overrides = w4.test_planner_choices_without_overrid
 test_prefill_bf16_row_magnitudes = w4.test_prefill_bf16_row_magnitudes
 test_bf16_scales_far_outside_the_fp16_range = w4.test_bf16_scales_far_outside_the_fp16_range
 test_k_odd_multiple_of_64 = w4.test_k_odd_multiple_of_64
+test_random_shapes = w4.test_random_shapes
 test_no_workspace_still_correct = w4.test_no_workspace_still_correct
 test_caller_bound_split_k_counters_and_launch_log = w4.test_caller_bound_split_k_counters_and_launch_log
 test_k_tiles_per_wave = w4.test_k_tiles_per_wave
@@ -74,6 +75,7 @@ test_gemm_per_tensor_scales_and_ragged_shapes = f8.test_gemm_per_tensor_scales_a
 test_gemm_large_m_ragged = f8.test_gemm_large_m_ragged
 test_gemm_large_m_both_tiles = f8.test_gemm_large_m_both_tiles
 test_gemm_k_phases_inside_the_workgroup = f8.test_gemm_k_phases_inside_the_workgroup
+test_gemm_random_shapes = f8.test_gemm_random_shapes
 test_gemm_large_m_small_integers_exact = f8.test_gemm_large_m_small_integers_exact
 test_gemm_small_integers_exact = f8.test_gemm_small_integers_exact
 test_convert_weight_per_channel = f8.test_convert_weight_per_channel

@@ -325,6 +325,26 @@ def test_gemm_k_phases_inside_the_workgroup(gpu, per_channel, M, K, N):
     assert np.array_equal(got2, got3)
 
 
+@pytest.mark.parametrize("seed", [21, 22, 23, 24])
+def test_gemm_random_shapes(gpu, seed):
+    """Ten shapes per seed from a seeded random walk over every family of M, N from 8 to a few thousand (ragged column
+    tiles included) and K from 16 to 2500 in steps of 16 (the streaming kernel for K % 128 != 0, the decode and tile
+    kernels otherwise), per-token x per-channel and per-tensor scales, with and without a workspace."""
+    rng = np.random.default_rng(seed)
+    for i in range(10):
+        M = int(rng.choice([rng.integers(1, 17), rng.integers(17, 65), rng.integers(65, 300)]))
+        N = 8 * int(rng.choice([rng.integers(1, 17), rng.integers(17, 300)]))
+        K = 16 * int(rng.choice([rng.integers(1, 9), rng.integers(9, 160)])) if rng.integers(0, 2) else 128 * int(rng.integers(1, 20))
+        xq, xs, wq, ws = _fp8_case(4000 + 100 * seed + i, M, K, N)
+        if rng.integers(0, 2):
+            xs, ws = xs[:1].copy(), ws[:1].copy()
+        want = orc.fp8_gemm(xq, xs, wq, ws)
+        got = _run_gemm(gpu, xq, xs, wq, ws, "bf16" if i % 2 else "f16")
+        orc.assert_parity(got, want, f"fp8 random seed {seed} #{i}: M={M} K={K} N={N} scales={len(xs)}x{len(ws)}")
+        got = _run_gemm(gpu, xq, xs, wq, ws, "bf16", use_workspace=False)
+        orc.assert_parity(got, want, f"fp8 random seed {seed} #{i}, no workspace")
+
+
 @pytest.mark.parametrize("M", [1, 64])
 def test_config4_qwen72b_shape(gpu, M):
     xq, xs, wq, ws = _fp8_case(403, M, 8192, 8192)

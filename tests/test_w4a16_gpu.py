@@ -312,6 +312,40 @@ def test_planner_choices_without_overrides(gpu, dtype, kind, g, M, K, N):
         orc.assert_parity(dev.gemm_f32(use_workspace=False), case.oracle(), f"planner, no workspace {dtype} M={M}")
 
 
+def _random_w4_shapes(seed, count):
+    """Shapes of a seeded random walk over what the planners distinguish: every family of M, widths from one column
+    tile to a few thousand columns (ragged last workgroups included), K from one k tile up, both group sizes (K = 64 x
+    odd with g = 64), both layouts and element types."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        M = int(rng.choice([rng.integers(1, 17), rng.integers(17, 33), rng.integers(33, 65), rng.integers(65, 300)]))
+        N = 16 * int(rng.choice([rng.integers(1, 9), rng.integers(9, 140)]))
+        g = int(rng.choice([64, 128]))
+        K = g * int(rng.choice([rng.integers(1, 5), rng.integers(5, 20)]))
+        if K % 128 == 64 and g == 128:
+            K += 64
+        out.append((M, K, N, g, str(rng.choice(["awq", "gptq"])), str(rng.choice(["f16", "bf16"]))))
+    return out
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+def test_random_shapes(gpu, seed):
+    """Twelve shapes per seed from a seeded random walk (and, with the first seed, the shape that used to read past the
+    weights: one k tile under the two-row-tile decode kernel), each through the planner's own choice with a workspace
+    and without one, against the oracle."""
+    shapes = _random_w4_shapes(seed, 12)
+    if seed == 11:
+        shapes += [(24, 128, 272, 128, "awq", "f16"), (32, 128, 16, 64, "gptq", "bf16")]
+    for i, (M, K, N, g, kind, dtype) in enumerate(shapes):
+        case = W4Case(3000 + 100 * seed + i, M, K, N, g=g, kind=kind, dtype=dtype)
+        dev = W4Device(case, gpu)
+        want = case.oracle()
+        orc.assert_parity(dev.gemm_f32(), want, f"random seed {seed} #{i}: M={M} K={K} N={N} g={g} {kind} {dtype}")
+        if K % 128 == 0 and not (dtype == "bf16" and M >= 65):  # K = 64 x odd needs the padded copy in the workspace
+            orc.assert_parity(dev.gemm_f32(use_workspace=False), want, f"random seed {seed} #{i}, no workspace")
+
+
 def test_prefill_bf16_row_magnitudes(gpu):
     """bf16 activations go through a per-row power-of-two re-encoding on the large-M route: rows of very different
     magnitude (up to 2^100, down to 2^-60, an all-zero row) must each keep full relative accuracy."""
