@@ -29,9 +29,14 @@ typedef enum ksq_status {
   KSQ_ERR_HIP = -4               /* a HIP runtime call or kernel launch failed */
 } ksq_status;
 
-/* Activation / output element type (the reference instantiates its layers for half and __nv_bfloat16:
- * KS/layers/nvidia/group_matmul_layer.cpp:171-175, fp8_matmul_layer.cpp:69-73). */
-typedef enum ksq_dtype { KSQ_F16 = 0, KSQ_BF16 = 1 } ksq_dtype;
+/* Activation / output element type (the reference instantiates its layers for float, half and __nv_bfloat16:
+ * KS/layers/nvidia/group_matmul_layer.cpp:171-175, fp8_matmul_layer.cpp:69-73).
+ * KSQ_F32 is accepted by the FP8 entry points that take activations or produce results -- ksq_fp8_quantize,
+ * ksq_fp8_gemm / _ex / _rowmax (out_dtype), ksq_fp8_gemm_dynamic (both) -- which is where the reference has an fp32
+ * path (Fp8E4m3Quantize<float>, Fp8QuantizedMatMul<float>: KS/kernels/nvidia/kernel_wrapper.cpp:1026, 1043); a
+ * bias row is then fp32 too.  The W4A16 entry points take KSQ_F16 and KSQ_BF16: the reference's float instantiation
+ * of that GEMM is empty (LK/asymmetric_gemm/asymmetric_gemm_wrapper.cu:44-85). */
+typedef enum ksq_dtype { KSQ_F16 = 0, KSQ_BF16 = 1, KSQ_F32 = 2 } ksq_dtype;
 
 /* Source layouts the repack step reads. */
 typedef enum ksq_w4_layout {

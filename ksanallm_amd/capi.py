@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libksq.so")
 
 # enums of include/ksq.h
-F16, BF16 = 0, 1
+F16, BF16, F32 = 0, 1, 2  # F32: the FP8 entry points only
 W4_GPTQ_INT32_KPACK, W4_AWQ_INT32_NPACK, W4_ROWMAJOR_INT4_SIGNED = 0, 1, 2
 W4_CUTLASS_SM80_INTERLEAVED, W4_CUTLASS_SM90_COLMAJOR, W4_MARLIN = 3, 4, 5
 COLS_NATURAL, COLS_HALVES_INTERLEAVED = 0, 1

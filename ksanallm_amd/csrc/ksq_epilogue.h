@@ -11,13 +11,28 @@ typedef float epi_f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t epi_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t epi_u32x2 __attribute__((ext_vector_type(2)));
 
+// The element a kernel stores: 16-bit patterns for fp16 / bf16 results, floats for fp32 ones (the FP8 GEMM only: the
+// reference's Fp8MatMulLayer<float> takes an fp32 result from its GEMM, KS/kernels/nvidia/kernel_wrapper.cpp:1043).
 template <typename T>
-__device__ inline uint16_t epi_bits(float v) {
-  return __builtin_bit_cast(uint16_t, (T)v);
+struct EpiElem {
+  typedef uint16_t type;
+};
+template <>
+struct EpiElem<float> {
+  typedef float type;
+};
+template <typename T>
+using epi_elem_t = typename EpiElem<T>::type;
+
+template <typename T>
+__device__ inline epi_elem_t<T> epi_bits(float v) {
+  if constexpr (__is_same(T, float)) return v;
+  else return __builtin_bit_cast(uint16_t, (T)v);
 }
 template <typename T>
-__device__ inline float epi_float(uint16_t b) {
-  return (float)__builtin_bit_cast(T, b);
+__device__ inline float epi_float(epi_elem_t<T> b) {
+  if constexpr (__is_same(T, float)) return b;
+  else return (float)__builtin_bit_cast(T, b);
 }
 
 __device__ inline float epi_silu(float x) { return x / (1.0f + __expf(-x)); }
@@ -26,9 +41,9 @@ __device__ inline float epi_silu(float x) { return x / (1.0f + __expf(-x)); }
 // same rows.  Every lane of the wave must make the call (it contains a cross-lane exchange); `ok` says whether this
 // lane's column exists, rows are clipped against M.  N is the width of the GEMM (of the weight).
 template <typename T>
-__device__ inline void epi_store_acc(const Epilogue& ep, uint16_t* out, epi_f32x4 v, int row0, int col, int M, int N,
+__device__ inline void epi_store_acc(const Epilogue& ep, epi_elem_t<T>* out, epi_f32x4 v, int row0, int col, int M, int N,
                                      bool ok) {
-  uint16_t bits[4];
+  epi_elem_t<T> bits[4];
   bool mine = ok;
   size_t width = (size_t)N;
   int ocol = col;
@@ -46,7 +61,7 @@ __device__ inline void epi_store_acc(const Epilogue& ep, uint16_t* out, epi_f32x
     ocol = col >> 1;
   } else {
     float b = 0.f;
-    if (ep.kind == KSQ_EPILOGUE_BIAS && ok) b = epi_float<T>(static_cast<const uint16_t*>(ep.bias)[col]);
+    if (ep.kind == KSQ_EPILOGUE_BIAS && ok) b = epi_float<T>(static_cast<const epi_elem_t<T>*>(ep.bias)[col]);
 #pragma unroll
     for (int e = 0; e < 4; ++e) bits[e] = epi_bits<T>(v[e] + b);
   }
@@ -74,9 +89,37 @@ __device__ inline void epi_store_acc(const Epilogue& ep, uint16_t* out, epi_f32x
 // Row segment: src[0..7] = results at (row, col .. col + 7), col a multiple of 8 and col + 8 <= N, row < M.  Returns the
 // largest |stored value| of the segment.
 template <typename T>
-__device__ inline float epi_store_row8(const Epilogue& ep, uint16_t* out, const float (&src)[8], int row, int col,
+__device__ inline float epi_store_row8(const Epilogue& ep, epi_elem_t<T>* out, const float (&src)[8], int row, int col,
                                        int N) {
   float mx = 0.f;
+  if constexpr (__is_same(T, float)) {  // 32-bit results: sixteen or thirty-two bytes per segment
+    if (ep.kind == KSQ_EPILOGUE_SILU_MUL) {
+      epi_f32x4 r;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        r[q] = epi_silu(src[2 * q]) * src[2 * q + 1];
+        mx = __builtin_fmaxf(mx, __builtin_fabsf(r[q]));
+      }
+      *reinterpret_cast<epi_f32x4*>(out + (size_t)row * (size_t)(N >> 1) + (col >> 1)) = r;
+      return mx;
+    }
+    epi_f32x4 lo, hi;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float b0 = 0.f, b1 = 0.f;
+      if (ep.kind == KSQ_EPILOGUE_BIAS) {
+        b0 = static_cast<const float*>(ep.bias)[col + q];
+        b1 = static_cast<const float*>(ep.bias)[col + 4 + q];
+      }
+      lo[q] = src[q] + b0;
+      hi[q] = src[4 + q] + b1;
+      mx = __builtin_fmaxf(mx, __builtin_fmaxf(__builtin_fabsf(lo[q]), __builtin_fabsf(hi[q])));
+    }
+    epi_f32x4* dst = reinterpret_cast<epi_f32x4*>(out + (size_t)row * N + col);
+    dst[0] = lo;
+    dst[1] = hi;
+    return mx;
+  } else {
   if (ep.kind == KSQ_EPILOGUE_SILU_MUL) {
     epi_u32x2 packed;
 #pragma unroll
@@ -107,13 +150,14 @@ __device__ inline float epi_store_row8(const Epilogue& ep, uint16_t* out, const 
   }
   *reinterpret_cast<epi_u32x4*>(out + (size_t)row * N + col) = packed;
   return mx;
+  }
 }
 
 // The tile kernels' form: every lane of the wave makes the call, `live` says whether this lane has a segment to store;
 // the eight lanes lane & ~7 .. hold the same row (when `row_ok`), so with ep.row_absmax set they agree on the row's
 // maximum over their 64 columns before one of them merges it.
 template <typename T>
-__device__ inline void epi_store_row8_wave(const Epilogue& ep, uint16_t* out, const float (&src)[8], int row, int col,
+__device__ inline void epi_store_row8_wave(const Epilogue& ep, epi_elem_t<T>* out, const float (&src)[8], int row, int col,
                                            int N, bool live, bool row_ok, int lane) {
   float mx = 0.f;
   if (live) mx = epi_store_row8<T>(ep, out, src, row, col, N);

@@ -17,6 +17,9 @@ using fp8ops::absmax8;
 using fp8ops::quantize8;
 using fp8ops::unpack8;
 
+// element i of a tensor of T, as float.  The pointer is the tensor's base as the entry points take it (16-bit patterns
+// for fp16 / bf16; for fp32 activations -- the reference's Fp8E4m3Quantize<float>, KS/kernels/nvidia/kernel_wrapper.cpp:1026
+// -- the same pointer is a float array, and only the element-wise kernels below serve it)
 template <typename T>
 __device__ inline float load_as_float(const uint16_t* p, size_t i);
 template <>
@@ -26,6 +29,10 @@ __device__ inline float load_as_float<_Float16>(const uint16_t* p, size_t i) {
 template <>
 __device__ inline float load_as_float<__bf16>(const uint16_t* p, size_t i) {
   return __builtin_bit_cast(float, (uint32_t)p[i] << 16);
+}
+template <>
+__device__ inline float load_as_float<float>(const uint16_t* p, size_t i) {
+  return reinterpret_cast<const float*>(p)[i];
 }
 
 template <typename T>
@@ -84,10 +91,9 @@ __global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* x, const 
                                                        size_t channel_size, uint8_t* q) {
   const size_t ch = blockIdx.y;
   const float s = scale[ch];
-  const uint16_t* xr = x + ch * channel_size;
   uint8_t* qr = q + ch * channel_size;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < channel_size; i += (size_t)gridDim.x * 256)
-    qr[i] = quantize_one(load_as_float<T>(xr, i), s);
+    qr[i] = quantize_one(load_as_float<T>(x, ch * channel_size + i), s);
 }
 
 // per-token with the rows' maxima known (merged in by the GEMM that produced x): the scale, then one pass over the row.
@@ -107,7 +113,7 @@ __global__ __launch_bounds__(256) void quantize_rows_from_absmax_kernel(const ui
       qv[i] = fp8ops::quantize8(f, s);
     }
   } else {
-    for (size_t i = threadIdx.x; i < k; i += 256) q[row * k + i] = quantize_one(load_as_float<T>(x + row * k, i), s);
+    for (size_t i = threadIdx.x; i < k; i += 256) q[row * k + i] = quantize_one(load_as_float<T>(x, row * k + i), s);
   }
 }
 
@@ -117,14 +123,13 @@ __global__ __launch_bounds__(256) void quantize_per_token_kernel(const uint16_t*
                                                                  float* scale) {
   __shared__ float smem[4];
   const size_t row = blockIdx.x;
-  const uint16_t* xr = x + row * k;
   uint8_t* qr = q + row * k;
   float mx = 0.0f;
-  for (size_t i = threadIdx.x; i < k; i += 256) mx = fmaxf(mx, fabsf(load_as_float<T>(xr, i)));
+  for (size_t i = threadIdx.x; i < k; i += 256) mx = fmaxf(mx, fabsf(load_as_float<T>(x, row * k + i)));
   mx = block_max_256(mx, smem);
   const float s = fmaxf(mx / kE4m3Max, kMinScale);
   if (threadIdx.x == 0) scale[row] = s;
-  for (size_t i = threadIdx.x; i < k; i += 256) qr[i] = quantize_one(load_as_float<T>(xr, i), s);
+  for (size_t i = threadIdx.x; i < k; i += 256) qr[i] = quantize_one(load_as_float<T>(x, row * k + i), s);
 }
 
 // ---- vector forms (k a multiple of 8, 16-byte aligned rows): eight elements per lane and access; unpack8, absmax8 and
@@ -379,7 +384,7 @@ __global__ __launch_bounds__(256) void fp8_stream_kernel(Fp8Args p) {
     }
   }
 
-  uint16_t* out = static_cast<uint16_t*>(p.out);
+  epi_elem_t<T>* out = static_cast<epi_elem_t<T>*>(p.out);
   const int col = nt * 16 + c;
   const float ws = p.w_scale[p.w_scale_per_col ? (col < p.N ? col : p.N - 1) : 0];
   auto store_out = [&](int mt, f32x4 v) {
@@ -439,7 +444,7 @@ extern "C" {
 
 int ksq_fp8_quantize(int dtype, const void* act, size_t m, size_t k, int mode, void* act_q, float* act_scale,
                      void* stream) {
-  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16 || dtype == KSQ_F32, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
   KSQ_REQUIRE(mode >= KSQ_FP8_PER_TENSOR_DYNAMIC && mode <= KSQ_FP8_PER_TOKEN_DYNAMIC, KSQ_ERR_INVALID_ARGUMENT,
               "bad quantisation mode %d", mode);
   KSQ_REQUIRE(act && act_q && act_scale, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
@@ -448,6 +453,22 @@ int ksq_fp8_quantize(int dtype, const void* act, size_t m, size_t k, int mode, v
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uint16_t* x = static_cast<const uint16_t*>(act);
   uint8_t* q = static_cast<uint8_t*>(act_q);
+  if (dtype == KSQ_F32) {  // fp32 activations: the element-wise kernels (the vector forms read 16-bit elements)
+    if (mode == KSQ_FP8_PER_TOKEN_DYNAMIC) {
+      KSQ_REQUIRE(m < (1ull << 31), KSQ_ERR_UNSUPPORTED, "m too large");
+      hipLaunchKernelGGL(quantize_per_token_kernel<float>, dim3((unsigned)m), dim3(256), 0, s, x, k, q, act_scale);
+    } else {
+      const size_t count = m * k;
+      if (mode == KSQ_FP8_PER_TENSOR_DYNAMIC) {
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, act_scale, 1);
+        hipLaunchKernelGGL(absmax_scale_kernel<float>, dim3(blocks_for(count, 2048)), dim3(256), 0, s, x, count, act_scale);
+      }
+      hipLaunchKernelGGL(quantize_kernel<float>, dim3(blocks_for(count, 4096), 1), dim3(256), 0, s, x, act_scale, (size_t)1,
+                         count, q);
+    }
+    KSQ_HIP_TRY(hipGetLastError());
+    return KSQ_OK;
+  }
   const bool f16 = dtype == KSQ_F16;
   if (mode == KSQ_FP8_PER_TOKEN_DYNAMIC) {
     KSQ_REQUIRE(m < (1ull << 31), KSQ_ERR_UNSUPPORTED, "m too large");
@@ -634,7 +655,7 @@ int ksq_fp8_gemm_dynamic_workspace_bytes(size_t max_m, size_t n, size_t k, size_
 int ksq_fp8_gemm_dynamic(int dtype, void* out, const void* act, const void* w_q, const float* w_scale,
                          size_t w_scale_count, size_t m, size_t n, size_t k, int epilogue, const void* bias,
                          void* workspace, size_t workspace_bytes, void* stream) {
-  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
+  KSQ_REQUIRE(dtype == KSQ_F16 || dtype == KSQ_BF16 || dtype == KSQ_F32, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", dtype);
   KSQ_REQUIRE(out && act && w_q && w_scale, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
   KSQ_REQUIRE(epilogue >= KSQ_EPILOGUE_NONE && epilogue <= KSQ_EPILOGUE_SILU_MUL, KSQ_ERR_INVALID_ARGUMENT,
               "bad epilogue %d", epilogue);
@@ -663,7 +684,7 @@ int ksq_fp8_gemm_dynamic(int dtype, void* out, const void* act, const void* w_q,
   // 29.9 against 23.6; K = 29568, split four ways: 65.9 against 59.3): it serves m = 1, and up to eight rows on request.
   const char* sw = tuning_env("KSQ_FP8_FUSED_QUANT");  // tuning / test switch: 0 = never, 1 = up to eight rows
   const size_t fused_rows = sw ? (atoi(sw) == 0 ? 0 : 8) : 1;
-  if (m <= fused_rows && k % 128 == 0 && m * k * 2 < 0x7FFFFF00ull) {
+  if (m <= fused_rows && dtype != KSQ_F32 && k % 128 == 0 && m * k * 2 < 0x7FFFFF00ull) {
     if (gemm_ws && !counter_slot_available(s)) gemm_ws = nullptr, gemm_ws_bytes = 0;
     const Fp8KstatPlan kp = fp8_kstat_plan(m, n, k, di->cus, gemm_ws_bytes, true);
     if (kp.ok && kp.nb <= 2 && kp.tpw <= 4 && (kp.ksplit == 1 || sw)) {
@@ -707,7 +728,8 @@ static int fp8_gemm_impl(int out_dtype, void* out, const void* act_q, const floa
   epi.kind = epilogue;
   epi.bias = bias;
   epi.row_absmax = row_absmax;
-  KSQ_REQUIRE(out_dtype == KSQ_F16 || out_dtype == KSQ_BF16, KSQ_ERR_INVALID_ARGUMENT, "bad dtype %d", out_dtype);
+  KSQ_REQUIRE(out_dtype == KSQ_F16 || out_dtype == KSQ_BF16 || out_dtype == KSQ_F32, KSQ_ERR_INVALID_ARGUMENT,
+              "bad dtype %d", out_dtype);
   KSQ_REQUIRE(out && act_q && w_q, KSQ_ERR_INVALID_ARGUMENT, "null tensor pointer");
   // the reference layer refuses a missing weight scale (KS/layers/nvidia/fp8_matmul_layer.cpp:49-51)
   KSQ_REQUIRE(w_scale != nullptr, KSQ_ERR_INVALID_ARGUMENT, "weight scale is null");
@@ -767,6 +789,7 @@ static int fp8_gemm_impl(int out_dtype, void* out, const void* act_q, const floa
   hipStream_t s = static_cast<hipStream_t>(stream);
   note_launch("fp8_stream_kernel<mt=%d> grid=(%u,%u,%u)", plan.MT, grid.x, grid.y, grid.z);
   if (out_dtype == KSQ_F16) launch_fp8_stream<_Float16>(plan.MT, a, grid, s);
+  else if (out_dtype == KSQ_F32) launch_fp8_stream<float>(plan.MT, a, grid, s);
   else launch_fp8_stream<__bf16>(plan.MT, a, grid, s);
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;

@@ -294,7 +294,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4)
     }
   }
 
-  uint16_t* out = static_cast<uint16_t*>(p.out);
+  epi_elem_t<T>* out = static_cast<epi_elem_t<T>*>(p.out);
   for (int b = 0; b < nbatches; ++b) {
     f32x4 accb[NB][MT];
 #pragma unroll
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4))) void 
       sum[e] = sum[e] * ws * as;
     }
     // every lane makes the call (the epilogue may exchange lanes); a column tile past the range stores nothing
-    epi_store_acc<T>(p.epi, static_cast<uint16_t*>(p.out), sum, row0, col, p.M, p.N, wave < count && col < p.N);
+    epi_store_acc<T>(p.epi, static_cast<epi_elem_t<T>*>(p.out), sum, row0, col, p.M, p.N, wave < count && col < p.N);
   }
 }
 
@@ -719,8 +719,9 @@ int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const v
   if (plan.phases) {
     KSQ_REQUIRE(act_src == nullptr, KSQ_ERR_UNSUPPORTED, "no fused quantisation in the phase kernel");
     note_launch("fp8_kphase_kernel<nb=%d,ar=%d> grid=(%d)", plan.nb, m <= 4 ? 4 : 16, plan.grid_x);
-    const bool ok = out_dtype == KSQ_F16 ? launch_kphase<_Float16>(plan.nb, (int)m, a, grid, s)
-                                         : launch_kphase<__bf16>(plan.nb, (int)m, a, grid, s);
+    const bool ok = out_dtype == KSQ_F16   ? launch_kphase<_Float16>(plan.nb, (int)m, a, grid, s)
+                    : out_dtype == KSQ_F32 ? launch_kphase<float>(plan.nb, (int)m, a, grid, s)
+                                           : launch_kphase<__bf16>(plan.nb, (int)m, a, grid, s);
     KSQ_REQUIRE(ok, KSQ_ERR_UNSUPPORTED, "no phase kernel for %d column tiles per workgroup", plan.nb);
     KSQ_HIP_TRY(hipGetLastError());
     return KSQ_OK;
@@ -728,12 +729,15 @@ int fp8_launch_kstat(int out_dtype, const Fp8KstatPlan& plan, void* out, const v
   note_launch("fp8_kstat_kernel<mt=%d,tpw=%d,nb=%d%s> grid=(%d,%d) nt_per_wg=%d", plan.mt, plan.tpw, plan.nb,
               act_src ? ",fused" : "", plan.grid_x, plan.ksplit, plan.nt_per_wg);
   if (act_src != nullptr) {
+    KSQ_REQUIRE(out_dtype != KSQ_F32, KSQ_ERR_UNSUPPORTED, "the kernel that quantises its own activations reads 16-bit ones");
     const bool ok = out_dtype == KSQ_F16 ? launch_fused<_Float16>(plan.tpw, plan.nb, a, grid, s)
                                          : launch_fused<__bf16>(plan.tpw, plan.nb, a, grid, s);
     KSQ_REQUIRE(ok, KSQ_ERR_UNSUPPORTED, "no fused kernel for %d stages per wave, %d column tiles per batch", plan.tpw,
                 plan.nb);
   } else if (out_dtype == KSQ_F16) {
     launch<_Float16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
+  } else if (out_dtype == KSQ_F32) {
+    launch<float>(plan.mt, plan.tpw, plan.nb, a, grid, s);
   } else {
     launch<__bf16>(plan.mt, plan.tpw, plan.nb, a, grid, s);
   }

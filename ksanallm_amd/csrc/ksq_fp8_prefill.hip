@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetches must not land on top of the transposes
   __syncthreads();
   float* epi = reinterpret_cast<float*>(wave == 0 ? lds0 : wave == 1 ? lds1 : wave == 2 ? lds2 : lds3);
-  uint16_t* out = static_cast<uint16_t*>(p.out);
+  epi_elem_t<T>* out = static_cast<epi_elem_t<T>*>(p.out);
   float ws[kNT];
 #pragma unroll
   for (int t = 0; t < kNT; ++t) {
@@ -442,7 +442,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void f
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the last (unused) prefetch must not land on top of the transposes
   __syncthreads();
   float* epi = reinterpret_cast<float*>(wave < 4 ? lds_a0 : lds_a1) + (wave & 3) * (16 * kEpiStride);
-  uint16_t* out = static_cast<uint16_t*>(p.out);
+  epi_elem_t<T>* out = static_cast<epi_elem_t<T>*>(p.out);
   const int mw = m0 + 16 * kMTW * wm, nw = n0 + 64 * wn;
   float ws[kNT];
 #pragma unroll
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(256) void fp8_tail_reduce_kernel(Fp8PrefillArgs p) 
     const float w = p.w_scale[p.w_scale_per_col ? col + q : 0];
     vals[q] = ((q < 4 ? lo[q] : hi[q - 4]) * w) * as;  // the order of the one-launch epilogue: column scale, then row scale
   }
-  const float mx = epi_store_row8<T>(p.epi, static_cast<uint16_t*>(p.out), vals, row, col, p.N);
+  const float mx = epi_store_row8<T>(p.epi, static_cast<epi_elem_t<T>*>(p.out), vals, row, col, p.N);
   if (p.epi.row_absmax) atomicMax(reinterpret_cast<unsigned*>(p.epi.row_absmax) + row, __builtin_bit_cast(unsigned, mx));
 }
 
@@ -637,12 +637,16 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     if (main_tiles) note_launch("fp8_prefill256_kernel grid=(%zu)", main_tiles);
     if (quarters) note_launch("fp8_prefill256_kernel<quarters> tiles=%d", tail_tiles);
     else if (ks > 1) note_launch("fp8_prefill256_kernel<ksplit=%d> tiles=%d + fp8_tail_reduce_kernel", ks, tail_tiles);
+#define KSQ_BY_TYPE(KERNEL, GRID, BLOCK, ARGS)                                                  \
+  do {                                                                                        \
+    if (out_dtype == KSQ_F16) hipLaunchKernelGGL((KERNEL<_Float16>), GRID, BLOCK, 0, s, ARGS); \
+    else if (out_dtype == KSQ_F32) hipLaunchKernelGGL((KERNEL<float>), GRID, BLOCK, 0, s, ARGS); \
+    else hipLaunchKernelGGL((KERNEL<__bf16>), GRID, BLOCK, 0, s, ARGS);                        \
+  } while (0)
     if (main_tiles == 0) {
       // every tile is in the split launch
-    } else if (out_dtype == KSQ_F16) {
-      hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
     } else {
-      hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, dim3((unsigned)main_tiles), dim3(512), 0, s, a);
+      KSQ_BY_TYPE(fp8_prefill256_kernel, dim3((unsigned)main_tiles), dim3(512), a);
     }
     if (quarters) {
       Fp8PrefillArgs t = a;
@@ -650,6 +654,8 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
       const dim3 qgrid((unsigned)((4 * (size_t)tail_tiles + 7) / 8 * 8));
       if (out_dtype == KSQ_F16)
         hipLaunchKernelGGL((fp8_prefill256_kernel<_Float16, 1>), qgrid, dim3(512), 0, s, t);
+      else if (out_dtype == KSQ_F32)
+        hipLaunchKernelGGL((fp8_prefill256_kernel<float, 1>), qgrid, dim3(512), 0, s, t);
       else
         hipLaunchKernelGGL((fp8_prefill256_kernel<__bf16, 1>), qgrid, dim3(512), 0, s, t);
     } else if (ks > 1) {
@@ -659,13 +665,8 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
       t.tail_tiles = tail_tiles;
       t.partial = static_cast<float*>(workspace);
       const dim3 tgrid((unsigned)((tail_tiles + 7) / 8 * 8), (unsigned)ks), rgrid((unsigned)((size_t)tail_tiles * 8192 / 256));
-      if (out_dtype == KSQ_F16) {
-        hipLaunchKernelGGL(fp8_prefill256_kernel<_Float16>, tgrid, dim3(512), 0, s, t);
-        hipLaunchKernelGGL(fp8_tail_reduce_kernel<_Float16>, rgrid, dim3(256), 0, s, t);
-      } else {
-        hipLaunchKernelGGL(fp8_prefill256_kernel<__bf16>, tgrid, dim3(512), 0, s, t);
-        hipLaunchKernelGGL(fp8_tail_reduce_kernel<__bf16>, rgrid, dim3(256), 0, s, t);
-      }
+      KSQ_BY_TYPE(fp8_prefill256_kernel, tgrid, dim3(512), t);
+      KSQ_BY_TYPE(fp8_tail_reduce_kernel, rgrid, dim3(256), t);
     }
   } else {
     a.mblocks = (int)((m + kBM - 1) / kBM);
@@ -673,11 +674,9 @@ int fp8_launch_prefill(int out_dtype, void* out, const void* act_q, const float*
     KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
     const dim3 grid(tile_grid(a.mblocks, a.nblocks));
     note_launch("fp8_prefill_kernel grid=(%u)", grid.x);
-    if (out_dtype == KSQ_F16)
-      hipLaunchKernelGGL(fp8_prefill_kernel<_Float16>, grid, dim3(256), 0, s, a);
-    else
-      hipLaunchKernelGGL(fp8_prefill_kernel<__bf16>, grid, dim3(256), 0, s, a);
+    KSQ_BY_TYPE(fp8_prefill_kernel, grid, dim3(256), a);
   }
+#undef KSQ_BY_TYPE
   KSQ_HIP_TRY(hipGetLastError());
   return KSQ_OK;
 }

@@ -45,7 +45,7 @@ struct PrefillArgs {
 };
 
 constexpr int kBM = 128;             // rows per workgroup
-constexpr int kMT = 8, kNT = 4;      // MFMA tiles per wave: 8 x 4
+constexpr int kMT = 8;  // 16-row MFMA tiles per wave (the column tiles per wave are a template parameter)
 
 // bf16 [M][K] -> fp16 [M][K] * 2^-e[row] (exact: power-of-two shift of an 8-bit significand into 11 bits), with
 // e[row] chosen so that the row maximum lands at 2^14; row_scale[row] = 2^e.  One workgroup per row; the row stays

@@ -92,6 +92,10 @@ template <>
 struct TypeTraits<bfloat16> {
   static constexpr DataType kDataType = TYPE_BF16;
 };
+template <>
+struct TypeTraits<float> {  // Fp8MatMulLayer<float> only (KS/layers/matmul_layer_factory.h:38)
+  static constexpr DataType kDataType = TYPE_FP32;
+};
 
 // Contiguous tensor over a raw pointer.  The side pointers are non-owning, as in the reference's weights map.
 class Tensor {

@@ -24,7 +24,7 @@ void ThrowOnKsqError(int code, const char* what) {
 
 template <typename T>
 int KsqDtype() {
-  return TypeTraits<T>::kDataType == TYPE_FP16 ? KSQ_F16 : KSQ_BF16;
+  return TypeTraits<T>::kDataType == TYPE_FP16 ? KSQ_F16 : (TypeTraits<T>::kDataType == TYPE_FP32 ? KSQ_F32 : KSQ_BF16);
 }
 
 constexpr size_t kFp8GemmWorkspaceBytes = 32ull << 20;  // the reference reserves 32 MiB for cuBLASLt here
@@ -432,6 +432,7 @@ Status MergeFp8QkvScales(Tensor& qkv_weight, const Tensor& q_scale, const Tensor
   return Status();
 }
 
+template class Fp8MatMulLayer<float>;  // fp32 activations and results (KS/layers/nvidia/fp8_matmul_layer.cpp:69)
 template class Fp8MatMulLayer<float16>;
 template class Fp8MatMulLayer<bfloat16>;
 

@@ -3,7 +3,7 @@
 //
 //   layer_driver w4a16 <dir> <f16|bf16> <m> <k> <n> <g> <gptq|awq> <gptq|awq|rowmajor> <none|awq|uint8|additive>
 //       reads <dir>/qweight.bin, qzeros.bin (unless none), scales.bin, act.bin; writes <dir>/out.bin
-//   layer_driver fp8 <dir> <f16|bf16> <m> <k> <n> <wscales: 1|n> <static: 0|1>
+//   layer_driver fp8 <dir> <f16|bf16|f32> <m> <k> <n> <wscales: 1|n> <static: 0|1>
 //   layer_driver fp8load <dir> <f16|bf16> <m> <k> <nq> <nkv> <per_channel: 0|1>
 //     q/k/v weights [k, n*] T from wq_src.bin / wk_src.bin / wv_src.bin: converted per tensor, fused, scales merged
 //       reads <dir>/wq.bin, wscale.bin, act.bin, iscale.bin (static); writes <dir>/out.bin
@@ -378,7 +378,9 @@ int main(int argc, char** argv) {
     if ((argc == 11 || argc == 12) && std::string(argv[1]) == "w4a16")
       return std::string(argv[3]) == "f16" ? RunW4<float16>(argc, argv) : RunW4<bfloat16>(argc, argv);
     if (argc == 9 && std::string(argv[1]) == "fp8")
-      return std::string(argv[3]) == "f16" ? RunFp8<float16>(argc, argv) : RunFp8<bfloat16>(argc, argv);
+      return std::string(argv[3]) == "f16"   ? RunFp8<float16>(argc, argv)
+             : std::string(argv[3]) == "f32" ? RunFp8<float>(argc, argv)
+                                             : RunFp8<bfloat16>(argc, argv);
     if (argc == 9 && std::string(argv[1]) == "fp8load")
       return std::string(argv[3]) == "f16" ? RunFp8Load<float16>(argc, argv) : RunFp8Load<bfloat16>(argc, argv);
     std::cerr << "usage: see the header of layer_driver.cpp" << std::endl;

@@ -14,6 +14,7 @@
 #include <memory>
 #include <sstream>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "base_layer.h"
@@ -64,9 +65,15 @@ class LayerHarness {
   // A layer of the class that goes with `weight_type`, from an explicit parameter pack.
   std::shared_ptr<BaseLayer> Make(DataType weight_type, DataType io_type, const std::vector<std::any>& pack) {
     std::shared_ptr<BaseLayer> layer;
-    const bool io_ok = io_type == TYPE_FP16 || io_type == TYPE_BF16;
-    if (io_ok && weight_type == TYPE_I4_GROUP) layer = std::make_shared<GroupMatMulLayer<T, TYPE_I4_GROUP>>();
-    if (io_ok && weight_type == TYPE_FP8_E4M3) layer = std::make_shared<Fp8MatMulLayer<T>>();
+    // fp16 and bf16 for both layers; fp32 for the FP8 layer only (the reference registers no fp32 group layer, and
+    // its float instantiation of that GEMM is empty)
+    if constexpr (std::is_same<T, float>::value) {
+      if (io_type == TYPE_FP32 && weight_type == TYPE_FP8_E4M3) layer = std::make_shared<Fp8MatMulLayer<T>>();
+    } else {
+      const bool io_ok = io_type == TYPE_FP16 || io_type == TYPE_BF16;
+      if (io_ok && weight_type == TYPE_I4_GROUP) layer = std::make_shared<GroupMatMulLayer<T, TYPE_I4_GROUP>>();
+      if (io_ok && weight_type == TYPE_FP8_E4M3) layer = std::make_shared<Fp8MatMulLayer<T>>();
+    }
     if (!layer) {
       std::ostringstream os;
       os << "no layer class for weight type " << weight_type << " with activations of type " << io_type;

@@ -4,19 +4,19 @@ import numpy as np
 
 from oracle import oracle as orc
 
-ORC_DT = {"f16": orc.F16, "bf16": orc.BF16}
+ORC_DT = {"f16": orc.F16, "bf16": orc.BF16, "f32": orc.F32}
 
 
 def torch_dtype(name):
     import torch
 
-    return {"f16": torch.float16, "bf16": torch.bfloat16}[name]
+    return {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[name]
 
 
 def capi_dtype(name):
     from ksanallm_amd import capi
 
-    return {"f16": capi.F16, "bf16": capi.BF16}[name]
+    return {"f16": capi.F16, "bf16": capi.BF16, "f32": capi.F32}[name]
 
 
 class W4Case:

@@ -65,7 +65,8 @@ def test_group_matmul_layer_takes_the_reference_loaders_tensors_at_forward(on_cp
     cases._adopt_case(_run, tmp_path, dtype, layout, kind, M)
 
 
-@pytest.mark.parametrize("dtype,wscales,static,M", [("f16", "1", 0, 16), ("bf16", "n", 0, 70), ("f16", "1", 1, 5)])
+@pytest.mark.parametrize("dtype,wscales,static,M", [("f16", "1", 0, 16), ("bf16", "n", 0, 70), ("f16", "1", 1, 5),
+                                                    ("f32", "n", 0, 9), ("f32", "1", 0, 70), ("f32", "1", 1, 5)])
 def test_fp8_matmul_layer_forward(on_cpu, tmp_path, dtype, wscales, static, M):
     cases.test_fp8_matmul_layer_forward(None, tmp_path, dtype, wscales, static, M)
 

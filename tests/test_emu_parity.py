@@ -76,6 +76,8 @@ test_gemm_large_m_ragged = f8.test_gemm_large_m_ragged
 test_gemm_large_m_both_tiles = f8.test_gemm_large_m_both_tiles
 test_gemm_k_phases_inside_the_workgroup = f8.test_gemm_k_phases_inside_the_workgroup
 test_gemm_random_shapes = f8.test_gemm_random_shapes
+test_gemm_fp32_results_every_route = f8.test_gemm_fp32_results_every_route
+test_gemm_dynamic_fp32 = f8.test_gemm_dynamic_fp32
 test_gemm_large_m_small_integers_exact = f8.test_gemm_large_m_small_integers_exact
 test_gemm_small_integers_exact = f8.test_gemm_small_integers_exact
 test_convert_weight_per_channel = f8.test_convert_weight_per_channel

@@ -6,6 +6,7 @@ import pytest
 
 from oracle import oracle as orc
 from tests.ksq_testlib import ORC_DT, bits_of, capi_dtype, torch_dtype
+from tests.test_w4a16_gpu import _env
 
 pytestmark = pytest.mark.gpu
 
@@ -21,6 +22,8 @@ def _announce(request):
 def _upload_bits(bits, dtype, gpu):
     import torch
 
+    if dtype == "f32":  # the oracle's "bits" of fp32 are the floats themselves
+        return torch.from_numpy(np.ascontiguousarray(bits, dtype=np.float32)).to(gpu)
     return torch.from_numpy(bits.view(np.int16)).to(gpu).view(torch_dtype(dtype))
 
 
@@ -41,7 +44,7 @@ def _quantize(gpu, xbits, dtype, mode, static_scale=None):
     return q.cpu().numpy(), scale.cpu().numpy()
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("shape", REF_SHAPES)
 def test_per_channel_quantize_reference_shapes(gpu, dtype, shape):
     from ksanallm_amd import capi
@@ -55,7 +58,7 @@ def test_per_channel_quantize_reference_shapes(gpu, dtype, shape):
     assert np.array_equal(q, orc.fp8_quantize(x, ORC_DT[dtype], want_s, C, L))
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("m,k", [(1, 4096), (16, 8192), (64, 1000), (300, 512)])
 def test_per_tensor_dynamic_and_static(gpu, dtype, m, k):
     from ksanallm_amd import capi
@@ -165,7 +168,7 @@ def _run_gemm(gpu, xq, x_scale, wq, w_scale, out_dtype, use_workspace=True):
     return out.float().cpu().numpy()
 
 
-@pytest.mark.parametrize("out_dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("out_dtype", ["bf16", "f16", "f32"])
 @pytest.mark.parametrize("M", [1, 3, 16, 17, 64, 65, 130])
 def test_gemm_rowwise_scales(gpu, out_dtype, M):
     xq, xs, wq, ws = _fp8_case(400 + M, M, 1024, 272)
@@ -289,6 +292,58 @@ def test_gemm_one_row_tile_both_workgroup_shapes(gpu, wide, M, K, N):
             os.environ["KSQ_FP8_WIDE"] = old
     orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"fp8 wide={wide} M={M} K={K} N={N}")
     assert np.array_equal(got, got2)
+
+
+@pytest.mark.parametrize("M,K,N,env", [
+    (5, 1024, 272, {}),                                   # decode kernel
+    (3, 4224, 528, {"KSQ_FP8_KPHASE": 1}),                # K in phases inside the workgroup
+    (40, 1008, 100, {}),                                  # K % 128 != 0: streaming kernel
+    (70, 1024, 264, {"KSQ_FP8_KSTAT": 0, "KSQ_FP8_PREFILL_MIN_M": 1000}),  # streaming kernel, several row tiles
+    (300, 1024, 264, {}),                                 # 256 x 256 tiles
+    (300, 4096, 2600, {"KSQ_FP8_TAIL_KSPLIT": 2}),        # ... with K split and the reduction kernel
+    (300, 4096, 9208, {"KSQ_FP8_TAIL_KSPLIT": 1}),        # ... with a last round of column quarters
+    (130, 1024, 520, {"KSQ_FP8_PREFILL_TILE": 128}),      # 128 x 256 tiles
+])
+def test_gemm_fp32_results_every_route(gpu, M, K, N, env):
+    """out_dtype = fp32 (what the reference's Fp8MatMulLayer<float> gets from its GEMM) through every kernel family:
+    the result is the fp32 accumulator times the scales, so it must agree with the oracle far inside the tolerance
+    of the 16-bit outputs; twice, bit for bit."""
+    xq, xs, wq, ws = _fp8_case(480 + M, M, K, N)
+    with _env(**env):
+        got = _run_gemm(gpu, xq, xs, wq, ws, "f32")
+        got2 = _run_gemm(gpu, xq, xs, wq, ws, "f32")
+    want = orc.fp8_gemm(xq, xs, wq, ws)
+    orc.assert_parity(got, want, f"fp8 fp32 out M={M} K={K} N={N} {env}")
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert float(np.max(np.abs(got - want))) <= 2e-5 * rms * np.sqrt(K), "fp32 results carry no 16-bit rounding"
+    assert np.array_equal(got, got2)
+
+
+@pytest.mark.parametrize("M", [1, 8, 70])
+def test_gemm_dynamic_fp32(gpu, M):
+    """fp32 activations in, fp32 results out: per-token quantisation (bit-identical to the oracle's, through the
+    element-wise kernels) and the GEMM as one call, with a bias row in fp32."""
+    import torch
+
+    from ksanallm_amd import capi
+
+    K, N = 1024, 272
+    rng = np.random.default_rng(490 + M)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    w_scale = orc.fp8_compute_scale(w, orc.F32, N, K)
+    wq = orc.fp8_quantize(w, orc.F32, w_scale, N, K)
+    x_scale = orc.fp8_compute_scale(x, orc.F32, M, K)
+    xq = orc.fp8_quantize(x, orc.F32, x_scale, M, K)
+    want = orc.fp8_gemm(xq, x_scale, wq, w_scale) + bias[None, :]
+    dx, dw, dws, db = (torch.from_numpy(a).to(gpu) for a in (x, wq, w_scale, bias))
+    out = torch.full((M, N), float("nan"), dtype=torch.float32, device=gpu)
+    wsb = capi.fp8_gemm_dynamic_workspace_bytes(M, N, K)
+    ws = torch.empty(max(wsb, 256), dtype=torch.uint8, device=gpu)
+    capi.fp8_gemm_dynamic(capi.F32, out, dx, dw, dws, N, M, N, K, capi.EPILOGUE_BIAS, db, ws, wsb)
+    torch.cuda.synchronize()
+    orc.assert_parity(out.cpu().numpy(), want, f"fp8 dynamic fp32 M={M}")
 
 
 @pytest.mark.parametrize("per_channel", [True, False])

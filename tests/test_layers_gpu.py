@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DRIVER = os.path.join(ROOT, "ksanallm_amd", "layer_driver")
-DTYPE_ENUM = {"f16": 11, "bf16": 10}  # TYPE_FP16 / TYPE_BF16 of the reference's DataType
+DTYPE_ENUM = {"f16": 11, "bf16": 10, "f32": 12}  # TYPE_FP16 / TYPE_BF16 / TYPE_FP32 of the reference's DataType
 
 
 def _run(args):
@@ -184,7 +184,7 @@ def test_group_matmul_layer_fused_from_separate_projections(gpu, tmp_path, dtype
     orc.assert_parity(got, case.oracle(), f"fused q/k/v {dtype}")
 
 
-@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("wscales,static,M", [("1", 0, 7), ("1", 1, 7), ("n", 0, 40)])
 def test_fp8_matmul_layer_forward(gpu, tmp_path, dtype, wscales, static, M):
     K, N = 512, 208
@@ -213,7 +213,8 @@ def test_fp8_matmul_layer_forward(gpu, tmp_path, dtype, wscales, static, M):
         xq = orc.fp8_quantize(x, ORC_DT[dtype], xs, 1, M * K).reshape(M, K)
     rc, out = _run(["fp8", d, dtype, M, K, N, wscales, static])
     assert rc == 0 and out.splitlines()[-1] == f"OK {M} {N} {DTYPE_ENUM[dtype]}", out
-    got = orc.from_bits(np.fromfile(d + "/out.bin", dtype=np.uint16).reshape(M, N), ORC_DT[dtype])
+    raw = np.fromfile(d + "/out.bin", dtype=np.float32 if dtype == "f32" else np.uint16).reshape(M, N)
+    got = orc.from_bits(raw, ORC_DT[dtype])
     orc.assert_parity(got, orc.fp8_gemm(xq, xs, wq, ws), f"Fp8MatMulLayer wscales={wscales} static={static} {dtype}")
 
 
