@@ -39,8 +39,8 @@ struct PrefillArgs {
   void* out;
   const float* row_scale;  // bf16 route: 2^e per row of the re-encoded activations
   int M, N, K, KT, G, ntiles, mblocks, nblocks;
-  int ksplit;          // 64-row kernel only: grid.y
-  float* partial;      // [ksplit][mblocks * 64][N] fp32, ksplit > 1 only
+  int ksplit;          // grid.y: K split over workgroups
+  float* partial;      // [ksplit][mblocks * rows per block][N] fp32, ksplit > 1 only
   Epilogue epi;
 };
 
@@ -303,12 +303,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
     }
   };
 
-  // The k loop of one k group over its pair of stages: k tiles kg, kg + KG, ...  Both groups make the same number of
-  // steps (a step is one barrier); with an odd number of k tiles the second group's last step has no tile.
+  // k tiles of this workgroup: all of them, or (K split over grid.y, for grids that would leave most compute units
+  // without a tile) the range of its split, whose raw fp32 tile goes to the workspace for the reduction kernel
+  int kt0, kt1;
+  split_range(p.KT, blockIdx.y, p.ksplit, &kt0, &kt1);
+  // The k loop of one k group over its pair of stages: k tiles kt0 + kg, kt0 + kg + KG, ...  Both groups make the same
+  // number of steps (a step is one barrier); with an odd number of k tiles the second group's last step has no tile.
   // (everything here has to be inlined: a call would put the accumulators, captured by reference, into memory)
   auto k_loop = [&](u32x4* s0, u32x4* s1) __attribute__((always_inline)) {
     auto run = [&](const u32x4* cur, u32x4* nxt, const BTile& bt, BTile& bn, int kt) __attribute__((always_inline)) {
-      if (KG == 1 || kt < p.KT) {
+      if (KG == 1 || kt < kt1) {
         step(cur, nxt, bt, bn, kt);
       } else {
         __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -316,14 +320,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       }
     };
 #pragma unroll
-    for (int q = 0; q < 4; ++q) load_part(s0, b0, kg, q);
-    const int nsteps = (p.KT + KG - 1) / KG;
+    for (int q = 0; q < 4; ++q) load_part(s0, b0, kt0 + kg, q);
+    const int nsteps = (kt1 - kt0 + KG - 1) / KG;
     int st = 0;
     for (; st + 2 <= nsteps; st += 2) {
-      run(s0, s1, b0, b1, kg + st * KG);
-      run(s1, s0, b1, b0, kg + (st + 1) * KG);
+      run(s0, s1, b0, b1, kt0 + kg + st * KG);
+      run(s1, s0, b1, b0, kt0 + kg + (st + 1) * KG);
     }
-    if (st < nsteps) run(s0, s1, b0, b1, kg + st * KG);
+    if (st < nsteps) run(s0, s1, b0, b1, kt0 + kg + st * KG);
   };
   if (KG == 1 || kg == 0) k_loop(lds_a0, lds_a1);
   else k_loop(lds_a2, lds_a3);
@@ -370,6 +374,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
       const int rr = (lane >> 3) + 8 * pass, cc = (lane & 7) * 8;
       const float* src = epi + rr * kEpiStride + cc;
       const int row = m0 + 16 * mt + rr, col = ncol0 + cc;
+      if (p.ksplit > 1) {  // the fp32 segment of this split; the reduction kernel finishes it
+        if (row < p.M && col + 8 <= p.N && cc < 16 * CT) {
+          f32x4* dst = reinterpret_cast<f32x4*>(p.partial + ((size_t)blockIdx.y * p.mblocks * kBM + row) * p.N + col);
+          dst[0] = f32x4{src[0], src[1], src[2], src[3]};
+          dst[1] = f32x4{src[4], src[5], src[6], src[7]};
+        }
+        continue;
+      }
       float rs = 1.f;
       if constexpr (kBF16) rs = p.row_scale[row < p.M ? row : p.M - 1];
       float vals[8];
@@ -772,6 +784,46 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     p.knt = knt;
     p.ksplit = (int)ks;
     p.partial_bytes = need(ks);
+    // The same K split with 128-row tiles (four waves side by side, two k groups, one workgroup per CU): the
+    // dequantisation of a weight tile then serves 128 rows instead of 64, which outweighs the rows that the taller
+    // tiles pad wherever both forms cover the device in one round.  Chosen by an estimate in microseconds fitted to
+    // sweeps over the Llama-2-7B/13B, Llama-3-8B/70B and Qwen-72B shapes at M = 96 .. 1024 (221 cases, every form
+    // three times; both fits within 5 to 8 % rms): per k tile of a workgroup 0.4 to 1.8 us for the 64-row form by
+    // tile width and by one or two workgroups per CU, 1.12 + 0.47 x (share of the CUs in use) for the 128-row one
+    // (0.94 + 0.34 x with three column tiles per wave), a fixed part, and the partial tiles at 6 TB/s.  The 128-row
+    // form is taken where it is estimated 5 % ahead.  Measured afterwards on those shapes and on three families the
+    // fit had not seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes), 392 cases: taken in 120, there 1 to 29 % faster
+    // than the better of the two forms without it (11 % on average), e.g. Llama-2-7B down M = 512 62 -> 58 us,
+    // M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212.
+    if (!tuning_env("KSQ_W4_PREFILL_ROWS") && !tuning_env("KSQ_W4_PREFILL_KSPLIT") && !tuning_env("KSQ_W4_PREFILL_NT") &&
+        wgs(knt) * ks <= 2 * (size_t)cus) {
+      const bool two = wgs(knt) * ks > (size_t)cus;
+      const double b64 = knt == 1 ? (two ? 0.751 : 0.412) : knt == 2 ? (two ? 1.171 : 0.80) : (two ? 1.813 : 1.024);
+      const double a64 = knt == 4 ? (two ? 8.6 : 6.0) : knt == 2 ? (two ? 3.1 : 4.0) : (two ? 3.0 : 4.8);
+      auto partial_us = [&](size_t c, size_t rows) { return 3.0 + 2.0 * (double)c * (double)rows * (double)n * 4.0 / 6e6; };
+      const double est64 = a64 + b64 * (double)((kt + ks - 1) / ks) + (ks > 1 ? partial_us(ks, mb * 64) : 0.0);
+      auto need128 = [&](size_t x) { return x * mb128 * 128 * n * 4; };
+      double best = 0.95 * est64;
+      for (int ct = 4; ct >= 3; --ct) {
+        const size_t w = mb128 * ((ntiles + (size_t)(4 * ct) - 1) / (size_t)(4 * ct));
+        // (workgroup ids go to the 8 XCDs in turn, y-slab after y-slab: what has to fit is every XCD's share)
+        for (size_t c = 2; c <= 8 && (w + 7) / 8 * c <= (size_t)cus / 8 && kt / c >= 8; ++c) {
+          if (need128(c) > workspace_bytes) break;
+          const double fill = (double)(w * c) / (double)cus;
+          const double per_tile = ct == 4 ? 1.122 + 0.473 * fill : 0.938 + 0.339 * fill;
+          const double est = (ct == 4 ? 6.4 : 6.1) + per_tile * (double)((kt + c - 1) / c) + partial_us(c, mb128 * 128);
+          if (est < best) {
+            best = est;
+            p.rows = 128;
+            p.nw = 4;
+            p.kg = 2;
+            p.ct = ct;
+            p.ksplit = (int)c;
+            p.partial_bytes = need128(c);
+          }
+        }
+      }
+    }
   } else {
     p.nw = cost128w8 < cost128w4 ? 8 : 4;
     p.ct = p.nw == 8 ? ct_w8 : ct_w4;
@@ -789,6 +841,16 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     // one workgroup per CU at most: two k groups of four waves each
     const size_t nbw = (ntiles + (size_t)(4 * p.ct) - 1) / (size_t)(4 * p.ct);
     p.kg = (p.nw == 4 && mb128 * nbw <= (size_t)cus && kt >= 4) ? 2 : 1;
+    // (a K split of this form is the planner's choice only from the 64-row side, above)
+    size_t ks = 1;
+    if (const char* e = tuning_env("KSQ_W4_PREFILL_KSPLIT")) {  // tuning / test override
+      const size_t v = (size_t)atoi(e);
+      if (v >= 1 && v <= 8 && v <= kt) ks = v;
+    }
+    auto need128 = [&](size_t x) { return x <= 1 ? (size_t)0 : x * mb128 * 128 * n * 4; };
+    while (ks > 1 && need128(ks) > workspace_bytes) --ks;
+    p.ksplit = (int)ks;
+    p.partial_bytes = need128(ks);
     if (const char* e = tuning_env("KSQ_W4_PREFILL_KG")) {  // tuning / test override
       const int v = atoi(e);
       if (v == 1 || (v == 2 && kt >= 2)) p.kg = v;
@@ -839,7 +901,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     const int bnt = nw * plan.ct;
     a.nblocks = (a.ntiles + bnt - 1) / bnt;
     KSQ_REQUIRE((size_t)a.mblocks * a.nblocks < (1ull << 30), KSQ_ERR_UNSUPPORTED, "grid too large");
-    grid = dim3(tile_grid(a.mblocks, a.nblocks));
+    grid = dim3(tile_grid(a.mblocks, a.nblocks), (unsigned)plan.ksplit);
     block = dim3(64 * nw * plan.kg);
   }
   const int gpt = (int)(kTileK / g);
@@ -847,7 +909,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
   if (plan.rows == 64)
     note_launch("w4a16_mid_kernel<gpt=%d,knt=%d> grid=(%u,%u)", gpt, plan.knt, grid.x, grid.y);
   else
-    note_launch("w4a16_prefill_kernel<gpt=%d,nw=%d,kg=%d,ct=%d> grid=(%u)", gpt, plan.nw, plan.kg, plan.ct, grid.x);
+    note_launch("w4a16_prefill_kernel<gpt=%d,nw=%d,kg=%d,ct=%d> grid=(%u,%u)", gpt, plan.nw, plan.kg, plan.ct, grid.x, grid.y);
   if (plan.ksplit > 1) note_launch("w4a16_splitk_reduce_kernel");
   if (dtype == KSQ_F16) {
     launch_typed<_Float16>(a, gpt, nw, plan.kg, plan.ct, grid, block, s);
@@ -867,7 +929,7 @@ int w4a16_launch_prefill(int dtype, void* out, const void* act, const void* weig
     launch_typed<__bf16>(a, gpt, nw, plan.kg, plan.ct, grid, block, s);
   }
   if (plan.ksplit > 1) {  // add the splits up and store
-    const size_t stride = (size_t)a.mblocks * 64 * n;
+    const size_t stride = (size_t)a.mblocks * (plan.rows == 64 ? 64 : kBM) * n;
     const dim3 rgrid((unsigned)((m * (n / 8) + 255) / 256));
     uint16_t* o = static_cast<uint16_t*>(out);
     if (dtype == KSQ_F16)

@@ -52,6 +52,7 @@ test_prefill_kernel_widths = w4.test_prefill_kernel_widths
 test_prefill_row_tiles = w4.test_prefill_row_tiles
 test_prefill_128_rows_k_groups = w4.test_prefill_128_rows_k_groups
 test_prefill_split_k = w4.test_prefill_split_k
+test_prefill_128_rows_split_k = w4.test_prefill_128_rows_split_k
 test_accumulator_stationary_route = w4.test_accumulator_stationary_route
 test_accumulator_stationary_split_k = w4.test_accumulator_stationary_split_k
 test_planner_choices_without_overrides = w4.test_planner_choices_without_overrides

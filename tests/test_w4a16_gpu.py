@@ -212,6 +212,40 @@ def test_prefill_128_rows_k_groups(gpu, kg, ct, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
+@pytest.mark.parametrize("ksplit,waves,kg,ct", [(2, 4, 2, 4), (3, 4, 2, 3), (8, 4, 1, 4), (2, 8, 1, 3), (5, 4, 2, 4)])
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "awq", 128, 130, 1152, 528),    # nine k tiles: splits of one to five tiles, odd ones for the two k groups
+    ("bf16", "awq", 128, 200, 2048, 272),
+    ("f16", "gptq", 64, 128, 4096, 512),
+    ("bf16", "gptq", 64, 300, 1024, 256),
+])
+def test_prefill_128_rows_split_k(gpu, ksplit, waves, kg, ct, dtype, kind, g, M, K, N):
+    """The 128-row kernel with K split over workgroups (each split's fp32 tile through the workspace, summed in split
+    order by the reduction kernel), in every form of the workgroup; twice, bit for bit, and with a workspace that holds
+    no partial tiles."""
+    from ksanallm_amd import capi
+
+    case = W4Case(1290 + ksplit + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    forms = dict(KSQ_W4_PREFILL_ROWS=128, KSQ_W4_PREFILL_WAVES=waves, KSQ_W4_PREFILL_KG=kg, KSQ_W4_PREFILL_CT=ct)
+    with _env(KSQ_W4_PREFILL_KSPLIT=ksplit, **forms):
+        dev = W4Device(case, gpu)   # sizes the workspace for the split
+        got1 = dev.gemm_f32()
+        capi.set_launch_log(True)
+        got2 = dev.gemm_f32()
+        log = capi.last_launch()
+        capi.set_launch_log(False)
+    assert f"kg={kg},ct={ct}> grid=(" in log and f",{ksplit})" in log and "w4a16_splitk_reduce_kernel" in log, log
+    with _env(KSQ_W4_PREFILL_KSPLIT=1, **forms):
+        front = capi.w4a16_workspace_bytes(M, N, K)
+    assert dev.workspace_bytes > front
+    dev.workspace_bytes = front
+    with _env(KSQ_W4_PREFILL_KSPLIT=ksplit, **forms):
+        got3 = dev.gemm_f32()
+    orc.assert_parity(got1, case.oracle(), f"prefill 128 rows ksplit={ksplit} kg={kg} ct={ct} {dtype} {kind} g={g} M={M}")
+    assert np.array_equal(got1, got2)
+    orc.assert_parity(got3, case.oracle(), f"prefill 128 rows one split {dtype} {kind} g={g} M={M}")
+
+
 @pytest.mark.parametrize("ksplit", [2, 3, 8])
 @pytest.mark.parametrize("nt", [1, 4])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
@@ -310,6 +344,28 @@ def test_planner_choices_without_overrides(gpu, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
     if not (dtype == "bf16" and M >= 65):  # the bf16 large-M route needs its workspace and falls back to a slower kernel
         orc.assert_parity(dev.gemm_f32(use_workspace=False), case.oracle(), f"planner, no workspace {dtype} M={M}")
+
+
+@pytest.mark.parametrize("dtype,kind,g,M,K,N", [
+    ("f16", "gptq", 128, 512, 11008, 4096),   # Llama-2-7B down: 64 workgroups of 128 x 256, K split in four
+    ("bf16", "awq", 128, 256, 8192, 8192),    # Llama-3-70B o
+    ("f16", "awq", 128, 200, 4096, 12288),    # Llama-2-7B qkv, ragged rows: 128 x 192 tiles, K split in two
+])
+def test_planner_splits_k_over_128_row_tiles(gpu, dtype, kind, g, M, K, N):
+    """Full-size shapes with few output tiles and a long K, where the planner, left alone, takes the 128-row kernel
+    with K split over workgroups; twice, bit for bit."""
+    from ksanallm_amd import capi
+
+    case = W4Case(1450 + M, M, K, N, g=g, kind=kind, dtype=dtype)
+    dev = W4Device(case, gpu)
+    got1 = dev.gemm_f32()
+    capi.set_launch_log(True)
+    got2 = dev.gemm_f32()
+    log = capi.last_launch()
+    capi.set_launch_log(False)
+    assert "w4a16_prefill_kernel" in log and "w4a16_splitk_reduce_kernel" in log, log
+    orc.assert_parity(got1, case.oracle(), f"planner, 128-row split {dtype} {kind} M={M} K={K} N={N}")
+    assert np.array_equal(got1, got2)
 
 
 def _random_w4_shapes(seed, count):
