@@ -792,9 +792,11 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     // tile width and by one or two workgroups per CU, 1.12 + 0.47 x (share of the CUs in use) for the 128-row one
     // (0.94 + 0.34 x with three column tiles per wave), a fixed part, and the partial tiles at 6 TB/s.  The 128-row
     // form is taken where it is estimated 5 % ahead.  Measured afterwards on those shapes and on three families the
-    // fit had not seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes), 392 cases: taken in 120, there 1 to 29 % faster
+    // fit had not seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes), 392 cases: taken in 120, there 0 to 29 % faster
     // than the better of the two forms without it (11 % on average), e.g. Llama-2-7B down M = 512 62 -> 58 us,
-    // M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212.
+    // M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212.  Only with three quarters of the
+    // CUs in use or more: every case of the fit where the form won has that, and on narrow shapes (N = 272 .. 2048
+    // at 65 .. 512 rows) the estimate, extrapolated below it, chose the form where it was 2 to 10 % slower.
     if (!tuning_env("KSQ_W4_PREFILL_ROWS") && !tuning_env("KSQ_W4_PREFILL_KSPLIT") && !tuning_env("KSQ_W4_PREFILL_NT") &&
         wgs(knt) * ks <= 2 * (size_t)cus) {
       const bool two = wgs(knt) * ks > (size_t)cus;
@@ -809,6 +811,7 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
         // (workgroup ids go to the 8 XCDs in turn, y-slab after y-slab: what has to fit is every XCD's share)
         for (size_t c = 2; c <= 8 && (w + 7) / 8 * c <= (size_t)cus / 8 && kt / c >= 8; ++c) {
           if (need128(c) > workspace_bytes) break;
+          if (4 * w * c < 3 * (size_t)cus) continue;  // the fit knows nothing below three quarters of the CUs in use
           const double fill = (double)(w * c) / (double)cus;
           const double per_tile = ct == 4 ? 1.122 + 0.473 * fill : 0.938 + 0.339 * fill;
           const double est = (ct == 4 ? 6.4 : 6.1) + per_tile * (double)((kt + c - 1) / c) + partial_us(c, mb128 * 128);

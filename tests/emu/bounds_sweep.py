@@ -33,6 +33,12 @@ def w4_cases(full):
         combos = list(itertools.product([64, 128], ["f16", "bf16"], [True, False]))
         for g, dt, ws in (combos if full else [combos[i % 8], combos[(i + 5) % 8]]):
             out.append((M, N, K, g, dt, ws))
+    # K long and output tiles few at 65 rows and more: the 64-row and the 128-row kernel with K split over workgroups
+    # (partial tiles of every split in the workspace, the reduction kernel behind them)
+    for i, (K, M, N) in enumerate(itertools.product([8192, 11008], [65, 128, 129, 256, 300, 513], [272, 4096, 4112, 8192])):
+        combos = list(itertools.product([64, 128], ["f16", "bf16"], [True, False]))
+        for g, dt, ws in (combos if full else [combos[i % 8], combos[(i + 5) % 8]]):
+            out.append((M, N, K, g, dt, ws))
     return out
 
 
