@@ -526,10 +526,12 @@ static int fp8_tail_split(size_t m, size_t n, size_t k, int cus, size_t workspac
   const size_t total = ((m + 255) / 256) * ((n + 255) / 256), per_round = (size_t)cus;
   if (total <= per_round) {
     // A single round.  With at most half the CUs holding a tile and K long, the whole grid is the "tail": K split
-    // so that the splits fill the device, 16 k stages each at least (Qwen-72B qkv at M = 256: 40 tiles, 86 us unsplit).
+    // so that the splits fill the device, 12 k stages each at least (Qwen-72B qkv at M = 256: 40 tiles, 86 us unsplit;
+    // a sweep of every split count at M = 96 .. 1024: with 16 stages at least, o at M = 96 .. 256 ran 5 to 8 % and a
+    // K = 11008, N = 4096 shape 8 to 11 % behind their best, with 10 qkv loses 3 %).
     size_t ks = per_round / total;
     if (ks > 8) ks = 8;
-    if (ks > k / 128 / 16) ks = k / 128 / 16;
+    if (ks > k / 128 / 12) ks = k / 128 / 12;
     if (const char* e = tuning_env("KSQ_FP8_TAIL_KSPLIT")) {  // tuning / test override (1 switches the split off)
       const int v = atoi(e);
       if (v >= 1 && v <= 8 && (size_t)v <= k / 128) ks = (size_t)v;
