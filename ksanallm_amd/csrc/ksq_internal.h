@@ -212,8 +212,8 @@ struct PrefillPlan {
   int knt;     // 64-row kernel: column tiles per wave (1, 2 or 4)
   int nw;      // 128-row kernel: waves side by side (4 or 8)
   int kg;      // 128-row kernel with four waves side by side: k groups of such waves (1 or 2)
-  int ct;      // 128-row kernel: column tiles per wave (4 or 3: 64 or 48 columns)
-  int ksplit;  // 64-row kernel: grid.y
+  int ct;      // 128-row kernel: column tiles per wave (1 to 4: 16 to 64 columns)
+  int ksplit;  // grid.y: K split over workgroups
   size_t partial_bytes;
 };
 PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t workspace_bytes);

@@ -144,11 +144,12 @@ __global__ __launch_bounds__(256) void bf16_rows_to_f16_long_kernel(const uint16
 }
 
 // CT = column tiles per wave: 4 (64 columns: tiles of 256 or 512 columns) or 3 (48 columns: 192 or 384), for
-// widths whose number of tiles falls better on the compute units (a partly filled last round costs a full one).
+// widths whose number of tiles falls better on the compute units (a partly filled last round costs a full one);
+// 2 or 1 (tiles of 128 or 64 columns) where a single row block has to be spread over the device (65 to 128 rows).
 template <typename T, int GPT, int NW, int KG = 1, int CT = 4>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w4a16_prefill_kernel(PrefillArgs p) {
   static_assert(NW == 4 || NW == 8, "four or eight waves side by side");
-  static_assert(CT == 3 || CT == 4, "three or four column tiles per wave");
+  static_assert(CT >= 1 && CT <= 4, "one to four column tiles per wave");
   // KG = 2: two groups of four waves on the same 128 x 256 tile, the first on the even k tiles, the second on the
   // odd ones, each with its own pair of activation stages; the second group's accumulators reach the first through
   // LDS at the end.  For grids that put one workgroup on a CU: two waves per SIMD instead of one.
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void w
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (lds_ptr)(buf + (kFPW * wave + i) * 64), 16, a_off[i],
                                                  (kt < p.KT ? kt : p.KT - 1) * 256, 0, 0);
       }
-    } else if (q >= CT) {  // three column tiles per wave: part 3 carries activations only
+    } else if (q >= CT) {  // fewer than four column tiles per wave: the other parts carry activations only
     } else if (item == 2) {
       b.w[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_w[q], w_voff + kt * 1024u, 0, 0));
     } else {
@@ -652,7 +653,9 @@ void launch_typed(const PrefillArgs& a, int gpt, int nw, int kg, int ct, dim3 gr
   }
 #define KSQ_PF(GPT, NW, KG)                                                                              \
   do {                                                                                                   \
-    if (ct == 3) hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 3>), grid, block, 0, s, a);    \
+    if (ct == 1) hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 1>), grid, block, 0, s, a);    \
+    else if (ct == 2) hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 2>), grid, block, 0, s, a); \
+    else if (ct == 3) hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 3>), grid, block, 0, s, a); \
     else hipLaunchKernelGGL((w4a16_prefill_kernel<T, GPT, NW, KG, 4>), grid, block, 0, s, a);            \
   } while (0)
   if (nw == 4 && kg == 2) {
@@ -784,37 +787,45 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     p.knt = knt;
     p.ksplit = (int)ks;
     p.partial_bytes = need(ks);
-    // The same K split with 128-row tiles (four waves side by side, two k groups, one workgroup per CU): the
-    // dequantisation of a weight tile then serves 128 rows instead of 64, which outweighs the rows that the taller
-    // tiles pad wherever both forms cover the device in one round.  Chosen by an estimate in microseconds fitted to
-    // sweeps over the Llama-2-7B/13B, Llama-3-8B/70B and Qwen-72B shapes at M = 96 .. 1024 (221 cases, every form
-    // three times; both fits within 5 to 8 % rms): per k tile of a workgroup 0.4 to 1.8 us for the 64-row form by
-    // tile width and by one or two workgroups per CU, 1.12 + 0.47 x (share of the CUs in use) for the 128-row one
-    // (0.94 + 0.34 x with three column tiles per wave), a fixed part, and the partial tiles at 6 TB/s.  The 128-row
-    // form is taken where it is estimated 5 % ahead.  Measured afterwards on those shapes and on three families the
-    // fit had not seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes), 392 cases: taken in 120, there 0 to 29 % faster
-    // than the better of the two forms without it (11 % on average), e.g. Llama-2-7B down M = 512 62 -> 58 us,
-    // M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212.  Only with three quarters of the
-    // CUs in use or more: every case of the fit where the form won has that, and on narrow shapes (N = 272 .. 2048
-    // at 65 .. 512 rows) the estimate, extrapolated below it, chose the form where it was 2 to 10 % slower.
+    // The 128-row kernel in its one-workgroup-per-CU form (four waves side by side, two k groups), with tiles of 64
+    // to 256 columns and K split over workgroups like the 64-row kernel's: the dequantisation of a weight tile then
+    // serves 128 rows instead of 64, which outweighs the rows that the taller tiles pad wherever both forms cover the
+    // device in one round, and at 65 .. 128 rows the narrow tiles (128 x 128, 128 x 64) give one row block the
+    // workgroups that two 64-row blocks get from their second block.  Chosen by an estimate in microseconds fitted
+    // to sweeps over the Llama-2-7B/13B, Llama-3-8B/70B and Qwen-72B shapes at M = 65 .. 1024 (every form three
+    // times; the fits within 7 to 9 % rms): per k tile of a workgroup 0.4 to 1.8 us for the 64-row form by tile width
+    // and by one or two workgroups per CU; for the 128-row form 0.57 + 0.13 x, 0.69 + 0.24 x, 0.98 + 0.27 x and
+    // 1.12 + 0.47 x us with one to four column tiles per wave (x = the share of the CUs in use: the per-tile time
+    // grows as the device fills), a fixed part, and the partial tiles at 6 TB/s.  The 128-row form is taken where it
+    // is estimated 5 % ahead, and only on grids that use three quarters of the CUs or more: every case of the fits
+    // where it won has that, and on narrow shapes (N = 272 .. 2048) the estimate, extrapolated below it, chose the
+    // form where it was 2 to 10 % slower.  Measured afterwards on those shapes and on three families the fit had not
+    // seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes): see the design notes; e.g. Llama-2-7B down M = 512
+    // 62 -> 58 us, M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212; at M = 65 .. 128
+    // Llama-2-7B qkv 27 -> 23.5 .. 27, 70B qkv 34 -> 30 .. 35, 13B gate_up 50 -> 43 .. 49.
+    // (not for a single 64-row block: half of a 128-row tile would be padding, and the fits start at 65 rows)
     if (!tuning_env("KSQ_W4_PREFILL_ROWS") && !tuning_env("KSQ_W4_PREFILL_KSPLIT") && !tuning_env("KSQ_W4_PREFILL_NT") &&
-        wgs(knt) * ks <= 2 * (size_t)cus) {
+        mb >= 2 && wgs(knt) * ks <= 2 * (size_t)cus) {
       const bool two = wgs(knt) * ks > (size_t)cus;
       const double b64 = knt == 1 ? (two ? 0.751 : 0.412) : knt == 2 ? (two ? 1.171 : 0.80) : (two ? 1.813 : 1.024);
       const double a64 = knt == 4 ? (two ? 8.6 : 6.0) : knt == 2 ? (two ? 3.1 : 4.0) : (two ? 3.0 : 4.8);
       auto partial_us = [&](size_t c, size_t rows) { return 3.0 + 2.0 * (double)c * (double)rows * (double)n * 4.0 / 6e6; };
       const double est64 = a64 + b64 * (double)((kt + ks - 1) / ks) + (ks > 1 ? partial_us(ks, mb * 64) : 0.0);
-      auto need128 = [&](size_t x) { return x * mb128 * 128 * n * 4; };
+      auto need128 = [&](size_t x) { return x <= 1 ? (size_t)0 : x * mb128 * 128 * n * 4; };
+      static const double kTile[5] = {0, 0.574, 0.693, 0.981, 1.122}, kFill[5] = {0, 0.125, 0.238, 0.266, 0.473},
+                          kFixed[5] = {0, 4.7, 5.5, 5.85, 6.35};
       double best = 0.95 * est64;
-      for (int ct = 4; ct >= 3; --ct) {
+      for (int ct = 4; ct >= 1; --ct) {
+        if (ct <= 2 && mb128 > 3) break;  // the narrow tiles were fitted at up to 384 rows (narrow shapes at 512 and
+                                          // 1000 rows: chosen there, they ran 4 to 14 % behind the 64-row form)
         const size_t w = mb128 * ((ntiles + (size_t)(4 * ct) - 1) / (size_t)(4 * ct));
         // (workgroup ids go to the 8 XCDs in turn, y-slab after y-slab: what has to fit is every XCD's share)
-        for (size_t c = 2; c <= 8 && (w + 7) / 8 * c <= (size_t)cus / 8 && kt / c >= 8; ++c) {
+        for (size_t c = 1; c <= 8 && (w + 7) / 8 * c <= (size_t)cus / 8 && kt / c >= 8; ++c) {
           if (need128(c) > workspace_bytes) break;
-          if (4 * w * c < 3 * (size_t)cus) continue;  // the fit knows nothing below three quarters of the CUs in use
+          if (4 * w * c < 3 * (size_t)cus) continue;  // the fits know nothing below three quarters of the CUs in use
           const double fill = (double)(w * c) / (double)cus;
-          const double per_tile = ct == 4 ? 1.122 + 0.473 * fill : 0.938 + 0.339 * fill;
-          const double est = (ct == 4 ? 6.4 : 6.1) + per_tile * (double)((kt + c - 1) / c) + partial_us(c, mb128 * 128);
+          const double est = kFixed[ct] + (kTile[ct] + kFill[ct] * fill) * (double)((kt + c - 1) / c) +
+                             (c > 1 ? partial_us(c, mb128 * 128) : 0.0);
           if (est < best) {
             best = est;
             p.rows = 128;
@@ -839,7 +850,7 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     }
     if (const char* e = tuning_env("KSQ_W4_PREFILL_CT")) {  // tuning / test override
       const int v = atoi(e);
-      if (v == 3 || v == 4) p.ct = v;
+      if (v >= 1 && v <= 4) p.ct = v;
     }
     // one workgroup per CU at most: two k groups of four waves each
     const size_t nbw = (ntiles + (size_t)(4 * p.ct) - 1) / (size_t)(4 * p.ct);

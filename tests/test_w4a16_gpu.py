@@ -137,7 +137,7 @@ def test_forced_split_k_and_tile_widths(gpu, dtype, M, ksplit, nt, slices):
     assert np.array_equal(got1, got2), "split-K result must be deterministic and repeatable"
 
 
-@pytest.mark.parametrize("waves,ct", [(4, 4), (8, 4), (4, 3), (8, 3)])
+@pytest.mark.parametrize("waves,ct", [(4, 4), (8, 4), (4, 3), (8, 3), (4, 2), (8, 2), (4, 1), (8, 1)])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "awq", 128, 128, 384, 528),    # odd number of k tiles, 33 column tiles: ragged in N for both widths
     ("bf16", "awq", 128, 333, 512, 1040),  # ragged rows, three column blocks of 512
@@ -349,11 +349,12 @@ def test_planner_choices_without_overrides(gpu, dtype, kind, g, M, K, N):
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "gptq", 128, 512, 11008, 4096),   # Llama-2-7B down: 64 workgroups of 128 x 256, K split in four
     ("bf16", "awq", 128, 256, 8192, 8192),    # Llama-3-70B o
-    ("f16", "awq", 128, 200, 4096, 12288),    # Llama-2-7B qkv, ragged rows: 128 x 192 tiles, K split in two
+    ("f16", "awq", 128, 200, 4096, 12288),    # Llama-2-7B qkv, ragged rows: 192 tiles of 128 x 128, no split
+    ("bf16", "gptq", 128, 96, 4096, 4096),    # Llama-2-7B o, one row block: 128 x 64 tiles, K split
 ])
 def test_planner_splits_k_over_128_row_tiles(gpu, dtype, kind, g, M, K, N):
-    """Full-size shapes with few output tiles and a long K, where the planner, left alone, takes the 128-row kernel
-    with K split over workgroups; twice, bit for bit."""
+    """Full-size shapes with few output tiles, where the planner, left alone, takes the 128-row kernel in its
+    one-workgroup-per-CU form, with K split over workgroups where K is long; twice, bit for bit."""
     from ksanallm_amd import capi
 
     case = W4Case(1450 + M, M, K, N, g=g, kind=kind, dtype=dtype)
@@ -363,7 +364,9 @@ def test_planner_splits_k_over_128_row_tiles(gpu, dtype, kind, g, M, K, N):
     got2 = dev.gemm_f32()
     log = capi.last_launch()
     capi.set_launch_log(False)
-    assert "w4a16_prefill_kernel" in log and "w4a16_splitk_reduce_kernel" in log, log
+    assert "w4a16_prefill_kernel" in log and "kg=2" in log, log
+    if K >= 8192:
+        assert "w4a16_splitk_reduce_kernel" in log, log
     orc.assert_parity(got1, case.oracle(), f"planner, 128-row split {dtype} {kind} M={M} K={K} N={N}")
     assert np.array_equal(got1, got2)
 
