@@ -800,8 +800,10 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     // is estimated 5 % ahead, and only on grids that use three quarters of the CUs or more: every case of the fits
     // where it won has that, and on narrow shapes (N = 272 .. 2048) the estimate, extrapolated below it, chose the
     // form where it was 2 to 10 % slower.  Measured afterwards on those shapes and on three families the fit had not
-    // seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes): see the design notes; e.g. Llama-2-7B down M = 512
-    // 62 -> 58 us, M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212; at M = 65 .. 128
+    // seen (Qwen2.5-32B, Yi-34B, half of the 70B shapes), 448 cases at M = 65 .. 1024, against the better of the
+    // 64-row kernel and the unsplit 128 x 192 .. 512 tiles: 5.4 % faster on average (8.4 % at M = 65 .. 128), the 266
+    // cases that take one of these forms 9.2 % (-33 .. +4.6 %); e.g. Llama-2-7B down M = 512 62 -> 58 us,
+    // M = 1024 107 -> 92; Llama-3-70B o M = 384 75 -> 66, down M = 512 276 -> 212; at M = 65 .. 128
     // Llama-2-7B qkv 27 -> 23.5 .. 27, 70B qkv 34 -> 30 .. 35, 13B gate_up 50 -> 43 .. 49.
     // (not for a single 64-row block: half of a 128-row tile would be padding, and the fits start at 65 rows)
     if (!tuning_env("KSQ_W4_PREFILL_ROWS") && !tuning_env("KSQ_W4_PREFILL_KSPLIT") && !tuning_env("KSQ_W4_PREFILL_NT") &&
