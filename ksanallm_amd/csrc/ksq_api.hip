@@ -337,11 +337,15 @@ int ksq_w4a16_workspace_bytes(size_t max_m, size_t n, size_t k, size_t* bytes) {
   }
   if (max_m >= 33) {  // the large-M kernels serve 33 rows and more where the shape suits them
     // the element type is not known here: size for the bf16 route of the prefill kernel, plus the largest set of
-    // split-K partial tiles any m up to max_m asks for (the plan depends on the number of 64-row blocks only)
+    // split-K partial tiles any m up to max_m asks for
     size_t partial = 0;
+    // (the forms are chosen by an estimate in which the partial tiles count by their rows, so the plan can differ
+    // between the first and the last row count of a block: both are asked)
     for (size_t mb = 1; mb <= (max_m + 63) / 64 && mb <= 2 * (size_t)cus; ++mb) {
-      const PrefillPlan pp = w4a16_prefill_plan(mb * 64, n, k, cus, (size_t)-1);
-      if (pp.partial_bytes > partial) partial = pp.partial_bytes;
+      for (size_t mm : {(mb - 1) * 64 + 1, mb * 64 < max_m ? mb * 64 : max_m}) {
+        const PrefillPlan pp = w4a16_prefill_plan(mm, n, k, cus, (size_t)-1);
+        if (pp.partial_bytes > partial) partial = pp.partial_bytes;
+      }
     }
     const size_t pf = w4a16_prefill_workspace_bytes(KSQ_BF16, max_m, k) + partial;
     if (pf > best) best = pf;

@@ -795,9 +795,9 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     // device in one round, and at 65 .. 128 rows the narrow tiles (128 x 128, 128 x 64) give one row block the
     // workgroups that two 64-row blocks get from their second block.  Chosen by an estimate in microseconds fitted
     // to sweeps over the Llama-2-7B/13B, Llama-3-8B/70B and Qwen-72B shapes at M = 65 .. 1024 (every form three
-    // times; the fits within 7 to 9 % rms): per k tile of a workgroup 0.4 to 1.8 us for the 64-row form by tile width
-    // and by one or two workgroups per CU; for the 128-row form 0.57 + 0.13 x, 0.69 + 0.24 x, 0.98 + 0.27 x and
-    // 1.12 + 0.47 x us with one to four column tiles per wave (x = the share of the CUs in use: the per-tile time
+    // times; the fits within 4 to 7 % rms): per k tile of a workgroup 0.4 to 1.8 us for the 64-row form by tile width
+    // and by one or two workgroups per CU; for the 128-row form 0.57 + 0.13 x, 0.68 + 0.25 x, 0.96 + 0.29 x and
+    // 1.11 + 0.50 x us with one to four column tiles per wave (x = the share of the CUs in use: the per-tile time
     // grows as the device fills), a fixed part, and the partial tiles at 6 TB/s.  The 128-row form is taken where it
     // is estimated 5 % ahead, and only on grids that use three quarters of the CUs or more: every case of the fits
     // where it won has that, and on narrow shapes (N = 272 .. 2048) the estimate, extrapolated below it, chose the
@@ -811,13 +811,14 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
     if (!tuning_env("KSQ_W4_PREFILL_ROWS") && !tuning_env("KSQ_W4_PREFILL_KSPLIT") && !tuning_env("KSQ_W4_PREFILL_NT") &&
         mb >= 2 && wgs(knt) * ks <= 2 * (size_t)cus) {
       const bool two = wgs(knt) * ks > (size_t)cus;
-      const double b64 = knt == 1 ? (two ? 0.751 : 0.412) : knt == 2 ? (two ? 1.171 : 0.80) : (two ? 1.813 : 1.024);
-      const double a64 = knt == 4 ? (two ? 8.6 : 6.0) : knt == 2 ? (two ? 3.1 : 4.0) : (two ? 3.0 : 4.8);
+      const double b64 = knt == 1 ? (two ? 0.751 : 0.412) : knt == 2 ? (two ? 1.171 : 0.80) : (two ? 1.811 : 1.004);
+      const double a64 = knt == 4 ? (two ? 9.0 : 6.9) : knt == 2 ? (two ? 3.1 : 4.0) : (two ? 3.0 : 4.8);
       auto partial_us = [&](size_t c, size_t rows) { return 3.0 + 2.0 * (double)c * (double)rows * (double)n * 4.0 / 6e6; };
-      const double est64 = a64 + b64 * (double)((kt + ks - 1) / ks) + (ks > 1 ? partial_us(ks, mb * 64) : 0.0);
+      // (both kernels store and the reduction reads the rows below m only: the traffic follows m, not the blocks)
+      const double est64 = a64 + b64 * (double)((kt + ks - 1) / ks) + (ks > 1 ? partial_us(ks, m) : 0.0);
       auto need128 = [&](size_t x) { return x <= 1 ? (size_t)0 : x * mb128 * 128 * n * 4; };
-      static const double kTile[5] = {0, 0.574, 0.693, 0.981, 1.122}, kFill[5] = {0, 0.125, 0.238, 0.266, 0.473},
-                          kFixed[5] = {0, 4.7, 5.5, 5.85, 6.35};
+      static const double kTile[5] = {0, 0.569, 0.682, 0.962, 1.106}, kFill[5] = {0, 0.129, 0.250, 0.292, 0.495},
+                          kFixed[5] = {0, 5.1, 6.3, 6.75, 7.35};
       double best = 0.95 * est64;
       for (int ct = 4; ct >= 1; --ct) {
         if (ct <= 2 && mb128 > 3) break;  // the narrow tiles were fitted at up to 384 rows (narrow shapes at 512 and
@@ -829,7 +830,7 @@ PrefillPlan w4a16_prefill_plan(size_t m, size_t n, size_t k, int cus, size_t wor
           if (4 * w * c < 3 * (size_t)cus) continue;  // the fits know nothing below three quarters of the CUs in use
           const double fill = (double)(w * c) / (double)cus;
           const double est = kFixed[ct] + (kTile[ct] + kFill[ct] * fill) * (double)((kt + c - 1) / c) +
-                             (c > 1 ? partial_us(c, mb128 * 128) : 0.0);
+                             (c > 1 ? partial_us(c, m) : 0.0);
           if (est < best) {
             best = est;
             p.rows = 128;
