@@ -212,7 +212,8 @@ def test_prefill_128_rows_k_groups(gpu, kg, ct, dtype, kind, g, M, K, N):
     assert np.array_equal(got1, got2)
 
 
-@pytest.mark.parametrize("ksplit,waves,kg,ct", [(2, 4, 2, 4), (3, 4, 2, 3), (8, 4, 1, 4), (2, 8, 1, 3), (5, 4, 2, 4)])
+@pytest.mark.parametrize("ksplit,waves,kg,ct", [(2, 4, 2, 4), (3, 4, 2, 3), (8, 4, 1, 4), (2, 8, 1, 3), (5, 4, 2, 4), (4, 4, 2, 2),
+                                                (3, 4, 2, 1), (2, 4, 1, 1)])
 @pytest.mark.parametrize("dtype,kind,g,M,K,N", [
     ("f16", "awq", 128, 130, 1152, 528),    # nine k tiles: splits of one to five tiles, odd ones for the two k groups
     ("bf16", "awq", 128, 200, 2048, 272),
